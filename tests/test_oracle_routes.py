@@ -1,0 +1,429 @@
+"""Pins the CPU oracle's dispatch / combine data movement: row order, counts, source-index map and reductions.
+
+Pins used: the reference checker's known answers (tests/checker/unit/test_checker_oracles.cpp:279-323,
+test_checker_executor.cpp:389-401), the reference checker compiled in place (oracle/_ref: ExpectedEpDispatchRoutes
+and the executor's output blobs), numpy stable sorts / bincount / cumsum as an independent model of the
+memory-route order (design: local expert -> source rank -> route order), brute force for the capacity rule and
+numpy sequential float16 / float32 sums for the two combine contracts.
+"""
+import numpy as np
+import pytest
+import torch
+
+from oracle import ep as O
+
+
+def rand_ids(rng, R, bs, K, E, invalid_frac=0.0):
+    ids = np.stack([np.stack([rng.permutation(E)[:K] for _ in range(bs)]) for _ in range(R)]).astype(np.int32)
+    if invalid_frac:
+        bad = rng.random(ids.shape) < invalid_frac
+        ids[bad] = rng.choice([-1, -7, E, E + 5], size=int(bad.sum()))
+    return ids
+
+
+def rand_x(rng, R, bs, h):
+    return rng.integers(0, 0x7bff, size=(R, bs, h), dtype=np.uint16)
+
+
+# ---------------------------------------------------------------------------------------------
+# MVP route vs the reference checker
+# ---------------------------------------------------------------------------------------------
+def test_mvp_checker_known_answers(known, orc):
+    k = known["checker_case"]
+    s = k["shape"]
+    case = O.Case(s["rank_size"], s["bs"], s["h"], s["top_k"], s["moe_expert_num"], dtype=s["dtype"])
+    # DefaultEpDispatchExpertIds (tools/checker/src/oracle.cpp:422-445), restated for the known answers
+    ids = np.zeros((s["bs"], s["top_k"]), np.int32)
+    le = case.local_experts
+    for t in range(s["bs"]):
+        for kk in range(s["top_k"]):
+            grp = t % s["rank_size"] if kk % 2 == 0 else s["rank_size"] - 1 - (t % s["rank_size"])
+            loc = ((0 if kk % 2 == 0 else le - 1) + kk // 2) % le
+            ids[t, kk] = (grp * le + loc) % s["moe_expert_num"]
+    assert ids.size == k["default_ids_len"] and ids.reshape(-1)[:2].tolist() == k["default_ids_first"]
+    iv = k["input_value"]
+    assert (0x1000 + iv["rank"] * 0x100 + iv["token"] * 0x10 + iv["h"]) & 0xffff == iv["value"]
+    x = np.zeros((s["rank_size"], s["bs"], s["h"]), np.uint16)
+    for r in range(s["rank_size"]):
+        for t in range(s["bs"]):
+            for hh in range(s["h"]):
+                x[r, t, hh] = (0x1000 + r * 0x100 + t * 0x10 + hh) & 0xffff
+    all_ids = np.broadcast_to(ids, (s["rank_size"],) + ids.shape).copy()
+    out = orc.mvp_dispatch(case, 1, x, all_ids)
+    assert out["rows"] == k["rank1_route_count"]
+    assert out["assist"][0].tolist() == k["rank1_first_route"]
+    assert out["recv_counts"][0] == k["rank1_recv_count_src0"]
+    assert out["expert_token_nums"][0] == k["rank1_local_expert0_count"]
+    # payload rows are byte copies of the source rows
+    for row in range(out["rows"]):
+        src, tok = out["assist"][row][:2]
+        assert np.array_equal(out["expand_x"][row].view(np.uint16), x[src, tok])
+
+
+@pytest.mark.parametrize("shape", [(2, 3, 4, 2, 4), (4, 16, 8, 2, 16), (4, 9, 8, 3, 8), (8, 5, 8, 4, 32), (1, 7, 8, 2, 5)])
+def test_mvp_routes_match_compiled_checker(ref, orc, shape):
+    R, bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape))
+    ids = rand_ids(rng, 1, bs, K, E, invalid_frac=0.15)[0]
+    x = rand_x(rng, R, bs, h)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16)
+    all_ids = np.broadcast_to(ids, (R,) + ids.shape).copy()
+    for dst in range(R):
+        want = ref.checker_routes(R, bs, K, E, ids, dst)
+        got = orc.mvp_dispatch(case, dst, x, all_ids)
+        assert got["rows"] == len(want)
+        assert np.array_equal(got["assist"][: len(want)], want)
+        assert np.array_equal(got["recv_counts"], np.bincount(want[:, 0], minlength=R))
+        le = case.local_experts
+        assert np.array_equal(got["expert_token_nums"], np.bincount(want[:, 3] % le, minlength=le))
+
+
+@pytest.mark.parametrize("shape,dtype", [((2, 3, 4, 2, 4), 3), ((4, 8, 16, 2, 8), 11), ((4, 128, 1024, 2, 16), 11)])
+def test_mvp_dispatch_and_restore_match_checker_blobs(ref, orc, shape, dtype):
+    """The checker's executor output blob: [R*bs*K*h payload | bs*K assist | R int32 | localE int64]
+    (tools/checker/src/oracle.cpp:661-708); ep_combine restores rows to [bs, K, h] (executor.cpp:471-541)."""
+    R, bs, h, K, E = shape
+    st, blobs, events = ref.checker_run(0, R, bs, h, K, E, dtype)
+    assert st == 0
+    ids = ref.checker_default_ids(R, bs, K, E)
+    x = np.zeros((R, bs, h), np.uint16)
+    tt, hh = np.meshgrid(np.arange(bs), np.arange(h), indexing="ij")
+    for r in range(R):
+        x[r] = (0x1000 + r * 0x100 + tt * 0x10 + hh) & 0xffff
+    case = O.Case(R, bs, h, K, E, dtype=dtype)
+    all_ids = np.broadcast_to(ids, (R,) + ids.shape).copy()
+    payload_bytes = R * bs * K * h * 2
+    assist_bytes = bs * K * 16
+    le = case.local_experts
+    for dst in range(R):
+        got = orc.mvp_dispatch(case, dst, x, all_ids)
+        n = got["rows"]
+        assert n == bs * K          # the checker's default ids are balanced (oracle.cpp:432-441)
+        blob = blobs[dst]
+        assert np.array_equal(blob[: n * h * 2], got["expand_x"][:n].reshape(-1))
+        assert np.array_equal(blob[payload_bytes: payload_bytes + assist_bytes].view(np.int32).reshape(-1, 4),
+                              got["assist"][:n])
+        off = payload_bytes + assist_bytes
+        assert np.array_equal(blob[off: off + 4 * R].view(np.int32), got["recv_counts"])
+        assert np.array_equal(blob[off + 4 * R: off + 4 * R + 8 * le].view(np.int64), got["expert_token_nums"])
+    if shape == (4, 128, 1024, 2, 16):
+        assert events == 4148       # event count the reference CLI reports for this configuration
+    # inverse route: every source rank gets its rows back at [token, k]
+    st, cblobs, cevents = ref.checker_run(1, R, bs, h, K, E, dtype)
+    assert st == 0
+    for r in range(R):
+        restored = cblobs[r].view(np.uint16).reshape(bs, K, h)
+        assert np.array_equal(restored, np.broadcast_to(x[r][:, None, :], (bs, K, h)))
+    if shape == (4, 128, 1024, 2, 16):
+        assert cevents == 6164
+
+
+def test_mvp_token_mask_and_prefix_type(orc):
+    rng = np.random.default_rng(4)
+    R, bs, h, K, E = 2, 10, 8, 3, 8
+    ids = rand_ids(rng, R, bs, K, E, 0.1)
+    x = rand_x(rng, R, bs, h)
+    mask = (rng.random((R, bs)) < 0.6).astype(np.uint8)
+    base = orc.mvp_dispatch(O.Case(R, bs, h, K, E, token_nums_type=1), 0, x, ids, mask)
+    pref = orc.mvp_dispatch(O.Case(R, bs, h, K, E, token_nums_type=0), 0, x, ids, mask)
+    assert np.array_equal(np.cumsum(base["expert_token_nums"]), pref["expert_token_nums"])
+    # every emitted route comes from an active token and nothing else is emitted
+    a = base["assist"][: base["rows"]]
+    assert all(mask[s, t] for s, t in a[:, :2])
+    expected = sum(int(mask[s, t]) and 0 <= ids[s, t, k] < E and ids[s, t, k] // (E // R) == 0
+                   for s in range(R) for t in range(bs) for k in range(K))
+    assert base["rows"] == expected
+
+
+# ---------------------------------------------------------------------------------------------
+# memory route
+# ---------------------------------------------------------------------------------------------
+def np_memory_order(case, dst, ids, live):
+    """Independent model: stable sort of live routes by (local expert, source rank), keeping flat order."""
+    R, bs, K = ids.shape
+    le = case.local_experts
+    src, tok, k = np.meshgrid(np.arange(R), np.arange(bs), np.arange(K), indexing="ij")
+    flat = np.stack([src.ravel(), tok.ravel(), k.ravel(), ids.ravel()], axis=1)
+    ok = live.ravel() & (flat[:, 3] >= 0) & (flat[:, 3] < case.moe_expert_num)
+    ok &= np.where(ok, flat[:, 3] // le == dst, False)
+    sel = flat[ok]
+    key = (sel[:, 3] % le) * R + sel[:, 0]
+    order = np.argsort(key, kind="stable")
+    return sel[order], np.cumsum(np.bincount(key, minlength=le * R))
+
+
+@pytest.mark.parametrize("shape", [(1, 16, 8, 2, 4), (1, 64, 16, 8, 32), (2, 12, 8, 2, 8), (4, 20, 8, 3, 16)])
+@pytest.mark.parametrize("mask_type", [O.MASK_NONE, O.MASK_TOKEN, O.MASK_EXPERT])
+def test_memory_order_and_counts(orc, shape, mask_type):
+    R, bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + mask_type)
+    ids = rand_ids(rng, R, bs, K, E, 0.1)
+    x = rand_x(rng, R, bs, h)
+    mask = None
+    live = np.ones((R, bs, K), bool)
+    if mask_type == O.MASK_TOKEN:
+        mask = (rng.random((R, bs)) < 0.7).astype(np.uint8)
+        # prefix semantics (tilexr_ep_dispatch_memory_kernel.h:1387-1410,1538-1544): the first sum(mask) tokens
+        for r in range(R):
+            live[r] = (np.arange(bs) < mask[r].sum())[:, None]
+    elif mask_type == O.MASK_EXPERT:
+        mask = (rng.random((R, bs, K)) < 0.7).astype(np.uint8)
+        live = mask.astype(bool)
+    for nums_type in (0, 1):
+        case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16, mask_type=mask_type, token_nums_type=nums_type)
+        for dst in range(R):
+            got = orc.mem_dispatch(case, dst, x, ids, mask)
+            want, send = np_memory_order(case, dst, ids, live)
+            assert got["rows"] == len(want)
+            assert np.array_equal(got["assist"][: len(want)], want)
+            assert np.array_equal(got["send_counts"], send)
+            per_expert = send[R - 1:: R]
+            want_nums = per_expert if nums_type == 0 else np.diff(np.concatenate([[0], per_expert]))
+            assert np.array_equal(got["expert_token_nums"], want_nums)
+            for row in range(got["rows"]):
+                s, t = got["assist"][row][:2]
+                assert np.array_equal(got["expand_x"][row].view(np.uint16), x[s, t])
+
+
+def test_memory_route_is_a_permutation_of_the_mvp_route(orc):
+    rng = np.random.default_rng(8)
+    R, bs, h, K, E = 4, 24, 8, 3, 16
+    ids = rand_ids(rng, R, bs, K, E, 0.05)
+    x = rand_x(rng, R, bs, h)
+    case = O.Case(R, bs, h, K, E)
+    for dst in range(R):
+        a = orc.mvp_dispatch(case, dst, x, ids)
+        b = orc.mem_dispatch(case, dst, x, ids)
+        assert a["rows"] == b["rows"]
+        sa = {tuple(t) for t in a["assist"][: a["rows"]]}
+        sb = {tuple(t) for t in b["assist"][: b["rows"]]}
+        assert sa == sb and len(sa) == a["rows"]
+        # expert counts agree between the two routes
+        assert np.array_equal(a["expert_token_nums"], b["expert_token_nums"])
+
+
+def test_capacity_drops_highest_route_indices(orc):
+    """ext rule: per (source rank, expert) keep the `capacity` lowest flat route indices."""
+    rng = np.random.default_rng(13)
+    R, bs, h, K, E, cap = 2, 40, 8, 4, 8, 5
+    ids = rand_ids(rng, R, bs, K, E)
+    x = rand_x(rng, R, bs, h)
+    case = O.Case(R, bs, h, K, E, capacity=cap)
+    le = case.local_experts
+    for dst in range(R):
+        got = orc.mem_dispatch(case, dst, x, ids)
+        want = []
+        for e in range(dst * le, (dst + 1) * le):
+            for s in range(R):
+                flat = [i for i in range(bs * K) if ids[s].reshape(-1)[i] == e][:cap]
+                want += [(s, i // K, i % K, e) for i in flat]
+        assert got["rows"] == len(want)
+        assert [tuple(t) for t in got["assist"][: got["rows"]]] == want
+    # a capacity at least as large as the biggest bucket changes nothing
+    big = orc.mem_dispatch(O.Case(R, bs, h, K, E, capacity=bs * K), 0, x, ids)
+    none = orc.mem_dispatch(O.Case(R, bs, h, K, E), 0, x, ids)
+    assert big["rows"] == none["rows"] and np.array_equal(big["assist"], none["assist"])
+
+
+def test_memory_dispatch_quantised_payloads(orc):
+    rng = np.random.default_rng(17)
+    R, bs, h, K, E = 1, 12, 160, 2, 4
+    ids = rand_ids(rng, R, bs, K, E)
+    xf = torch.from_numpy((rng.standard_normal((R, bs, h)) * 2).astype(np.float32)).to(torch.bfloat16)
+    x = xf.view(torch.int16).numpy().view(np.uint16)
+    plain = orc.mem_dispatch(O.Case(R, bs, h, K, E), 0, x, ids)
+    for mode in (O.Q_TOKEN_INT8, O.Q_MXFP8, O.Q_FP8_BLOCK128):
+        case = O.Case(R, bs, h, K, E, quant_mode=mode)
+        got = orc.mem_dispatch(case, 0, x, ids)
+        assert got["rows"] == plain["rows"] and np.array_equal(got["assist"], plain["assist"])
+        for row in range(got["rows"]):
+            tok = got["assist"][row][1]
+            if mode == O.Q_TOKEN_INT8:
+                q, s = orc.quant_row_token_int8(x[0, tok], O.DT_BF16)
+                assert np.array_equal(got["expand_x"][row].view(np.int8), q) and got["dyn_scales"][row, 0] == s
+            elif mode == O.Q_MXFP8:
+                q, s = orc.quant_row_mxfp8(x[0, tok], O.DT_BF16, O.DT_FP8E4M3)
+                assert np.array_equal(got["expand_x"][row], q) and np.array_equal(got["dyn_scales"][row], s)
+            else:
+                q, s = orc.quant_row_fp8_block128(x[0, tok], O.DT_BF16)
+                assert np.array_equal(got["expand_x"][row], q) and np.array_equal(got["dyn_scales"][row], s)
+
+
+# ---------------------------------------------------------------------------------------------
+# combine
+# ---------------------------------------------------------------------------------------------
+def _dispatch_all(orc, case, x, ids, memory):
+    R = case.rank_size
+    outs = [(orc.mem_dispatch if memory else orc.mvp_dispatch)(case, d, x, ids) for d in range(R)]
+    expert_out = np.stack([o["expand_x"].view(np.uint16) for o in outs])
+    assist = np.stack([o["assist"] for o in outs])
+    counts = np.stack([o["send_counts" if memory else "recv_counts"] for o in outs])
+    return expert_out, assist, counts
+
+
+def test_mvp_combine_is_a_sequential_float16_sum(orc):
+    rng = np.random.default_rng(23)
+    R, bs, h, K, E = 2, 6, 32, 4, 8
+    ids = rand_ids(rng, R, bs, K, E, 0.1)
+    xf = (rng.standard_normal((R, bs, h)) * 30).astype(np.float16)
+    x = xf.view(np.uint16)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16)
+    expert_out, assist, counts = _dispatch_all(orc, case, x, ids, memory=False)
+    # make the rows differ per route so the order of additions matters
+    scale = (1 + 0.37 * np.arange(expert_out.shape[1]) % 5).astype(np.float16)
+    eo = (expert_out.view(np.float16) * scale[None, :, None]).astype(np.float16)
+    for rank in range(R):
+        y = orc.mvp_combine(case, rank, eo.view(np.uint16), assist, counts)
+        want = np.zeros((bs, h), np.float16)
+        for er in range(R):                     # expert-rank major, then row order
+            start = int(counts[er][:rank].sum())
+            for row in range(start, start + int(counts[er][rank])):
+                tok = assist[er, row, 1]
+                want[tok] = (want[tok].astype(np.float32) + eo[er, row].astype(np.float32)).astype(np.float16)
+        assert np.array_equal(y, want.view(np.uint16))
+    # per-add rounding is observable: a single fp32 accumulation gives a different answer somewhere
+    acc = np.zeros((bs, h), np.float32)
+    for er in range(R):
+        for row in range(int(counts[er][0])):
+            acc[assist[er, row, 1]] += eo[er, row].astype(np.float32)
+    y0 = orc.mvp_combine(case, 0, eo.view(np.uint16), assist, counts)
+    assert not np.array_equal(y0, acc.astype(np.float16).view(np.uint16))
+
+
+@pytest.mark.parametrize("dtype", [O.DT_BF16, O.DT_FP16])
+def test_memory_combine_is_fp32_k_ordered(orc, dtype):
+    rng = np.random.default_rng(29)
+    R, bs, h, K, E = 2, 9, 64, 4, 8
+    ids = rand_ids(rng, R, bs, K, E)
+    f = (rng.standard_normal((R, bs, h)) * 3).astype(np.float32)
+    if dtype == O.DT_BF16:
+        x = torch.from_numpy(f).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    else:
+        x = f.astype(np.float16).view(np.uint16)
+    case = O.Case(R, bs, h, K, E, dtype=dtype)
+    expert_out, assist, counts = _dispatch_all(orc, case, x, ids, memory=True)
+    # perturb rows per route so each k contributes a different vector
+    rows = expert_out.shape[1]
+    for er in range(R):
+        for row in range(rows):
+            expert_out[er, row] = np.roll(expert_out[er, row], row % 7)
+    w = (0.5 + rng.random((R, bs, K))).astype(np.float32)
+    shared = rand_x(rng, R, bs, h) if dtype == O.DT_FP16 else None
+    tmask = (rng.random((R, bs)) < 0.8).astype(np.uint8)
+
+    def dec(u):
+        if dtype == O.DT_BF16:
+            return (u.astype(np.uint32) << 16).view(np.float32)
+        return u.view(np.float16).astype(np.float32)
+
+    for rank in range(R):
+        sh = None if shared is None else (shared[rank] & 0x3fff)
+        y = orc.mem_combine(case, rank, expert_out, assist, counts, expert_scales=w[rank], token_mask=tmask[rank],
+                            shared_expert_x=sh)
+        slot = -np.ones((bs, K, 2), np.int64)
+        for er in range(R):
+            for row in range(int(counts[er][-1])):
+                s, t, k, _ = assist[er, row]
+                if s == rank:
+                    slot[t, k] = (er, row)
+        want = np.zeros((bs, h), np.float32)
+        for t in range(bs):
+            if not tmask[rank, t]:
+                continue
+            acc = np.zeros(h, np.float32)
+            for k in range(K):
+                er, row = slot[t, k]
+                if er < 0:
+                    continue
+                acc = (acc + (dec(expert_out[er, row]) * w[rank, t, k]).astype(np.float32)).astype(np.float32)
+            if sh is not None:
+                acc = (acc + dec(sh[t])).astype(np.float32)
+            want[t] = acc
+        if dtype == O.DT_BF16:
+            wb = torch.from_numpy(want).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+        else:
+            wb = np.clip(want, -65504, 65504).astype(np.float16).view(np.uint16)
+        assert np.array_equal(y, wb)
+        assert not y[tmask[rank] == 0].any()
+
+
+def test_memory_combine_k_order_is_observable(orc):
+    """Summing the same rows in reverse k order changes some bf16 results: the order is part of the contract."""
+    rng = np.random.default_rng(31)
+    bs, h, K, E = 64, 128, 8, 16
+    ids = rand_ids(rng, 1, bs, K, E)
+    f = (rng.standard_normal((1, bs, h)) * 100).astype(np.float32)
+    x = torch.from_numpy(f).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+    case = O.Case(1, bs, h, K, E)
+    d = orc.mem_dispatch(case, 0, x, ids)
+    eo = d["expand_x"].view(np.uint16)[None]
+    for row in range(d["rows"]):
+        eo[0, row] = np.roll(eo[0, row], row % 11)
+    w = (rng.random((bs, K)) * 4).astype(np.float32)
+    a = orc.mem_combine(case, 0, eo, d["assist"][None], d["send_counts"][None], expert_scales=w)
+    rev_assist = d["assist"].copy()
+    rev_assist[:, 2] = K - 1 - rev_assist[:, 2]
+    b = orc.mem_combine(case, 0, eo, rev_assist[None], d["send_counts"][None], expert_scales=w[:, ::-1].copy())
+    assert not np.array_equal(a, b)
+    assert np.mean(a != b) < 0.2     # ...but only by final-rounding effects
+
+
+def test_memory_combine_mxfp8_comm_quant(orc):
+    """comm quant 3/4: each row goes through the MXFP8 round trip, then (fp8*2^(s-127))*w is accumulated
+    (tilexr_ep_mxfp8_quant.h:286-352).  Checked against the quantiser + numpy."""
+    rng = np.random.default_rng(37)
+    bs, h, K, E = 5, 96, 2, 4
+    ids = rand_ids(rng, 1, bs, K, E)
+    f = (rng.standard_normal((1, bs, h)) * 4).astype(np.float16)
+    x = f.view(np.uint16)
+    w = (0.5 + rng.random((bs, K))).astype(np.float32)
+    case = O.Case(1, bs, h, K, E, dtype=O.DT_FP16)
+    d = orc.mem_dispatch(case, 0, x, ids)
+    eo = d["expand_x"].view(np.uint16)[None]
+    for mode, fp8 in ((3, O.DT_FP8E5M2), (4, O.DT_FP8E4M3)):
+        y = orc.mem_combine(case, 0, eo, d["assist"][None], d["send_counts"][None], expert_scales=w, comm_quant=mode)
+        want = np.zeros((bs, h), np.float32)
+        inv = {(int(t), int(k)): r for r, (_, t, k, _) in enumerate(d["assist"][: d["rows"]])}
+        for t in range(bs):
+            acc = np.zeros(h, np.float32)
+            for k in range(K):
+                row = inv[(t, k)]
+                q, s = orc.quant_row_mxfp8(eo[0, row], O.DT_FP16, fp8)
+                dq = np.array([orc.fp8_decode(int(b), fp8) for b in q], np.float32) * \
+                    np.exp2(s[np.arange(h) // 32].astype(np.float32) - 127).astype(np.float32)
+                acc = (acc + (dq * w[t, k]).astype(np.float32)).astype(np.float32)
+            want[t] = acc
+        assert np.array_equal(y, np.clip(want, -65504, 65504).astype(np.float16).view(np.uint16))
+        # and it stays within the demo's tolerance of the unquantised combine (tilexr_ep_dispatch_demo.cpp:1039-1040)
+        exact = orc.mem_combine(case, 0, eo, d["assist"][None], d["send_counts"][None], expert_scales=w)
+        ya, yb = y.view(np.float16).astype(np.float32), exact.view(np.float16).astype(np.float32)
+        tol = np.maximum(1e-3, np.abs(yb) * (0.30 if mode == 3 else 0.15))
+        assert np.all(np.abs(ya - yb) <= tol)
+
+
+def test_memory_combine_quantised_input_equals_combine_of_dequantised_rows(orc):
+    """ext: combine(q, scales) == combine(round_to_dtype(dequant(q, scales)))."""
+    rng = np.random.default_rng(41)
+    bs, h, K, E = 10, 256, 3, 8
+    ids = rand_ids(rng, 1, bs, K, E)
+    xf = torch.from_numpy((rng.standard_normal((1, bs, h)) * 2).astype(np.float32)).to(torch.bfloat16)
+    x = xf.view(torch.int16).numpy().view(np.uint16)
+    w = (rng.random((bs, K)) + 0.1).astype(np.float32)
+    for mode in (O.Q_TOKEN_INT8, O.Q_FP8_BLOCK128):
+        case = O.Case(1, bs, h, K, E, quant_mode=mode)
+        d = orc.mem_dispatch(case, 0, x, ids)
+        rows = d["rows"]
+        if mode == O.Q_TOKEN_INT8:
+            deq = d["expand_x"].view(np.int8).astype(np.float32) * d["dyn_scales"][:, :1]
+        else:
+            dec = np.array([orc.fp8_decode(c) for c in range(256)], np.float32)
+            deq = dec[d["expand_x"]] * np.repeat(d["dyn_scales"], 128, axis=1)[:, :h]
+        deq_bits = torch.from_numpy(np.ascontiguousarray(deq, np.float32)).to(torch.bfloat16).view(torch.int16) \
+            .numpy().view(np.uint16)
+        plain_case = O.Case(1, bs, h, K, E)
+        want = orc.mem_combine(plain_case, 0, deq_bits[None], d["assist"][None], d["send_counts"][None],
+                               expert_scales=w)
+        got = orc.mem_combine(plain_case, 0, d["expand_x"][None], d["assist"][None], d["send_counts"][None],
+                              expert_scales=w, in_quant=mode, in_scales=d["dyn_scales"])
+        assert np.array_equal(got, want)
+        assert rows > 0
