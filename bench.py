@@ -1,0 +1,187 @@
+"""Benchmark of the EP dispatch + combine hot path on one MI355X.
+
+A "step" is one MoE layer's dispatch followed by its combine (identity expert in between) on synthetic inputs that
+are already resident in HBM.  The default workload is the prefill shape the headline metric is quoted on:
+4096 tokens x 7168 bf16, 256 experts, top-8, Zipf(1.0) expert popularity ("C3").
+
+Prints one JSON line: whole-step effective bandwidth (algorithmic bytes / time), per-layer latency, a roofline object
+for the dominant kernel (timed with HIP events around that kernel on the stream it runs on) and the CPU oracle
+timed on this box's host cores as a baseline.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def parse():
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=100)
+    p.add_argument("--warmup", type=int, default=20)
+    p.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
+    p.add_argument("--no-cpu-baseline", action="store_true")
+    p.add_argument("--no-kernel-events", action="store_true",
+                   help="do not record per-kernel HIP events inside the timed region")
+    return p.parse_args()
+
+
+def cpu_baseline(w, x, ids, weights, kept_rows):
+    """The CPU oracle (a scalar C port of the reference path) on one host core, full layer, best of 3."""
+    import numpy as np
+
+    from oracle import ep as O
+    from tilexr_amd import workloads
+
+    xb = x.view(__import__("torch").int16).numpy().view(np.uint16)
+    quant = {"none": O.Q_NONE, "int8": O.Q_TOKEN_INT8, "fp8_block128": O.Q_FP8_BLOCK128}[w.quant]
+    case = O.Case(1, w.bs, w.h, w.top_k, w.experts, dtype=O.DT_BF16, quant_mode=quant, capacity=w.capacity)
+    idn = ids.numpy()
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        d = O.mem_dispatch(case, 0, xb[None], idn[None])
+        t1 = time.perf_counter()
+        O.mem_combine(O.Case(1, w.bs, w.h, w.top_k, w.experts, dtype=O.DT_BF16), 0, d["expand_x"][None]
+                      if quant else d["expand_x"].view(np.uint16)[None], d["assist"][None], d["send_counts"][None],
+                      expert_scales=weights.numpy(), in_quant=quant if quant else 0,
+                      in_scales=d["dyn_scales"] if quant else None)
+        t2 = time.perf_counter()
+        if best is None or t2 - t0 < best[0]:
+            best = (t2 - t0, t1 - t0, t2 - t1)
+    db, cb = workloads.algorithmic_bytes(w, kept_rows, inverse_index=True)
+    return {
+        "value": round((db + cb) / best[0] / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "us_per_layer": round(best[0] * 1e6, 1), "dispatch_us": round(best[1] * 1e6, 1),
+        "combine_us": round(best[2] * 1e6, 1), "host_cores_available": os.cpu_count(),
+        "sample": f"full {w.name} layer ({w.bs} tokens), oracle C port, single thread, best of 3",
+    }
+
+
+def main():
+    args = parse()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one device's share of the dispatch/combine path: run it with --gpus 1 "
+              "(no collective or second GPU is part of this build)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    from tilexr_amd import ep, workloads
+
+    w = workloads.CONFIGS[args.workload]
+    x = workloads.make_x(w)
+    ids, weights = workloads.make_routing(w)
+    bs, h, K, E = w.bs, w.h, w.top_k, w.experts
+    quant = {"none": ep.Q_NONE, "int8": ep.Q_TOKEN_INT8, "fp8_block128": ep.Q_FP8_BLOCK128}[w.quant]
+
+    torch.cuda.set_device(0)
+    dev = "cuda:0"
+    stream = torch.cuda.Stream()
+    comm = ep.Comm(1, 0)
+    rows_max = bs * K
+    row_bytes = h * 2 if quant == ep.Q_NONE else h
+    d_x, d_ids, d_w = x.to(dev), ids.to(dev), weights.to(dev)
+    expand_x = torch.empty((rows_max, row_bytes), dtype=torch.uint8, device=dev)
+    assist = torch.empty((rows_max, 4), dtype=torch.int32, device=dev)
+    token_nums = torch.empty((E,), dtype=torch.int64, device=dev)
+    send_counts = torch.empty((E,), dtype=torch.int32, device=dev)
+    row_map = torch.empty((bs, K), dtype=torch.int32, device=dev)
+    y = torch.empty((bs, h), dtype=torch.bfloat16, device=dev)
+    scales = None
+    if quant == ep.Q_TOKEN_INT8:
+        scales = torch.empty((rows_max,), dtype=torch.float32, device=dev)
+    elif quant == ep.Q_FP8_BLOCK128:
+        scales = torch.empty((rows_max, (h + 127) // 128), dtype=torch.float32, device=dev)
+
+    def step():
+        st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
+                                      ep.DT_BF16, stream, quant_mode=quant, expert_capacity=w.capacity,
+                                      dynamic_scales=scales, row_index_map=row_map)
+        ep.check(st, "dispatch")
+        ep.check(ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
+                                      expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
+                                      row_index_map=row_map), "combine")
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    kept_rows = int(send_counts[-1].item())
+    dispatch_bytes, combine_bytes = workloads.algorithmic_bytes(w, kept_rows, inverse_index=True)
+
+    # per-kernel events: one (start, stop) pair per step for the scatter and the reduce kernel
+    pairs = []
+    use_events = not args.no_kernel_events
+    if use_events:
+        pairs = [[(ep.HipEvent(timing=True), ep.HipEvent(timing=True)) for _ in range(args.steps)] for _ in range(2)]
+    d_ev = [ep.HipEvent(timing=True) for _ in range(3)]
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        if use_events:
+            ep.set_kernel_timing_events(comm, ep.K_SCATTER, *pairs[0][i])
+            ep.set_kernel_timing_events(comm, ep.K_REDUCE, *pairs[1][i])
+        step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    for k in (ep.K_SCATTER, ep.K_REDUCE):
+        ep.set_kernel_timing_events(comm, k, None, None)
+
+    # split of one step into its two calls (outside the timed region)
+    d_ev[0].record(stream)
+    st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts, ep.DT_BF16,
+                                  stream, quant_mode=quant, expert_capacity=w.capacity, dynamic_scales=scales,
+                                  row_index_map=row_map)
+    d_ev[1].record(stream)
+    ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
+                         expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w, row_index_map=row_map)
+    d_ev[2].record(stream)
+    torch.cuda.synchronize()
+    dispatch_us = d_ev[0].elapsed_ms(d_ev[1]) * 1e3
+    combine_us = d_ev[1].elapsed_ms(d_ev[2]) * 1e3
+
+    ms_per_step = elapsed / args.steps * 1e3
+    total_bytes = dispatch_bytes + combine_bytes
+    gbps = total_bytes / (ms_per_step * 1e-3) / 1e9
+
+    roofline = None
+    kernels = {}
+    if use_events:
+        for name, plist, nbytes in (("scatter", pairs[0], dispatch_bytes), ("reduce", pairs[1], combine_bytes)):
+            times = sorted(a.elapsed_ms(b) * 1e3 for a, b in plist)
+            avg = sum(times) / len(times)
+            kernels[name] = {"avg_us": round(avg, 2), "min_us": round(times[0], 2), "p50_us": round(times[len(times) // 2], 2),
+                             "max_us": round(times[-1], 2), "algorithmic_bytes": nbytes,
+                             "achieved_GBps": round(nbytes / (avg * 1e-6) / 1e9, 1)}
+        dom = "scatter" if kernels["scatter"]["avg_us"] >= kernels["reduce"]["avg_us"] else "reduce"
+        roofline = {"bound": "hbm", "kernel": "ep_scatter_vec_kernel" if dom == "scatter" else "ep_reduce_vec_kernel",
+                    "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                    "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "avg_launch_us": kernels[dom]["avg_us"], "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
+
+    result = {
+        "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "us_per_layer": round(ms_per_step * 1e3, 2),
+        "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": dict(workloads.describe(w, ids), kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+                       combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
+        "roofline": roofline, "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = cpu_baseline(w, x, ids, weights, kept_rows)
+    comm.destroy()
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,183 @@
+// libtilexr-ep for one MI355X: MoE expert-parallel dispatch and combine.
+//
+// Part 1 declares the eight entry points of the reference's EP library (src/include/tilexr_ep.h:23-71) with the
+// same names, argument order, argument meaning and return codes, so code written against that header links
+// against this library unchanged.  `aclrtStream` is an opaque pointer there; here it carries a `hipStream_t`.
+// All tensor arguments are caller-owned device memory (HBM), every call is asynchronous on `stream`, and
+// validation happens before a magic is drawn or anything is enqueued (reference:
+// src/ep/host/ep_kernel_launch.cpp:304-317).
+//
+// Part 2 declares additions that have no counterpart in the reference; each says so.
+//
+// Common contract (reference: src/ep/host/ep_host.h:17-78, src/ep/common/ep_window.h:47-52):
+//   x                     [bs, h] fp16 / bf16, row-major
+//   expertIds             [bs, topK] int32; ids outside [0, moeExpertNum) are skipped, not errors
+//   expandXOut            [rows, h] rows gathered for this rank's experts (same type as x, or int8 / fp8)
+//   assistInfoForCombine  [rows, 4] int32 = {srcRank, tokenId, topKId, expertId}
+//   expertTokenNumsOut    [localExpertNum] int64; type 1 = counts, type 0 = inclusive prefix sum
+//   counts                MVP route: epRecvCounts[srcRank] plain counts;
+//                         memory route: sendCounts[localExpert * rankSize + srcRank] inclusive prefix sum
+//   yOut                  [bs, h] combined rows in token order
+// Row order on a destination rank: MVP route = source rank, token, topK; memory route = local expert, source rank,
+// route order (expert-contiguous).
+#ifndef TILEXR_EP_H
+#define TILEXR_EP_H
+
+#ifdef __cplusplus
+
+#include <cstdint>
+
+#include "tilexr_api.h"
+#include "tilexr_types.h"
+
+#ifndef TILEXR_EP_HAVE_ACL_STREAM
+typedef void *aclrtStream;   // holds a hipStream_t
+#endif
+
+namespace TileXREp {
+
+// reference: src/include/tilexr_ep.h:14-18
+enum TileXREpActiveMaskType : int64_t {
+    TILEXR_EP_ACTIVE_MASK_NONE = 0,
+    TILEXR_EP_ACTIVE_MASK_TOKEN = 1,    // bool [bs]
+    TILEXR_EP_ACTIVE_MASK_EXPERT = 2,   // bool [bs, topK] (memory-route dispatch only)
+};
+
+// quantMode values accepted by the entry points below
+enum TileXREpQuantMode : int64_t {
+    TILEXR_EP_QUANT_NONE = 0,
+    TILEXR_EP_QUANT_STATIC_INT8 = 1,        // MVP dispatch: q = clamp(round(x * scales[0]))
+    TILEXR_EP_QUANT_TOKEN_INT8 = 2,         // per-row absmax int8 with one fp32 scale per row
+    TILEXR_EP_QUANT_COMM_MXFP8_E5M2 = 3,    // memory combine: rows cross the exchange as MXFP8 e5m2
+    TILEXR_EP_QUANT_MXFP8 = 4,              // memory dispatch: MXFP8 output; memory combine: MXFP8 e4m3 exchange
+    TILEXR_EP_QUANT_FP8_BLOCK128 = 5,       // Part 2 only: fp8 e4m3 with one fp32 scale per 128 columns
+};
+
+} // namespace TileXREp
+
+extern "C" {
+
+// ---------------------------------------------------------------------------------------------------------
+// Part 1: the reference's entry points
+// ---------------------------------------------------------------------------------------------------------
+
+// reference: src/include/tilexr_ep.h:25-28, src/ep/host/tilexr_ep_dispatch.cpp:85-94
+int TileXRMoeEpDispatch(void *x, int32_t *expertIds, TileXRCommPtr comm,
+    int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    void *expandXOut, int64_t *expertTokenNumsOut, int32_t *epRecvCountsOut,
+    int32_t *assistInfoForCombineOut, TileXR::TileXRDataType dtype, aclrtStream stream);
+
+// reference: src/include/tilexr_ep.h:30-33, src/ep/host/tilexr_ep_memory_dispatch.cpp:73-82
+int TileXRMoeEpDispatchMemory(void *x, int32_t *expertIds, TileXRCommPtr comm,
+    int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    void *expandXOut, int64_t *expertTokenNumsOut, int32_t *sendCountsOut,
+    int32_t *assistInfoForCombineOut, TileXR::TileXRDataType dtype, aclrtStream stream);
+
+// reference: src/include/tilexr_ep.h:35-37, src/ep/host/tilexr_ep_dispatch.cpp:96-102
+int TileXRMoeEpCombine(void *expertOut, int32_t *assistInfoForCombine, int32_t *epRecvCounts,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    void *yOut, TileXR::TileXRDataType dtype, aclrtStream stream);
+
+// reference: src/include/tilexr_ep.h:39-41, src/ep/host/tilexr_ep_memory_combine.cpp:61-68
+int TileXRMoeEpCombineMemory(void *expertOut, int32_t *assistInfoForCombine, int32_t *epRecvCounts,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    void *yOut, TileXR::TileXRDataType dtype, aclrtStream stream);
+
+// reference: src/include/tilexr_ep.h:43-45, src/ep/host/tilexr_ep_dispatch.cpp:104-123
+int TileXRMoeEpCombineV2(void *expertOut, int32_t *assistInfoForCombine, int32_t *epRecvCounts,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    void *yOut, void *workspace, TileXR::TileXRDataType dtype, aclrtStream stream);
+
+// reference: src/include/tilexr_ep.h:47-52, src/ep/host/tilexr_ep_memory_combine.cpp:25-59
+int TileXRMoeEpCombineMemoryV2(void *expertOut, int32_t *assistInfoForCombine, int32_t *sendCounts,
+    float *expertScales, bool *xActiveMask, int64_t activeMaskType, void *sharedExpertX,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    int64_t epWorldSize, int64_t epRankId, int64_t tpWorldSize, int64_t tpRankId,
+    int64_t expertShardType, int64_t sharedExpertNum, int64_t sharedExpertRankNum,
+    int64_t quantMode, int64_t globalBs, void *yOut, TileXR::TileXRDataType dtype, aclrtStream stream);
+
+// reference: src/include/tilexr_ep.h:54-60, src/ep/host/tilexr_ep_dispatch.cpp:42-83
+int TileXRMoeEpDispatchV2(void *x, int32_t *expertIds, void *scales, bool *xActiveMask, void *expertScales,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum, int64_t epWorldSize,
+    int64_t epRankId, int64_t tpWorldSize, int64_t tpRankId, int64_t expertShardType, int64_t sharedExpertNum,
+    int64_t sharedExpertRankNum, int64_t quantMode, int64_t globalBs, int64_t expertTokenNumsType, void *expandXOut,
+    void *dynamicScalesOut, int32_t *assistInfoForCombineOut, int64_t *expertTokenNumsOut, int32_t *epRecvCountsOut,
+    int32_t *tpRecvCountsOut, void *expandScalesOut, void *workspace, TileXR::TileXRDataType dtype,
+    aclrtStream stream);
+
+// reference: src/include/tilexr_ep.h:62-69, src/ep/host/tilexr_ep_memory_dispatch.cpp:27-71
+int TileXRMoeEpDispatchMemoryV2(void *x, int32_t *expertIds, void *scales, bool *xActiveMask,
+    int64_t activeMaskType, void *expertScales, TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK,
+    int64_t moeExpertNum,
+    int64_t epWorldSize, int64_t epRankId, int64_t tpWorldSize, int64_t tpRankId, int64_t expertShardType,
+    int64_t sharedExpertNum, int64_t sharedExpertRankNum, int64_t quantMode, int64_t globalBs,
+    int64_t expertTokenNumsType, void *expandXOut, void *dynamicScalesOut, int32_t *assistInfoForCombineOut,
+    int64_t *expertTokenNumsOut, int32_t *sendCountsOut, int32_t *tpRecvCountsOut, void *expandScalesOut,
+    TileXR::TileXRDataType dtype, TileXR::TileXRDataType expandXOutDtype, aclrtStream stream);
+
+// ---------------------------------------------------------------------------------------------------------
+// Part 2: additions without a counterpart in the reference
+// ---------------------------------------------------------------------------------------------------------
+
+// Options of the extended memory-route calls.  Zero-initialise, then set what is needed.
+struct TileXREpDispatchExOptions {
+    int64_t quantMode;            // 0, 2 (input decoded by `dtype`), 4, 5
+    int64_t expertCapacity;       // > 0: a source rank sends at most this many rows per expert, lowest flat
+                                  //      route indices first; dropped routes get no row
+    int64_t expertTokenNumsType;  // 0 prefix sum, 1 counts
+    int64_t activeMaskType;
+    bool *xActiveMask;
+    int32_t *rowIndexMapOut;      // optional [bs, topK]: row of each route in expandXOut, -1 when it has none
+    uint64_t *tileFlagsOut;       // optional readiness words, one per `tileRows` rows of expandXOut:
+                                  //      (epoch << 32) | rows landed, release-published at agent scope
+    int64_t tileRows;
+    int64_t *epochOut;            // optional host pointer: receives the epoch the flags are tagged with
+    void *metaReadyEvent;         // optional hipEvent_t recorded on `stream` once counts, assist tuples,
+                                  //      rowIndexMapOut and the reset flag words are enqueued (before rows move)
+};
+
+// Memory-route dispatch (same outputs and order as TileXRMoeEpDispatchMemoryV2) for one rank per device, with
+// per-token int8 / block fp8 payloads, per-expert capacity and tile readiness flags.  No reference counterpart:
+// the reference's memory route accepts quantMode 0 and 4 only and has no capacity or caller-visible flags.
+int TileXRMoeEpDispatchMemoryEx(void *x, int32_t *expertIds, TileXRCommPtr comm, int64_t bs, int64_t h,
+    int64_t topK, int64_t moeExpertNum, const TileXREpDispatchExOptions *options, void *expandXOut,
+    void *dynamicScalesOut, int32_t *assistInfoForCombineOut, int64_t *expertTokenNumsOut, int32_t *sendCountsOut,
+    TileXR::TileXRDataType dtype, TileXR::TileXRDataType expandXOutDtype, aclrtStream stream);
+
+struct TileXREpCombineExOptions {
+    int64_t commQuantMode;        // 0, 3, 4: as quantMode of TileXRMoeEpCombineMemoryV2
+    int64_t expertOutQuantMode;   // 0: expertOut is `dtype`; 2 / 5: expertOut holds int8 / fp8 e4m3 rows that are
+                                  //    dequantised with expertOutScales, rounded to `dtype`, then reduced
+    void *expertOutScales;        // fp32 [rows] (mode 2) or [rows, ceil(h/128)] (mode 5)
+    float *expertScales;          // optional gate weights [bs, topK]
+    int64_t activeMaskType;       // NONE or TOKEN
+    bool *xActiveMask;
+    void *sharedExpertX;          // optional [bs, h]
+    const int32_t *rowIndexMap;   // optional [bs, topK] from dispatch: skips rebuilding the inverse map
+    const uint64_t *tileFlags;    // optional: wait (acquire, agent scope) for the tiles of each row read
+    int64_t tileRows;
+    int64_t flagEpoch;            // epoch the producer tags its flag words with
+    int64_t waitTimeoutUs;        // bound of every flag wait; 0 = library default (2 s)
+    int32_t *deviceStatusOut;     // optional device int32: set to 1 when a flag wait expired
+};
+
+// Memory-route combine (same result as TileXRMoeEpCombineMemoryV2) with quantised expert output, a ready-made
+// inverse map and tile readiness flags, so tiles can be reduced as soon as the expert stage publishes them.
+// No reference counterpart: there the flag protocol is private to the kernels.
+int TileXRMoeEpCombineMemoryEx(void *expertOut, int32_t *assistInfoForCombine, int32_t *sendCounts,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    const TileXREpCombineExOptions *options, void *yOut, TileXR::TileXRDataType dtype, aclrtStream stream);
+
+// Measurement aid without a reference counterpart: while a pair of hipEvent_t is set for a kernel, every call on
+// `comm` that launches that kernel records `startEvent` immediately before and `stopEvent` immediately after it, on
+// the stream of the call.  Pass null events to clear.  Kernel ids: 0 count, 1 place, 2 scatter, 3 invert, 4 reduce.
+int TileXREpSetKernelTimingEvents(TileXRCommPtr comm, int kernel, void *startEvent, void *stopEvent);
+
+// Library build identification ("tilexr-ep gfx950 <abi version>").
+const char *TileXREpVersion(void);
+
+}
+
+#endif // __cplusplus
+
+#endif // TILEXR_EP_H

@@ -1,0 +1,65 @@
+"""Drives libtilexr-ep through its C ABI with torch tensors as device memory, and fetches results as numpy arrays
+shaped like the oracle's outputs (tests/ and the smoke check use it)."""
+import numpy as np
+import torch
+
+from tilexr_amd import ep
+
+DEV = "cuda:0"
+
+
+def to_dev(a):
+    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+
+
+def bits16(t):
+    """bf16/fp16 torch tensor -> uint16 numpy."""
+    return t.contiguous().view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+class Session:
+    """One communicator (single rank) + a non-default stream."""
+
+    def __init__(self, rank_size=1, rank=0):
+        torch.cuda.set_device(0)
+        self.comm = ep.Comm(rank_size, rank)
+        self.stream = torch.cuda.Stream()
+
+    def close(self):
+        torch.cuda.synchronize()
+        self.comm.destroy()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def sync(self):
+        self.stream.synchronize()
+
+
+def alloc_dispatch_outputs(bs, h, top_k, experts, ranks=1, quant=ep.Q_NONE, fill=0x5a):
+    rows = ranks * bs * top_k
+    row_bytes = h * 2 if quant == ep.Q_NONE else h
+    out = dict(
+        expand_x=torch.full((rows, row_bytes), fill, dtype=torch.uint8, device=DEV),
+        assist=torch.full((rows, 4), -77, dtype=torch.int32, device=DEV),
+        token_nums=torch.full((experts // ranks,), -5, dtype=torch.int64, device=DEV),
+        row_map=torch.full((bs, top_k), -9, dtype=torch.int32, device=DEV),
+    )
+    if quant == ep.Q_MXFP8:
+        out["scales"] = torch.full((rows, ((h + 31) // 32 + 1) // 2 * 2), 0xee, dtype=torch.uint8, device=DEV)
+    elif quant == ep.Q_FP8_BLOCK128:
+        out["scales"] = torch.full((rows, (h + 127) // 128), -3.0, dtype=torch.float32, device=DEV)
+    elif quant in (ep.Q_TOKEN_INT8,):
+        out["scales"] = torch.full((rows, 1), -3.0, dtype=torch.float32, device=DEV)
+    else:
+        out["scales"] = None
+    return out
+
+
+def fetch(out, counts_name, counts):
+    res = {k: (None if v is None else v.cpu().numpy()) for k, v in out.items()}
+    res[counts_name] = counts.cpu().numpy()
+    return res

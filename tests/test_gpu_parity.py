@@ -1,0 +1,343 @@
+"""GPU parity: the HIP path, called through the C ABI, against the CPU oracle on the same seeded inputs.
+
+Integer / byte outputs (row order, counts, source-index map, int8 / fp8 payloads, scales) must be bit-exact.
+Combine outputs are compared bit-exactly too, because the kernels reproduce the reference's order of roundings;
+the looser bound the workload definition allows (1e-2 relative) is only used for the full-size property checks.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_harness import DEV, Session, alloc_dispatch_outputs, bits16, fetch, to_dev
+from oracle import ep as O
+from tilexr_amd import ep, workloads
+
+pytestmark = pytest.mark.gpu
+
+
+def ids_for(rng, bs, K, E, invalid=0.0):
+    ids = np.stack([rng.permutation(E)[:K] if E >= K else rng.integers(0, E, K) for _ in range(bs)]).astype(np.int32)
+    if invalid:
+        bad = rng.random(ids.shape) < invalid
+        ids[bad] = rng.choice([-1, -9, E, E + 3], size=int(bad.sum()))
+    return ids
+
+
+def x_for(rng, bs, h, dtype, scale=1.0):
+    f = (rng.standard_normal((bs, h)) * scale).astype(np.float32)
+    t = torch.from_numpy(f).to(torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16)
+    return t, bits16(t)
+
+
+def check_dispatch(got, want, rows_key="rows"):
+    n = want[rows_key]
+    assert np.array_equal(got["assist"][:n], want["assist"][:n])
+    assert np.array_equal(got["expand_x"][:n], want["expand_x"][:n])
+    assert np.array_equal(got["token_nums"], want["expert_token_nums"])
+    # rows beyond the last valid one are never written
+    assert np.all(got["assist"][n:] == -77)
+
+
+SHAPES = [(7, 8, 2, 5), (64, 64, 4, 16), (33, 40, 3, 7), (16, 33, 2, 4), (300, 1024, 8, 64), (2100, 256, 8, 256),
+          (128, 7168, 8, 256), (5, 16400, 2, 4)]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+def test_memory_dispatch_matches_oracle(shape, dtype):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + dtype)
+    ids = ids_for(rng, bs, K, E, invalid=0.1)
+    xt, xb = x_for(rng, bs, h, dtype)
+    with Session() as s:
+        for mask_type in (ep.MASK_NONE, ep.MASK_TOKEN, ep.MASK_EXPERT):
+            mask = None
+            if mask_type == ep.MASK_TOKEN:
+                mask = (rng.random(bs) < 0.7).astype(np.uint8)
+            elif mask_type == ep.MASK_EXPERT:
+                mask = (rng.random((bs, K)) < 0.7).astype(np.uint8)
+            for nums_type in (0, 1):
+                out = alloc_dispatch_outputs(bs, h, K, E)
+                counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
+                st = ep.dispatch_memory_v2(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                           out["token_nums"], counts, dtype, s.stream, active_mask=to_dev(mask),
+                                           active_mask_type=mask_type, token_nums_type=nums_type)
+                assert st == 0
+                s.sync()
+                got = fetch(out, "send_counts", counts)
+                case = O.Case(1, bs, h, K, E, dtype=dtype, mask_type=mask_type, token_nums_type=nums_type)
+                want = O.mem_dispatch(case, 0, xb[None], ids[None], None if mask is None else mask[None])
+                check_dispatch(got, want)
+                assert np.array_equal(got["send_counts"], want["send_counts"])
+
+
+@pytest.mark.parametrize("shape", SHAPES[:6])
+def test_mvp_dispatch_matches_oracle(shape):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + 99)
+    ids = ids_for(rng, bs, K, E, invalid=0.1)
+    xt, xb = x_for(rng, bs, h, ep.DT_FP16, scale=3.0)
+    mask = (rng.random(bs) < 0.7).astype(np.uint8)
+    static = np.array([1.75], np.float32)
+    with Session() as s:
+        for quant in (ep.Q_NONE, ep.Q_STATIC_INT8, ep.Q_TOKEN_INT8):
+            for use_mask in (False, True):
+                for nums_type in (1, 0):
+                    out = alloc_dispatch_outputs(bs, h, K, E, quant=quant)
+                    counts = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+                    tp_counts = torch.full((1,), -1, dtype=torch.int32, device=DEV)
+                    st = ep.dispatch_v2(
+                        xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"], out["token_nums"],
+                        counts, ep.DT_FP16 if quant == ep.Q_NONE else ep.DT_INT8, s.stream,
+                        scales=to_dev(static) if quant == ep.Q_STATIC_INT8 else None,
+                        active_mask=to_dev(mask) if use_mask else None, quant_mode=quant, token_nums_type=nums_type,
+                        dynamic_scales=out["scales"] if quant == ep.Q_TOKEN_INT8 else None, tp_recv_counts=tp_counts)
+                    assert st == 0
+                    s.sync()
+                    got = fetch(out, "recv_counts", counts)
+                    case = O.Case(1, bs, h, K, E, dtype=O.DT_FP16, quant_mode=quant, token_nums_type=nums_type)
+                    want = O.mvp_dispatch(case, 0, xb[None], ids[None], mask[None] if use_mask else None, static)
+                    check_dispatch(got, want)
+                    assert np.array_equal(got["recv_counts"], want["recv_counts"])
+                    assert tp_counts.item() == want["recv_counts"][0]
+                    if quant == ep.Q_TOKEN_INT8:
+                        n = want["rows"]
+                        assert np.array_equal(got["scales"][:n, 0], want["dyn_scales"][:n])
+
+
+def test_simple_entry_points():
+    bs, h, K, E = 50, 128, 4, 32
+    rng = np.random.default_rng(5)
+    ids = ids_for(rng, bs, K, E)
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+    w = np.ones((bs, K), np.float32)
+    with Session() as s:
+        for memory in (True, False):
+            out = alloc_dispatch_outputs(bs, h, K, E)
+            counts = torch.zeros((E if memory else 1,), dtype=torch.int32, device=DEV)
+            fn = ep.dispatch_memory if memory else ep.dispatch
+            assert fn(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["token_nums"], counts,
+                      out["assist"], ep.DT_BF16, s.stream) == 0
+            y = torch.zeros((bs, h), dtype=torch.bfloat16, device=DEV)
+            fnc = ep.combine_memory if memory else ep.combine
+            assert fnc(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream) == 0
+            s.sync()
+            case = O.Case(1, bs, h, K, E, token_nums_type=1)
+            want = (O.mem_dispatch if memory else O.mvp_dispatch)(case, 0, xb[None], ids[None])
+            got = fetch(out, "counts", counts)
+            check_dispatch(got, want)
+            eo = want["expand_x"].view(np.uint16)[None]
+            if memory:
+                wy = O.mem_combine(case, 0, eo, want["assist"][None], want["send_counts"][None])
+            else:
+                wy = O.mvp_combine(case, 0, eo, want["assist"][None], want["recv_counts"][None])
+            assert np.array_equal(bits16(y), wy)
+    del w
+
+
+QUANT_SHAPES = [(40, 256, 4, 8), (17, 40, 2, 4), (9, 33, 2, 4), (130, 4096, 6, 64), (64, 2048, 8, 128),
+                (20, 7168, 8, 256)]
+
+
+@pytest.mark.parametrize("shape", QUANT_SHAPES)
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+@pytest.mark.parametrize("quant,fp8", [(ep.Q_TOKEN_INT8, None), (ep.Q_MXFP8, ep.DT_FP8E4M3), (ep.Q_MXFP8, ep.DT_FP8E5M2),
+                                       (ep.Q_FP8_BLOCK128, None)])
+def test_quantised_dispatch_matches_oracle(shape, dtype, quant, fp8):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + dtype + quant)
+    ids = ids_for(rng, bs, K, E, invalid=0.05)
+    xt, xb = x_for(rng, bs, h, dtype, scale=2.0)
+    xb[0, :] = 0                       # an all-zero row
+    if h >= 64:
+        xb[1, 32:64] = 0               # an all-zero block
+    xt = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16)
+    with Session() as s:
+        out = alloc_dispatch_outputs(bs, h, K, E, quant=quant)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        st, _ = ep.dispatch_memory_ex(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, dtype, s.stream, quant_mode=quant,
+                                      dynamic_scales=out["scales"], expand_x_dtype=fp8, row_index_map=out["row_map"])
+        assert st == 0
+        s.sync()
+        got = fetch(out, "send_counts", counts)
+        case = O.Case(1, bs, h, K, E, dtype=dtype, quant_mode=quant, out_dtype=fp8 or O.DT_FP8E4M3)
+        want = O.mem_dispatch(case, 0, xb[None], ids[None])
+        check_dispatch(got, want)
+        n = want["rows"]
+        assert np.array_equal(got["scales"][:n], want["dyn_scales"][:n])
+        # the row map is the inverse of the assist tuples
+        rm = got["row_map"]
+        for row in range(n):
+            _, t, k, _ = want["assist"][row]
+            assert rm[t, k] == row
+        assert (rm >= 0).sum() == n
+        if quant == ep.Q_MXFP8:
+            # the reference API takes the same mode through DispatchMemoryV2
+            out2 = alloc_dispatch_outputs(bs, h, K, E, quant=quant)
+            st = ep.dispatch_memory_v2(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out2["expand_x"], out2["assist"],
+                                       out2["token_nums"], counts, dtype, s.stream, quant_mode=4,
+                                       dynamic_scales=out2["scales"], expand_x_dtype=fp8)
+            assert st == 0
+            s.sync()
+            assert torch.equal(out2["expand_x"][:n], out["expand_x"][:n])
+            assert torch.equal(out2["scales"][:n], out["scales"][:n])
+
+
+def test_capacity_drop_matches_oracle():
+    rng = np.random.default_rng(77)
+    bs, h, K, E, cap = 700, 64, 8, 16, 300
+    w = workloads.Workload("t", 1, bs, h, K, E, routing="zipf", zipf_s=1.2, seed=3)
+    ids = workloads.make_routing(w)[0].numpy()
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+    with Session() as s:
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        st, _ = ep.dispatch_memory_ex(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, ep.DT_BF16, s.stream, expert_capacity=cap,
+                                      row_index_map=out["row_map"])
+        assert st == 0
+        s.sync()
+        got = fetch(out, "send_counts", counts)
+        want = O.mem_dispatch(O.Case(1, bs, h, K, E, capacity=cap), 0, xb[None], ids[None])
+        assert want["rows"] < bs * K                     # something was dropped
+        assert want["expert_token_nums"].max() == cap
+        check_dispatch(got, want)
+        assert np.array_equal(got["send_counts"], want["send_counts"])
+        assert (got["row_map"] >= 0).sum() == want["rows"]
+
+
+COMBINE_SHAPES = [(7, 8, 2, 5), (64, 64, 4, 16), (33, 40, 3, 7), (16, 33, 2, 4), (100, 1024, 8, 64),
+                  (40, 7168, 8, 256), (3, 16400, 2, 4)]
+
+
+@pytest.mark.parametrize("shape", COMBINE_SHAPES)
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+def test_memory_combine_matches_oracle(shape, dtype):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + 3 * dtype)
+    ids = ids_for(rng, bs, K, E, invalid=0.1)
+    xt, xb = x_for(rng, bs, h, dtype, scale=3.0)
+    case = O.Case(1, bs, h, K, E, dtype=dtype)
+    d = O.mem_dispatch(case, 0, xb[None], ids[None])
+    rows = d["rows"]
+    eo = d["expand_x"].view(np.uint16).copy()
+    for r in range(rows):
+        eo[r] = np.roll(eo[r], r % 5)          # make every route's row different
+    w = (0.25 + rng.random((bs, K))).astype(np.float32)
+    w[0, 0] = 1.0
+    tmask = (rng.random(bs) < 0.8).astype(np.uint8)
+    _, sxb = x_for(rng, bs, h, dtype)
+    with Session() as s:
+        d_eo, d_assist, d_counts = to_dev(eo), to_dev(d["assist"]), to_dev(d["send_counts"])
+        for use_w, use_mask, use_shared in ((False, False, False), (True, False, False), (True, True, True)):
+            y = torch.full((bs, h), 7.0, dtype=torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16, device=DEV)
+            st = ep.combine_memory_v2(d_eo, d_assist, d_counts, s.comm, bs, h, K, E, y, dtype, s.stream,
+                                      expert_scales=to_dev(w) if use_w else None,
+                                      active_mask=to_dev(tmask) if use_mask else None,
+                                      active_mask_type=ep.MASK_TOKEN if use_mask else ep.MASK_NONE,
+                                      shared_expert_x=to_dev(sxb) if use_shared else None)
+            assert st == 0
+            s.sync()
+            want = O.mem_combine(case, 0, eo[None], d["assist"][None], d["send_counts"][None],
+                                 expert_scales=w if use_w else None, token_mask=tmask if use_mask else None,
+                                 shared_expert_x=sxb if use_shared else None)
+            assert np.array_equal(bits16(y), want)
+
+
+@pytest.mark.parametrize("shape", [(24, 64, 4, 16), (33, 96, 3, 7), (12, 1024, 8, 64), (6, 7168, 8, 256), (9, 40, 2, 4)])
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+@pytest.mark.parametrize("mode", [3, 4])
+def test_memory_combine_mxfp8_exchange_matches_oracle(shape, dtype, mode):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + dtype + mode)
+    ids = ids_for(rng, bs, K, E)
+    xt, xb = x_for(rng, bs, h, dtype, scale=4.0)
+    case = O.Case(1, bs, h, K, E, dtype=dtype)
+    d = O.mem_dispatch(case, 0, xb[None], ids[None])
+    eo = d["expand_x"].view(np.uint16)
+    w = (0.5 + rng.random((bs, K))).astype(np.float32)
+    with Session() as s:
+        y = torch.zeros((bs, h), dtype=torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16, device=DEV)
+        st = ep.combine_memory_v2(to_dev(eo), to_dev(d["assist"]), to_dev(d["send_counts"]), s.comm, bs, h, K, E, y,
+                                  dtype, s.stream, expert_scales=to_dev(w), quant_mode=mode)
+        assert st == 0
+        s.sync()
+        want = O.mem_combine(case, 0, eo[None], d["assist"][None], d["send_counts"][None], expert_scales=w,
+                             comm_quant=mode)
+        assert np.array_equal(bits16(y), want)
+
+
+@pytest.mark.parametrize("shape", [(24, 64, 4, 16), (12, 1024, 6, 64), (10, 2048, 8, 128), (9, 40, 2, 4), (5, 33, 2, 4)])
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+@pytest.mark.parametrize("quant", [ep.Q_TOKEN_INT8, ep.Q_FP8_BLOCK128])
+def test_quantised_combine_matches_oracle(shape, dtype, quant):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + dtype + quant)
+    ids = ids_for(rng, bs, K, E)
+    xt, xb = x_for(rng, bs, h, dtype, scale=2.0)
+    d = O.mem_dispatch(O.Case(1, bs, h, K, E, dtype=dtype, quant_mode=quant), 0, xb[None], ids[None])
+    w = (0.5 + rng.random((bs, K))).astype(np.float32)
+    with Session() as s:
+        y = torch.zeros((bs, h), dtype=torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16, device=DEV)
+        st = ep.combine_memory_ex(to_dev(d["expand_x"]), to_dev(d["assist"]), to_dev(d["send_counts"]), s.comm, bs, h,
+                                  K, E, y, dtype, s.stream, expert_out_quant_mode=quant,
+                                  expert_out_scales=to_dev(d["dyn_scales"]), expert_scales=to_dev(w))
+        assert st == 0
+        s.sync()
+        want = O.mem_combine(O.Case(1, bs, h, K, E, dtype=dtype), 0, d["expand_x"][None], d["assist"][None],
+                             d["send_counts"][None], expert_scales=w, in_quant=quant, in_scales=d["dyn_scales"])
+        assert np.array_equal(bits16(y), want)
+
+
+@pytest.mark.parametrize("shape", [(7, 8, 2, 5), (64, 64, 4, 16), (16, 33, 2, 4), (60, 1024, 8, 64), (20, 7168, 8, 256)])
+@pytest.mark.parametrize("dtype", [ep.DT_FP16, ep.DT_BF16])
+def test_mvp_combine_matches_oracle(shape, dtype):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + 11 * dtype)
+    ids = ids_for(rng, bs, K, E, invalid=0.1)
+    xt, xb = x_for(rng, bs, h, dtype, scale=20.0)
+    case = O.Case(1, bs, h, K, E, dtype=dtype)
+    d = O.mvp_dispatch(case, 0, xb[None], ids[None])
+    eo = d["expand_x"].view(np.uint16).copy()
+    for r in range(d["rows"]):
+        eo[r] = np.roll(eo[r], r % 3)
+    with Session() as s:
+        y = torch.full((bs, h), 3.0, dtype=torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16, device=DEV)
+        st = ep.combine_v2(to_dev(eo), to_dev(d["assist"]), to_dev(d["recv_counts"]), s.comm, bs, h, K, E, y, dtype,
+                           s.stream)
+        assert st == 0
+        s.sync()
+        want = O.mvp_combine(case, 0, eo[None], d["assist"][None], d["recv_counts"][None])
+        assert np.array_equal(bits16(y), want)
+
+
+def test_unsupported_requests_are_reported():
+    bs, h, K, E = 8, 64, 2, 4
+    with Session() as s:
+        x = torch.zeros((bs, h), dtype=torch.bfloat16, device=DEV)
+        ids = torch.zeros((bs, K), dtype=torch.int32, device=DEV)
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        base = (x, ids, s.comm, bs, h, K, E, out["expand_x"], out["assist"], out["token_nums"], counts, ep.DT_BF16)
+        assert ep.dispatch_memory_v2(*base, None) == ep.ERR_PARA_CHECK_FAIL                 # null stream
+        assert ep.dispatch_memory_v2(*base, s.stream, quant_mode=2) == ep.ERR_NOT_SUPPORT
+        assert ep.dispatch_memory_v2(*base, s.stream, tp_world_size=2) == ep.ERR_NOT_SUPPORT
+        assert ep.dispatch_memory_v2(*base, s.stream, global_bs=bs + 1) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.dispatch_memory_v2(*base, s.stream, ep_world_size=2) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.dispatch_memory_v2(*base, s.stream, active_mask_type=ep.MASK_TOKEN) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.dispatch_v2(*base, s.stream, quant_mode=3) == ep.ERR_NOT_SUPPORT
+        assert ep.dispatch_v2(*base, s.stream, quant_mode=2) == ep.ERR_PARA_CHECK_FAIL      # needs int8 + scales out
+        st, _ = ep.dispatch_memory_ex(*base, s.stream, quant_mode=1)
+        assert st == ep.ERR_NOT_SUPPORT
+        st, _ = ep.dispatch_memory_ex(*base, s.stream, quant_mode=5)                         # no scales buffer
+        assert st == ep.ERR_PARA_CHECK_FAIL
+        y = torch.zeros((bs, h), dtype=torch.bfloat16, device=DEV)
+        cb = (out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream)
+        assert ep.combine_memory_v2(*cb, quant_mode=2) == ep.ERR_NOT_SUPPORT
+        assert ep.combine_memory_v2(*cb, quant_mode=4) == ep.ERR_PARA_CHECK_FAIL            # needs expertScales
+        assert ep.combine_memory_v2(*cb, active_mask_type=ep.MASK_EXPERT, active_mask=y) == ep.ERR_NOT_SUPPORT
+        assert ep.combine_v2(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_INT8, s.stream) == \
+            ep.ERR_NOT_SUPPORT
+        # nothing above consumed a magic or launched anything
+        assert s.comm.next_magic() == 1

@@ -1,0 +1,691 @@
+// Entry points of libtilexr-ep and the orchestration of one call: validate -> draw a magic -> enqueue kernels.
+//
+// The order of the host-side steps follows the reference (src/ep/host/tilexr_ep_dispatch.cpp:8-22,
+// tilexr_ep_memory_dispatch.cpp:9-23, tilexr_ep_memory_combine.cpp:9-21, ep_kernel_launch.cpp:252-416):
+// basic argument check, communicator lookup, configuration check, magic, launch.  Success means "enqueued on the
+// caller's stream"; nothing here waits for the device.
+#include <cstdio>
+#include <limits>
+
+#include <hip/hip_runtime_api.h>
+
+#include "ep_context.h"
+#include "ep_host.h"
+#include "ep_launch.h"
+#include "tilexr_ep.h"
+
+namespace TileXREp {
+
+int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, int64_t magic);
+int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, int64_t magic);
+
+namespace {
+
+constexpr int kOk = TileXR::TILEXR_SUCCESS;
+constexpr int64_t kDefaultWaitUs = 2 * 1000 * 1000;
+constexpr int64_t kWallClockTicksPerUs = 100;      // wall_clock64() counts at 100 MHz on CDNA3/CDNA4
+
+int LaunchStatus(hipError_t err, const char *what)
+{
+    if (err == hipSuccess) {
+        return kOk;
+    }
+    // reference: src/ep/host/ep_kernel_launch.cpp:153,177 reports launch failures on stderr and returns MKIRT
+    std::fprintf(stderr, "tilexr-ep: launching %s failed: %s\n", what, hipGetErrorString(err));
+    return TileXR::TILEXR_ERROR_MKIRT;
+}
+
+// Records the caller's timing events (if any) around one kernel launch.
+template <typename Launch>
+int Timed(EpComm *comm, int kernel, hipStream_t stream, const char *what, Launch launch)
+{
+    hipEvent_t start = comm->timing[kernel][0];
+    hipEvent_t stop = comm->timing[kernel][1];
+    if (start != nullptr && hipEventRecord(start, stream) != hipSuccess) {
+        return TileXR::TILEXR_ERROR_INTERNAL;
+    }
+    const int ret = LaunchStatus(launch(), what);
+    if (ret == kOk && stop != nullptr && hipEventRecord(stop, stream) != hipSuccess) {
+        return TileXR::TILEXR_ERROR_INTERNAL;
+    }
+    return ret;
+}
+
+bool WithinKernelLimits(int64_t bs, int64_t h, int64_t topK, int64_t experts)
+{
+    const int64_t intMax = std::numeric_limits<int32_t>::max();
+    return experts <= kMaxKeys && topK <= kMaxTopK && bs <= intMax / topK && h <= intMax / 2 && bs * topK <= intMax / 4;
+}
+
+CountScratch CarveCountScratch(void *base, const CountScratchLayout &plan, bool expertHist)
+{
+    auto at = [base](int64_t off) { return reinterpret_cast<int32_t *>(static_cast<char *>(base) + off); };
+    CountScratch s {};
+    s.ticket = static_cast<uint32_t *>(base);
+    s.localRank = at(plan.localRankOff);
+    s.chunkHist = at(plan.chunkHistOff);
+    s.chunkExpHist = expertHist ? at(plan.chunkExpHistOff) : nullptr;
+    s.keyOffset = at(plan.keyOffsetOff);
+    s.keyKept = at(plan.keyKeptOff);
+    s.expertTotal = at(plan.expertTotalOff);
+    return s;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// one rank per device: rows go straight from x to expandXOut
+// ---------------------------------------------------------------------------------------------------------
+int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, int64_t magic)
+{
+    if (!WithinKernelLimits(p.bs, p.h, p.topK, p.moeExpertNum)) {
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+    }
+    hipStream_t stream = static_cast<hipStream_t>(p.stream);
+    const int64_t n = p.bs * p.topK;
+    const int64_t experts = p.moeExpertNum;
+    const int64_t numKeys = memoryRoute ? experts : 1;
+    const int64_t keyDiv = memoryRoute ? 1 : experts;
+    const bool expertHist = !memoryRoute;
+
+    std::lock_guard<std::mutex> lock(comm->mu);
+    const CountScratchLayout plan = PlanCountScratch(n, numKeys, experts, expertHist);
+    if (!comm->dispatchScratch.Reserve(static_cast<size_t>(plan.totalBytes), true)) {
+        return TileXR::TILEXR_ERROR_INTERNAL;
+    }
+    const CountScratch scratch = CarveCountScratch(comm->dispatchScratch.ptr, plan, expertHist);
+    int32_t *rowOf = p.rowIndexMapOut != nullptr ? p.rowIndexMapOut :
+        reinterpret_cast<int32_t *>(static_cast<char *>(comm->dispatchScratch.ptr) + plan.rowOfOff);
+
+    RouteCountLaunch count {};
+    count.ids = p.expertIds;
+    count.mask = reinterpret_cast<const uint8_t *>(p.xActiveMask);
+    if (p.xActiveMask == nullptr) {
+        count.maskMode = kMaskNone;
+    } else if (!memoryRoute) {
+        count.maskMode = kMaskPerToken;        // reference: tilexr_ep_dispatch_helpers.h:3-21
+    } else {
+        count.maskMode = p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT ? kMaskPerRoute : kMaskTokenPrefix;
+    }
+    count.bs = p.bs;
+    count.topK = p.topK;
+    count.numExperts = experts;
+    count.keyDiv = keyDiv;
+    count.numKeys = numKeys;
+    count.capacity = p.expertCapacity;
+    count.scratch = scratch;
+    count.sendCountsOut = memoryRoute ? p.epRecvCountsOut : nullptr;
+    count.recvCountOut = memoryRoute ? nullptr : p.epRecvCountsOut;
+    count.expertTokenNumsOut = p.expertTokenNumsOut;
+    count.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
+    count.stream = stream;
+    int ret = Timed(comm, kKernelCount, stream, "route count", [&] { return LaunchRouteCount(count); });
+    if (ret != kOk) {
+        return ret;
+    }
+    if (!memoryRoute && p.tpRecvCountsOut != nullptr) {
+        // reference: tilexr_ep_combine_helpers.h:93-95 mirrors the per-source count into tpRecvCounts
+        if (hipMemcpyAsync(p.tpRecvCountsOut, p.epRecvCountsOut, sizeof(int32_t), hipMemcpyDeviceToDevice, stream) !=
+            hipSuccess) {
+            return TileXR::TILEXR_ERROR_INTERNAL;
+        }
+    }
+
+    RoutePlaceLaunch place {};
+    place.ids = p.expertIds;
+    place.bs = p.bs;
+    place.topK = p.topK;
+    place.keyDiv = keyDiv;
+    place.numKeys = numKeys;
+    place.capacity = p.expertCapacity;
+    place.scratch = scratch;
+    place.srcRank = comm->rank;
+    place.expertIdBias = static_cast<int32_t>(p.sharedExpertNum);
+    place.rowOf = rowOf;
+    place.assist = p.assistInfoForCombineOut;
+    place.tileFlags = p.tileFlagsOut;
+    place.numTiles = p.tileFlagsOut != nullptr ? (n + p.tileRows - 1) / p.tileRows : 0;
+    place.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
+    place.stream = stream;
+    ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
+    if (ret != kOk) {
+        return ret;
+    }
+    if (p.metaReadyEvent != nullptr &&
+        hipEventRecord(static_cast<hipEvent_t>(p.metaReadyEvent), stream) != hipSuccess) {
+        return TileXR::TILEXR_ERROR_INTERNAL;
+    }
+
+    ScatterLaunch scatter {};
+    scatter.x = p.x;
+    scatter.rowOf = rowOf;
+    scatter.bs = p.bs;
+    scatter.h = p.h;
+    scatter.topK = p.topK;
+    scatter.quantMode = static_cast<int>(p.quantMode);
+    // the MVP route's quantisers decode the input as fp16 whatever the caller's tensor holds
+    // (reference: tilexr_ep_dispatch_helpers.h:121,167)
+    scatter.inputBf16 = memoryRoute && p.dtype == TileXR::TILEXR_DATA_TYPE_BFP16;
+    scatter.fp8E5m2 = p.expandXOutDtype == TileXR::TILEXR_DATA_TYPE_FP8E5M2;
+    scatter.staticScale = static_cast<const float *>(p.scales);
+    scatter.out = p.expandXOut;
+    scatter.scalesOut = p.dynamicScalesOut;
+    scatter.tileFlags = p.tileFlagsOut;
+    scatter.tileRows = p.tileRows;
+    scatter.stream = stream;
+    return Timed(comm, kKernelScatter, stream, "scatter", [&] { return LaunchScatter(scatter); });
+}
+
+int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, int64_t magic)
+{
+    if (!WithinKernelLimits(p.bs, p.h, p.topK, p.moeExpertNum)) {
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+    }
+    hipStream_t stream = static_cast<hipStream_t>(p.stream);
+    const int64_t n = p.bs * p.topK;
+    std::lock_guard<std::mutex> lock(comm->mu);
+
+    const uint64_t epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
+    uint64_t *inverse = nullptr;
+    if (p.rowIndexMap == nullptr) {
+        if (!comm->combineScratch.Reserve(static_cast<size_t>(n) * sizeof(uint64_t), true)) {
+            return TileXR::TILEXR_ERROR_INTERNAL;
+        }
+        inverse = static_cast<uint64_t *>(comm->combineScratch.ptr);
+        InvertLaunch inv {};
+        inv.assist = p.assistInfoForCombine;
+        inv.counts = p.epRecvCounts;
+        inv.numCounts = memoryRoute ? p.moeExpertNum : 1;
+        inv.countsArePrefix = memoryRoute;
+        inv.maxRows = n;
+        inv.maxCountPerEntry = n;
+        inv.rank = comm->rank;
+        inv.bs = p.bs;
+        inv.topK = p.topK;
+        inv.epoch = epoch;
+        inv.inverse = inverse;
+        inv.stream = stream;
+        const int ret = Timed(comm, kKernelInvert, stream, "invert", [&] { return LaunchInvert(inv); });
+        if (ret != kOk) {
+            return ret;
+        }
+    }
+
+    ReduceLaunch red {};
+    red.expertOut = p.expertOut;
+    red.rowBytes = p.expertOutQuantMode == 0 ? p.h * 2 : p.h;
+    red.inverseTagged = inverse;
+    red.epoch = epoch;
+    red.rowIndexMap = p.rowIndexMap;
+    red.expertScales = memoryRoute ? p.expertScales : nullptr;
+    red.tokenMask = memoryRoute ? reinterpret_cast<const uint8_t *>(p.xActiveMask) : nullptr;
+    red.sharedExpertX = memoryRoute ? p.sharedExpertX : nullptr;
+    red.reduceKind = memoryRoute ? kReduceFp32 : kReducePerAdd;
+    red.commQuant = memoryRoute ? static_cast<int>(p.quantMode) : 0;
+    red.inQuant = static_cast<int>(p.expertOutQuantMode);
+    red.inScales = static_cast<const float *>(p.expertOutScales);
+    red.bf16 = p.dtype == TileXR::TILEXR_DATA_TYPE_BFP16;
+    red.bs = p.bs;
+    red.h = p.h;
+    red.topK = p.topK;
+    red.y = p.yOut;
+    red.tileFlags = p.tileFlags;
+    red.tileRows = p.tileRows;
+    red.totalRowsPtr = p.epRecvCounts + (p.moeExpertNum - 1);
+    red.flagEpoch = static_cast<uint64_t>(p.flagEpoch) & 0xffffffffull;
+    red.waitTimeoutTicks = (p.waitTimeoutUs > 0 ? p.waitTimeoutUs : kDefaultWaitUs) * kWallClockTicksPerUs;
+    red.deviceStatus = p.deviceStatusOut;
+    red.numComputeUnits = comm->world->numComputeUnits;
+    red.stream = stream;
+    return Timed(comm, kKernelReduce, stream, "reduce", [&] { return LaunchReduce(red); });
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// shared call prologues
+// ---------------------------------------------------------------------------------------------------------
+int CommArgsOf(TileXRCommPtr handle, EpComm **comm, TileXR::CommArgs **args)
+{
+    // reference: src/ep/host/ep_launch_context.cpp:61-99, ep_dispatch_memory_host.cpp:108-135
+    *comm = LookupComm(handle);
+    if (*comm == nullptr) {
+        return TileXR::TILEXR_ERROR_NOT_INITIALIZED;
+    }
+    *args = &(*comm)->host;
+    return kOk;
+}
+
+int DispatchMvp(const EpDispatchParams &p)
+{
+    int ret = TileXREpValidateBasicDispatchParams(p);
+    if (ret != kOk) {
+        return ret;
+    }
+    EpComm *comm = nullptr;
+    TileXR::CommArgs *args = nullptr;
+    ret = CommArgsOf(p.comm, &comm, &args);
+    if (ret != kOk) {
+        return ret;
+    }
+    EpWindowConfig window {};
+    ret = TileXREpValidateDispatchConfigUncapped(p, *args, &window);
+    if (ret != kOk) {
+        return ret;
+    }
+    if ((p.tpWorldSize != 0 && p.tpWorldSize != 1) || p.sharedExpertNum != 0) {
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // tensor-parallel groups and shared experts: not built yet
+    }
+    int64_t magic = 0;
+    ret = TileXRCommNextMagic(p.comm, &magic);
+    if (ret != kOk) {
+        return ret;
+    }
+    return args->rankSize == 1 ? RunDispatchSingle(comm, p, false, magic) : RunDispatchMulti(comm, p, false, magic);
+}
+
+int DispatchMemory(const EpDispatchParams &p)
+{
+    int ret = TileXREpValidateBasicDispatchParams(p);
+    if (ret != kOk) {
+        return ret;
+    }
+    EpComm *comm = nullptr;
+    TileXR::CommArgs *args = nullptr;
+    ret = CommArgsOf(p.comm, &comm, &args);
+    if (ret != kOk) {
+        return ret;
+    }
+    EpMemoryDispatchReferenceConfig config {};
+    EpDispatchParams rules = p;
+    if (p.extended) {
+        // the extended call accepts payload formats the reference's memory route rejects; its rule check runs with
+        // the nearest reference mode and the additions are checked here
+        if (p.quantMode != TILEXR_EP_QUANT_NONE && p.quantMode != TILEXR_EP_QUANT_TOKEN_INT8 &&
+            p.quantMode != TILEXR_EP_QUANT_MXFP8 && p.quantMode != TILEXR_EP_QUANT_FP8_BLOCK128) {
+            return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+        }
+        if (p.expertCapacity < 0 || (p.tileFlagsOut != nullptr && p.tileRows <= 0)) {
+            return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+        }
+        if (p.quantMode == TILEXR_EP_QUANT_TOKEN_INT8 || p.quantMode == TILEXR_EP_QUANT_FP8_BLOCK128) {
+            const TileXR::TileXRDataType want = p.quantMode == TILEXR_EP_QUANT_TOKEN_INT8 ?
+                TileXR::TILEXR_DATA_TYPE_INT8 : TileXR::TILEXR_DATA_TYPE_FP8E4M3;
+            if (p.dynamicScalesOut == nullptr || p.expandXOutDtype != want) {
+                return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+            }
+            rules.quantMode = TILEXR_EP_QUANT_NONE;
+            rules.dynamicScalesOut = nullptr;
+            rules.expandXOutDtype = p.dtype;
+        }
+        if (args->rankSize != 1) {
+            return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+        }
+    }
+    ret = TileXREpValidateDispatchMemoryConfig(rules, *args, kEpReferenceBlockDim, &config, false);
+    if (ret != kOk) {
+        return ret;
+    }
+    if (p.sharedExpertNum != 0) {
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // shared-expert ranks: not built yet
+    }
+    int64_t magic = 0;
+    ret = TileXRCommNextMagic(p.comm, &magic);
+    if (ret != kOk) {
+        return ret;
+    }
+    if (p.epochOut != nullptr) {
+        *p.epochOut = magic & 0xffffffffll;
+    }
+    return args->rankSize == 1 ? RunDispatchSingle(comm, p, true, magic) : RunDispatchMulti(comm, p, true, magic);
+}
+
+int CombineMvp(const EpCombineParams &p)
+{
+    int ret = TileXREpValidateBasicCombineParams(p);
+    if (ret != kOk) {
+        return ret;
+    }
+    EpComm *comm = nullptr;
+    TileXR::CommArgs *args = nullptr;
+    ret = CommArgsOf(p.comm, &comm, &args);
+    if (ret != kOk) {
+        return ret;
+    }
+    EpWindowConfig window {};
+    ret = TileXREpValidateCombineConfig(p, *args, &window, false);
+    if (ret != kOk) {
+        return ret;
+    }
+    if (p.dtype != TileXR::TILEXR_DATA_TYPE_FP16 && p.dtype != TileXR::TILEXR_DATA_TYPE_BFP16) {
+        // the reference's kernel leaves yOut untouched unless dtype is fp16 (tilexr_ep_combine_kernel.cpp:125);
+        // int8 rows cannot be summed, so that case is reported instead of silently skipped
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+    }
+    int64_t magic = 0;
+    ret = TileXRCommNextMagic(p.comm, &magic);
+    if (ret != kOk) {
+        return ret;
+    }
+    return args->rankSize == 1 ? RunCombineSingle(comm, p, false, magic) : RunCombineMulti(comm, p, false, magic);
+}
+
+int CombineMemory(const EpCombineParams &p)
+{
+    int ret = TileXREpValidateBasicCombineParams(p);
+    if (ret != kOk) {
+        return ret;
+    }
+    EpComm *comm = nullptr;
+    TileXR::CommArgs *args = nullptr;
+    ret = CommArgsOf(p.comm, &comm, &args);
+    if (ret != kOk) {
+        return ret;
+    }
+    if (p.extended) {
+        if (p.expertOutQuantMode != 0 && p.expertOutQuantMode != TILEXR_EP_QUANT_TOKEN_INT8 &&
+            p.expertOutQuantMode != TILEXR_EP_QUANT_FP8_BLOCK128) {
+            return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+        }
+        if ((p.expertOutQuantMode != 0 && (p.expertOutScales == nullptr || p.quantMode != 0)) ||
+            (p.tileFlags != nullptr && p.tileRows <= 0) || p.waitTimeoutUs < 0) {
+            return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+        }
+        if (args->rankSize != 1) {
+            return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+        }
+    }
+    EpMemoryCombineReferenceConfig config {};
+    ret = TileXREpValidateCombineMemoryConfig(p, *args, kEpReferenceBlockDim, &config, false);
+    if (ret != kOk) {
+        return ret;
+    }
+    if (p.sharedExpertNum != 0) {
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // shared-expert slots: not built yet
+    }
+    int64_t magic = 0;
+    ret = TileXRCommNextMagic(p.comm, &magic);
+    if (ret != kOk) {
+        return ret;
+    }
+    return args->rankSize == 1 ? RunCombineSingle(comm, p, true, magic) : RunCombineMulti(comm, p, true, magic);
+}
+
+} // namespace
+} // namespace TileXREp
+
+using namespace TileXREp;
+
+extern "C" {
+
+const char *TileXREpVersion(void)
+{
+    return "tilexr-ep gfx950 abi-1";
+}
+
+int TileXREpSetKernelTimingEvents(TileXRCommPtr comm, int kernel, void *startEvent, void *stopEvent)
+{
+    EpComm *c = LookupComm(comm);
+    if (c == nullptr) {
+        return TileXR::TILEXR_ERROR_NOT_INITIALIZED;
+    }
+    if (kernel < 0 || kernel > kKernelReduce || ((startEvent == nullptr) != (stopEvent == nullptr))) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    std::lock_guard<std::mutex> lock(c->mu);
+    c->timing[kernel][0] = static_cast<hipEvent_t>(startEvent);
+    c->timing[kernel][1] = static_cast<hipEvent_t>(stopEvent);
+    return TileXR::TILEXR_SUCCESS;
+}
+
+int TileXRMoeEpDispatchV2(void *x, int32_t *expertIds, void *scales, bool *xActiveMask, void *expertScales,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum, int64_t epWorldSize,
+    int64_t epRankId, int64_t tpWorldSize, int64_t tpRankId, int64_t expertShardType, int64_t sharedExpertNum,
+    int64_t sharedExpertRankNum, int64_t quantMode, int64_t globalBs, int64_t expertTokenNumsType, void *expandXOut,
+    void *dynamicScalesOut, int32_t *assistInfoForCombineOut, int64_t *expertTokenNumsOut, int32_t *epRecvCountsOut,
+    int32_t *tpRecvCountsOut, void *expandScalesOut, void *workspace, TileXR::TileXRDataType dtype,
+    aclrtStream stream)
+{
+    EpDispatchParams p {};
+    p.x = x;
+    p.expertIds = expertIds;
+    p.scales = scales;
+    p.xActiveMask = xActiveMask;
+    p.expertScales = expertScales;
+    p.comm = comm;
+    p.bs = bs;
+    p.h = h;
+    p.topK = topK;
+    p.moeExpertNum = moeExpertNum;
+    p.epWorldSize = epWorldSize;
+    p.epRankId = epRankId;
+    p.tpWorldSize = tpWorldSize;
+    p.tpRankId = tpRankId;
+    p.expertShardType = expertShardType;
+    p.sharedExpertNum = sharedExpertNum;
+    p.sharedExpertRankNum = sharedExpertRankNum;
+    p.quantMode = quantMode;
+    p.globalBs = globalBs;
+    p.expertTokenNumsType = expertTokenNumsType;
+    p.expandXOut = expandXOut;
+    p.dynamicScalesOut = dynamicScalesOut;
+    p.assistInfoForCombineOut = assistInfoForCombineOut;
+    p.expertTokenNumsOut = expertTokenNumsOut;
+    p.epRecvCountsOut = epRecvCountsOut;
+    p.tpRecvCountsOut = tpRecvCountsOut;
+    p.expandScalesOut = expandScalesOut;
+    p.workspace = workspace;
+    p.dtype = dtype;
+    p.stream = stream;
+    return DispatchMvp(p);
+}
+
+int TileXRMoeEpDispatch(void *x, int32_t *expertIds, TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK,
+    int64_t moeExpertNum, void *expandXOut, int64_t *expertTokenNumsOut, int32_t *epRecvCountsOut,
+    int32_t *assistInfoForCombineOut, TileXR::TileXRDataType dtype, aclrtStream stream)
+{
+    // reference: tilexr_ep_dispatch.cpp:85-94 -- V2 with everything optional off and counts (type 1)
+    return TileXRMoeEpDispatchV2(x, expertIds, nullptr, nullptr, nullptr, comm, bs, h, topK, moeExpertNum, 0, 0, 0, 0,
+        0, 0, 0, 0, 0, kEpExpertTokenNumsTypeCount, expandXOut, nullptr, assistInfoForCombineOut, expertTokenNumsOut,
+        epRecvCountsOut, nullptr, nullptr, nullptr, dtype, stream);
+}
+
+int TileXRMoeEpDispatchMemoryV2(void *x, int32_t *expertIds, void *scales, bool *xActiveMask,
+    int64_t activeMaskType, void *expertScales, TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK,
+    int64_t moeExpertNum, int64_t epWorldSize, int64_t epRankId, int64_t tpWorldSize, int64_t tpRankId,
+    int64_t expertShardType, int64_t sharedExpertNum, int64_t sharedExpertRankNum, int64_t quantMode,
+    int64_t globalBs, int64_t expertTokenNumsType, void *expandXOut, void *dynamicScalesOut,
+    int32_t *assistInfoForCombineOut, int64_t *expertTokenNumsOut, int32_t *sendCountsOut, int32_t *tpRecvCountsOut,
+    void *expandScalesOut, TileXR::TileXRDataType dtype, TileXR::TileXRDataType expandXOutDtype, aclrtStream stream)
+{
+    EpDispatchParams p {};
+    p.x = x;
+    p.expertIds = expertIds;
+    p.scales = scales;
+    p.xActiveMask = xActiveMask;
+    p.activeMaskType = activeMaskType;
+    p.expertScales = expertScales;
+    p.comm = comm;
+    p.bs = bs;
+    p.h = h;
+    p.topK = topK;
+    p.moeExpertNum = moeExpertNum;
+    p.epWorldSize = epWorldSize;
+    p.epRankId = epRankId;
+    p.tpWorldSize = tpWorldSize;
+    p.tpRankId = tpRankId;
+    p.expertShardType = expertShardType;
+    p.sharedExpertNum = sharedExpertNum;
+    p.sharedExpertRankNum = sharedExpertRankNum;
+    p.quantMode = quantMode;
+    p.globalBs = globalBs;
+    p.expertTokenNumsType = expertTokenNumsType;
+    p.expandXOut = expandXOut;
+    p.dynamicScalesOut = dynamicScalesOut;
+    p.assistInfoForCombineOut = assistInfoForCombineOut;
+    p.expertTokenNumsOut = expertTokenNumsOut;
+    p.epRecvCountsOut = sendCountsOut;
+    p.tpRecvCountsOut = tpRecvCountsOut;
+    p.expandScalesOut = expandScalesOut;
+    p.dtype = dtype;
+    p.expandXOutDtype = expandXOutDtype;
+    p.stream = stream;
+    return DispatchMemory(p);
+}
+
+int TileXRMoeEpDispatchMemory(void *x, int32_t *expertIds, TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK,
+    int64_t moeExpertNum, void *expandXOut, int64_t *expertTokenNumsOut, int32_t *sendCountsOut,
+    int32_t *assistInfoForCombineOut, TileXR::TileXRDataType dtype, aclrtStream stream)
+{
+    // reference: tilexr_ep_memory_dispatch.cpp:73-82 -- no mask, no quantisation, counts (type 1)
+    return TileXRMoeEpDispatchMemoryV2(x, expertIds, nullptr, nullptr, TILEXR_EP_ACTIVE_MASK_NONE, nullptr, comm, bs, h,
+        topK, moeExpertNum, 0, 0, 1, 0, 0, 0, 0, 0, 0, kEpExpertTokenNumsTypeCount, expandXOut, nullptr,
+        assistInfoForCombineOut, expertTokenNumsOut, sendCountsOut, nullptr, nullptr, dtype, dtype, stream);
+}
+
+int TileXRMoeEpDispatchMemoryEx(void *x, int32_t *expertIds, TileXRCommPtr comm, int64_t bs, int64_t h,
+    int64_t topK, int64_t moeExpertNum, const TileXREpDispatchExOptions *options, void *expandXOut,
+    void *dynamicScalesOut, int32_t *assistInfoForCombineOut, int64_t *expertTokenNumsOut, int32_t *sendCountsOut,
+    TileXR::TileXRDataType dtype, TileXR::TileXRDataType expandXOutDtype, aclrtStream stream)
+{
+    if (options == nullptr) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    EpDispatchParams p {};
+    p.x = x;
+    p.expertIds = expertIds;
+    p.xActiveMask = options->xActiveMask;
+    p.activeMaskType = options->activeMaskType;
+    p.comm = comm;
+    p.bs = bs;
+    p.h = h;
+    p.topK = topK;
+    p.moeExpertNum = moeExpertNum;
+    p.tpWorldSize = 1;
+    p.quantMode = options->quantMode;
+    p.expertTokenNumsType = options->expertTokenNumsType;
+    p.expandXOut = expandXOut;
+    p.dynamicScalesOut = dynamicScalesOut;
+    p.assistInfoForCombineOut = assistInfoForCombineOut;
+    p.expertTokenNumsOut = expertTokenNumsOut;
+    p.epRecvCountsOut = sendCountsOut;
+    p.dtype = dtype;
+    p.expandXOutDtype = expandXOutDtype;
+    p.stream = stream;
+    p.expertCapacity = options->expertCapacity;
+    p.rowIndexMapOut = options->rowIndexMapOut;
+    p.tileFlagsOut = options->tileFlagsOut;
+    p.tileRows = options->tileRows;
+    p.epochOut = options->epochOut;
+    p.metaReadyEvent = options->metaReadyEvent;
+    p.extended = true;
+    return DispatchMemory(p);
+}
+
+int TileXRMoeEpCombineV2(void *expertOut, int32_t *assistInfoForCombine, int32_t *epRecvCounts, TileXRCommPtr comm,
+    int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum, void *yOut, void *workspace,
+    TileXR::TileXRDataType dtype, aclrtStream stream)
+{
+    EpCombineParams p {};
+    p.expertOut = expertOut;
+    p.assistInfoForCombine = assistInfoForCombine;
+    p.epRecvCounts = epRecvCounts;
+    p.comm = comm;
+    p.bs = bs;
+    p.h = h;
+    p.topK = topK;
+    p.moeExpertNum = moeExpertNum;
+    p.yOut = yOut;
+    p.workspace = workspace;
+    p.dtype = dtype;
+    p.stream = stream;
+    return CombineMvp(p);
+}
+
+int TileXRMoeEpCombine(void *expertOut, int32_t *assistInfoForCombine, int32_t *epRecvCounts, TileXRCommPtr comm,
+    int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum, void *yOut, TileXR::TileXRDataType dtype,
+    aclrtStream stream)
+{
+    return TileXRMoeEpCombineV2(expertOut, assistInfoForCombine, epRecvCounts, comm, bs, h, topK, moeExpertNum, yOut,
+        nullptr, dtype, stream);
+}
+
+int TileXRMoeEpCombineMemoryV2(void *expertOut, int32_t *assistInfoForCombine, int32_t *sendCounts,
+    float *expertScales, bool *xActiveMask, int64_t activeMaskType, void *sharedExpertX, TileXRCommPtr comm,
+    int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum, int64_t epWorldSize, int64_t epRankId,
+    int64_t tpWorldSize, int64_t tpRankId, int64_t expertShardType, int64_t sharedExpertNum,
+    int64_t sharedExpertRankNum, int64_t quantMode, int64_t globalBs, void *yOut, TileXR::TileXRDataType dtype,
+    aclrtStream stream)
+{
+    EpCombineParams p {};
+    p.expertOut = expertOut;
+    p.assistInfoForCombine = assistInfoForCombine;
+    p.epRecvCounts = sendCounts;
+    p.expertScales = expertScales;
+    p.xActiveMask = xActiveMask;
+    p.activeMaskType = activeMaskType;
+    p.sharedExpertX = sharedExpertX;
+    p.comm = comm;
+    p.bs = bs;
+    p.h = h;
+    p.topK = topK;
+    p.moeExpertNum = moeExpertNum;
+    p.epWorldSize = epWorldSize;
+    p.epRankId = epRankId;
+    p.tpWorldSize = tpWorldSize;
+    p.tpRankId = tpRankId;
+    p.expertShardType = expertShardType;
+    p.sharedExpertNum = sharedExpertNum;
+    p.sharedExpertRankNum = sharedExpertRankNum;
+    p.quantMode = quantMode;
+    p.globalBs = globalBs;
+    p.yOut = yOut;
+    p.dtype = dtype;
+    p.stream = stream;
+    return CombineMemory(p);
+}
+
+int TileXRMoeEpCombineMemory(void *expertOut, int32_t *assistInfoForCombine, int32_t *epRecvCounts,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum, void *yOut,
+    TileXR::TileXRDataType dtype, aclrtStream stream)
+{
+    // reference: tilexr_ep_memory_combine.cpp:61-68
+    return TileXRMoeEpCombineMemoryV2(expertOut, assistInfoForCombine, epRecvCounts, nullptr, nullptr,
+        TILEXR_EP_ACTIVE_MASK_NONE, nullptr, comm, bs, h, topK, moeExpertNum, 0, 0, 1, 0, 0, 0, 0, 0, 0, yOut, dtype,
+        stream);
+}
+
+int TileXRMoeEpCombineMemoryEx(void *expertOut, int32_t *assistInfoForCombine, int32_t *sendCounts,
+    TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    const TileXREpCombineExOptions *options, void *yOut, TileXR::TileXRDataType dtype, aclrtStream stream)
+{
+    if (options == nullptr) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    EpCombineParams p {};
+    p.expertOut = expertOut;
+    p.assistInfoForCombine = assistInfoForCombine;
+    p.epRecvCounts = sendCounts;
+    p.expertScales = options->expertScales;
+    p.xActiveMask = options->xActiveMask;
+    p.activeMaskType = options->activeMaskType;
+    p.sharedExpertX = options->sharedExpertX;
+    p.comm = comm;
+    p.bs = bs;
+    p.h = h;
+    p.topK = topK;
+    p.moeExpertNum = moeExpertNum;
+    p.tpWorldSize = 1;
+    p.quantMode = options->commQuantMode;
+    p.yOut = yOut;
+    p.dtype = dtype;
+    p.stream = stream;
+    p.expertOutQuantMode = options->expertOutQuantMode;
+    p.expertOutScales = options->expertOutScales;
+    p.rowIndexMap = options->rowIndexMap;
+    p.tileFlags = options->tileFlags;
+    p.tileRows = options->tileRows;
+    p.flagEpoch = options->flagEpoch;
+    p.waitTimeoutUs = options->waitTimeoutUs;
+    p.deviceStatusOut = options->deviceStatusOut;
+    p.extended = true;
+    return CombineMemory(p);
+}
+
+}

@@ -1,0 +1,161 @@
+// Kernel launch interface between the host orchestration (api.cpp) and the HIP kernels (ep_kernels.hip).
+//
+// The data path of one dispatch is three launches on the caller's stream:
+//   count   per-chunk stable rank of every route within its key + per-chunk key histogram; the last workgroup
+//           to finish scans the histograms into per-chunk bases, per-key offsets and the count outputs
+//   place   destination row of every route, assist tuples, inverse row map, tile-flag reset
+//   scatter token rows read once and written to their topK destination rows (optionally quantised)
+// and of one combine two launches:
+//   invert  (skipped when the caller supplies the row map) row -> (token, k) inverse from the assist tuples
+//   reduce  per token: gather rows, dequantise, weighted fp32 sum in k order, one rounding to the output type
+// A "key" is what rows are grouped by: the expert (memory route), the destination rank (MVP route across logical
+// ranks) or nothing (MVP route on one rank: plain compaction of live routes).
+#ifndef TILEXR_AMD_EP_LAUNCH_H
+#define TILEXR_AMD_EP_LAUNCH_H
+
+#include <cstdint>
+
+#include <hip/hip_runtime_api.h>
+
+namespace TileXREp {
+
+constexpr int kChunkRoutes = 1024;      // routes handled by one counting workgroup
+constexpr int kMaxKeys = 2048;          // keys (experts) the counting kernel's LDS tables hold
+constexpr int kMaxTopK = 64;
+
+enum MaskMode : int {
+    kMaskNone = 0,
+    kMaskPerToken = 1,      // route live iff mask[token]           (MVP route, combine)
+    kMaskPerRoute = 2,      // route live iff mask[token, k]        (memory route, expert mask)
+    kMaskTokenPrefix = 3,   // route live iff token < sum(mask)     (memory route, token mask)
+};
+
+struct CountScratch {
+    uint32_t *ticket;       // 1 word, zero between launches
+    int32_t *localRank;     // [n]  rank of the route within (chunk, key); -1 when the route is not live
+    int32_t *chunkHist;     // [chunks, numKeys] in: counts; out: exclusive sum over earlier chunks
+    int32_t *chunkExpHist;  // [chunks, experts] only when keys are coarser than experts, else nullptr
+    int32_t *keyOffset;     // [numKeys + 1] exclusive sum of kept rows per key
+    int32_t *keyKept;       // [numKeys] rows kept per key (after capacity)
+    int32_t *expertTotal;   // [experts] live routes per expert (before capacity when keys are coarser)
+};
+
+struct RouteCountLaunch {
+    const int32_t *ids;
+    const uint8_t *mask;
+    int maskMode;
+    int64_t bs;
+    int64_t topK;
+    int64_t numExperts;
+    int64_t keyDiv;          // key = expert / keyDiv
+    int64_t numKeys;
+    int64_t capacity;        // rows kept per key, 0 = all
+    CountScratch scratch;
+    // outputs written by the last workgroup when non-null (single-rank fast path)
+    int32_t *sendCountsOut;      // [numKeys] inclusive sum of kept rows
+    int32_t *recvCountOut;       // [1] total kept rows
+    int64_t *expertTokenNumsOut; // [experts]
+    int tokenNumsType;
+    hipStream_t stream;
+};
+
+struct RoutePlaceLaunch {
+    const int32_t *ids;
+    int64_t bs;
+    int64_t topK;
+    int64_t keyDiv;
+    int64_t numKeys;
+    int64_t capacity;
+    CountScratch scratch;
+    int32_t srcRank;
+    int32_t expertIdBias;        // added to the id stored in the assist tuple (shared experts shift ids)
+    int32_t *rowOf;              // [n] out
+    int32_t *assist;             // [rows, 4] out
+    uint64_t *tileFlags;         // optional
+    int64_t numTiles;
+    uint64_t epoch;
+    hipStream_t stream;
+};
+
+struct ScatterLaunch {
+    const void *x;
+    const int32_t *rowOf;
+    int64_t bs;
+    int64_t h;
+    int64_t topK;
+    int quantMode;               // TileXREpQuantMode
+    bool inputBf16;              // decode of x when quantising
+    bool fp8E5m2;
+    const float *staticScale;
+    void *out;                   // rows of h*2 bytes (mode 0) or h bytes
+    void *scalesOut;             // fp32 [rows] (2), u8 [rows, mxScaleCount] (4), fp32 [rows, ceil(h/128)] (5)
+    uint64_t *tileFlags;         // optional: +1 (release, agent scope) on the row's tile after each row
+    int64_t tileRows;
+    hipStream_t stream;
+};
+
+struct InvertLaunch {
+    const int32_t *assist;
+    const int32_t *counts;       // device counts array
+    int64_t numCounts;
+    bool countsArePrefix;        // memory route: rows = counts[numCounts-1]; MVP: rows = sum(clamped counts)
+    int64_t maxRows;
+    int64_t maxCountPerEntry;    // MVP: entries outside [0, this] read as 0
+    int32_t rank;
+    int64_t bs;
+    int64_t topK;
+    uint64_t epoch;
+    uint64_t *inverse;           // [bs*topK] (epoch << 32) | row
+    hipStream_t stream;
+};
+
+enum ReduceKind : int {
+    kReduceFp32 = 0,             // memory route: fp32 accumulate in k order, one rounding
+    kReducePerAdd = 1,           // MVP route: accumulator rounded to the element type after every add, row order
+};
+
+struct ReduceLaunch {
+    const void *expertOut;
+    int64_t rowBytes;
+    const uint64_t *inverseTagged;   // either this (with epoch) ...
+    uint64_t epoch;
+    const int32_t *rowIndexMap;      // ... or a plain row map (-1 = none)
+    const float *expertScales;       // optional [bs, topK]
+    const uint8_t *tokenMask;        // optional [bs]
+    const void *sharedExpertX;       // optional [bs, h]
+    int reduceKind;
+    int commQuant;                   // 0, 3, 4
+    int inQuant;                     // 0, 2, 5
+    const float *inScales;
+    bool bf16;
+    int64_t bs;
+    int64_t h;
+    int64_t topK;
+    void *y;
+    const uint64_t *tileFlags;       // optional
+    int64_t tileRows;
+    const int32_t *totalRowsPtr;     // device word holding the number of valid rows (for the last tile's size)
+    uint64_t flagEpoch;
+    int64_t waitTimeoutTicks;        // in wall_clock64 ticks
+    int32_t *deviceStatus;
+    int numComputeUnits;
+    hipStream_t stream;
+};
+
+hipError_t LaunchRouteCount(const RouteCountLaunch &l);
+hipError_t LaunchRoutePlace(const RoutePlaceLaunch &l);
+hipError_t LaunchScatter(const ScatterLaunch &l);
+hipError_t LaunchInvert(const InvertLaunch &l);
+hipError_t LaunchReduce(const ReduceLaunch &l);
+
+// Bytes of CountScratch arrays for a problem (used by the host to carve one allocation).
+struct CountScratchLayout {
+    int64_t chunks;
+    int64_t localRankOff, chunkHistOff, chunkExpHistOff, keyOffsetOff, keyKeptOff, expertTotalOff, rowOfOff;
+    int64_t totalBytes;
+};
+CountScratchLayout PlanCountScratch(int64_t routes, int64_t numKeys, int64_t numExperts, bool expertHist);
+
+} // namespace TileXREp
+
+#endif // TILEXR_AMD_EP_LAUNCH_H

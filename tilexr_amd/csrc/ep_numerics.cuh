@@ -1,0 +1,167 @@
+// Device-side element conversions shared by the scatter and reduce kernels (gfx950, wave64).
+//
+// Every routine is written so that its result is a pure function of the input bits: separate multiplies and adds
+// (the build uses -ffp-contract=off and the explicit *_rn intrinsics), software fp8 encoders instead of the
+// hardware converts, and saturation made explicit.  That is what lets the parity tests demand bit equality.
+//   int8 rounding      reference: src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:183-193
+//   MXFP8 / fp8 codec  reference: tests/ep/demo/mxfp8_golden.h:45-152
+//   output casts       reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:595 (CAST_RINT, saturating)
+#ifndef TILEXR_AMD_EP_NUMERICS_CUH
+#define TILEXR_AMD_EP_NUMERICS_CUH
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+
+namespace TileXREp {
+
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
+
+template <bool BF16>
+__device__ __forceinline__ float Decode16(uint32_t bits16)
+{
+    if (BF16) {
+        return __uint_as_float(bits16 << 16);
+    }
+    return __half2float(__ushort_as_half(static_cast<unsigned short>(bits16)));
+}
+
+__device__ __forceinline__ uint32_t FloatToBf16Rne(float v)
+{
+    uint32_t u = __float_as_uint(v);
+    if ((u & 0x7fffffffu) > 0x7f800000u) {
+        return (u >> 16) | 0x0040u;
+    }
+    u += 0x7fffu + ((u >> 16) & 1u);
+    return u >> 16;
+}
+
+// IEEE round-to-nearest-even; overflow becomes infinity.
+__device__ __forceinline__ uint32_t FloatToHalfRne(float v)
+{
+    return __half_as_ushort(__float2half_rn(v));
+}
+
+// Same rounding, but magnitudes that would round past 65504 stay at +-65504.
+__device__ __forceinline__ uint32_t FloatToHalfRneSat(float v)
+{
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t a = u & 0x7fffffffu;
+    if (a >= 0x477ff000u && a <= 0x7f800000u) {
+        return ((u >> 16) & 0x8000u) | 0x7bffu;
+    }
+    return FloatToHalfRne(v);
+}
+
+template <bool BF16>
+__device__ __forceinline__ uint32_t Encode16Sat(float v)
+{
+    return BF16 ? FloatToBf16Rne(v) : FloatToHalfRneSat(v);
+}
+
+// Round an fp32 value to the 16-bit element type and return it as fp32 again (IEEE, non-saturating).
+template <bool BF16>
+__device__ __forceinline__ float RoundTo16(float v)
+{
+    return BF16 ? __uint_as_float(FloatToBf16Rne(v) << 16) : __half2float(__float2half_rn(v));
+}
+
+// add +-0.5, truncate toward zero, clamp to [-128, 127]
+__device__ __forceinline__ int ClampInt8(float v)
+{
+    float r = v >= 0.0f ? __fadd_rn(v, 0.5f) : __fadd_rn(v, -0.5f);
+    r = fminf(fmaxf(r, -129.0f), 128.0f);
+    int i = static_cast<int>(r);
+    i = i > 127 ? 127 : i;
+    i = i < -128 ? -128 : i;
+    return i;
+}
+
+// Saturating round-to-nearest-even fp32 -> fp8 code (OCP e4m3fn / e5m2), by bit manipulation.
+template <bool E5M2>
+__device__ __forceinline__ uint32_t Fp8Encode(float v)
+{
+    constexpr int kMantBits = E5M2 ? 2 : 3;
+    constexpr int kBias = E5M2 ? 15 : 7;
+    constexpr int kMinNormalExp = 1 - kBias;
+    constexpr uint32_t kMaxCode = E5M2 ? 0x7bu : 0x7eu;
+    const uint32_t u = __float_as_uint(v);
+    const uint32_t sign = (u >> 24) & 0x80u;
+    const uint32_t a = u & 0x7fffffffu;
+    if (a > 0x7f800000u) {
+        return sign | 0x7fu;
+    }
+    const int e = static_cast<int>(a >> 23) - 127;
+    const uint32_t mant = a & 0x7fffffu;
+    uint32_t code;
+    if (e < kMinNormalExp) {
+        const int shift = 23 - e + kMinNormalExp - kMantBits;   // value / subnormal step = full >> shift
+        if (shift > 24) {
+            code = 0;
+        } else {
+            const uint32_t full = mant | 0x800000u;
+            const uint32_t kept = full >> shift;
+            const uint32_t rem = full & ((1u << shift) - 1u);
+            const uint32_t half = 1u << (shift - 1);
+            code = kept + ((rem > half || (rem == half && (kept & 1u))) ? 1u : 0u);
+        }
+    } else if (e > 20) {
+        code = kMaxCode;
+    } else {
+        const uint32_t kept = mant >> (23 - kMantBits);
+        const uint32_t rem = mant & ((1u << (23 - kMantBits)) - 1u);
+        const uint32_t half = 1u << (22 - kMantBits);
+        code = (static_cast<uint32_t>(e + kBias) << kMantBits) + kept +
+            ((rem > half || (rem == half && (kept & 1u))) ? 1u : 0u);
+        code = code > kMaxCode ? kMaxCode : code;
+    }
+    return sign | code;
+}
+
+template <bool E5M2>
+__device__ __forceinline__ float Fp8Decode(uint32_t code)
+{
+    constexpr int kMantBits = E5M2 ? 2 : 3;
+    constexpr int kBias = E5M2 ? 15 : 7;
+    constexpr uint32_t kExpMask = E5M2 ? 31u : 15u;
+    constexpr uint32_t kMantMask = (1u << kMantBits) - 1u;
+    const uint32_t sign = (code & 0x80u) << 24;
+    const uint32_t exp = (code >> kMantBits) & kExpMask;
+    const uint32_t man = code & kMantMask;
+    if (exp == 0) {
+        const float mag = static_cast<float>(man) * __uint_as_float(static_cast<uint32_t>(127 + 1 - kBias - kMantBits) << 23);
+        return __uint_as_float(__float_as_uint(mag) | sign);
+    }
+    if (E5M2 && exp == kExpMask) {
+        return __uint_as_float(sign | 0x7f800000u | (man << 21));
+    }
+    if (!E5M2 && exp == kExpMask && man == kMantMask) {
+        return __uint_as_float(sign | 0x7fc00000u);
+    }
+    return __uint_as_float(sign | ((exp + 127u - kBias) << 23) | (man << (23 - kMantBits)));
+}
+
+// Shared exponent of an MXFP8 block: clamp(floor(log2 amax) - emax, -127, 127); all-zero block -> -127.
+template <bool E5M2>
+__device__ __forceinline__ int MxSharedExponent(float amax)
+{
+    constexpr int kEmax = E5M2 ? 15 : 8;
+    const uint32_t a = __float_as_uint(amax) & 0x7fffffffu;
+    if (a == 0) {
+        return -127;
+    }
+    int se = static_cast<int>(a >> 23) - 127 - kEmax;    // denormal amax gives < -127 and is clamped below
+    se = se < -127 ? -127 : se;
+    se = se > 127 ? 127 : se;
+    return se;
+}
+
+// 2^e for e in [-127, 127] (2^-127 is a denormal fp32 and is produced exactly)
+__device__ __forceinline__ float Exp2Int(int e)
+{
+    return e >= -126 ? __uint_as_float(static_cast<uint32_t>(e + 127) << 23) : __uint_as_float(0x00400000u);
+}
+
+} // namespace TileXREp
+
+#endif // TILEXR_AMD_EP_NUMERICS_CUH
