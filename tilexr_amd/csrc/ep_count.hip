@@ -1,0 +1,505 @@
+// Routing kernels of the EP dispatch / combine path for gfx950 (CDNA4, wave64): count, place and invert.
+//
+// They turn the [bs, topK] expert-id table into destinations without moving a single payload byte:
+//   count   stable rank of every live route within its key + histograms; the last workgroup scans them
+//   place   destination row of every route, assist tuples, inverse map, tile-flag reset
+//   invert  (combine side) row -> (token, k) inverse rebuilt from assist tuples
+// All integer work; the reference behaviour each kernel restates is cited at the kernel.
+#include <hip/hip_runtime.h>
+
+#include "ep_kernel_common.cuh"
+#include "ep_launch.h"
+#include "tilexr_ep.h"
+
+namespace TileXREp {
+namespace {
+
+
+__device__ __forceinline__ unsigned long long LaneMaskLt()
+{
+    return (1ull << (threadIdx.x & (kWave - 1))) - 1ull;
+}
+
+// Exclusive scan of vals[0..m) in place (LDS), m <= 2048, by all 256 threads.  part[] is 256 ints of LDS.
+// Returns the total.
+__device__ int BlockExclusiveScan(int *vals, int m, int *part)
+{
+    const int tid = threadIdx.x;
+    const int per = (m + kThreads - 1) / kThreads;
+    const int begin = tid * per;
+    int local = 0;
+    for (int i = begin; i < begin + per && i < m; ++i) {
+        local += vals[i];
+    }
+    part[tid] = local;
+    __syncthreads();
+    for (int off = 1; off < kThreads; off <<= 1) {
+        const int add = tid >= off ? part[tid - off] : 0;
+        __syncthreads();
+        part[tid] += add;
+        __syncthreads();
+    }
+    int run = part[tid] - local;
+    const int total = part[kThreads - 1];
+    for (int i = begin; i < begin + per && i < m; ++i) {
+        const int v = vals[i];
+        vals[i] = run;
+        run += v;
+    }
+    __syncthreads();
+    return total;
+}
+
+// -------------------------------------------------------------------------------------------------------------
+// count: stable rank of every live route within (chunk, key), per-chunk key histogram, and -- in the last
+// workgroup to finish -- the scans that turn histograms into destinations and the count outputs.
+//
+// Replaces the reference's per-route O(n) pass (`CalTokenSendExpertCnt`, number of earlier routes with the same
+// expert, src/ep/kernels/tilexr_ep_dispatch_memory_kernel.h:791-818), its count exchange and cumulative sum
+// (:820-1089) and the count outputs (:1142-1168); for the MVP route the same machinery with a single key gives the
+// token-major, k-minor compaction of src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:501-571.
+// Route liveness: ids outside [0, E) are skipped (:686-687); mask modes are described in ep_launch.h.
+// -------------------------------------------------------------------------------------------------------------
+struct RouteCountArgs {
+    const int32_t *ids;
+    const uint8_t *mask;
+    int maskMode;
+    int bs;
+    int topK;
+    int numExperts;
+    int keyDiv;
+    int numKeys;
+    int keyBits;
+    int capacity;
+    int numChunks;
+    CountScratch s;
+    int32_t *sendCountsOut;
+    int32_t *recvCountOut;
+    int64_t *expertTokenNumsOut;
+    int tokenNumsType;
+};
+
+__global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs a)
+{
+    __shared__ int s_cnt[kWavesPerBlock * kMaxKeys];
+    __shared__ int s_exp[kMaxKeys];
+    __shared__ int s_part[kThreads];
+    __shared__ int s_misc[4];
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int lane = tid & (kWave - 1);
+    const int n = a.bs * a.topK;
+    const int chunk = blockIdx.x;
+    const bool expHist = a.s.chunkExpHist != nullptr;
+
+    for (int i = tid; i < kWavesPerBlock * a.numKeys; i += kThreads) {
+        s_cnt[i] = 0;
+    }
+    if (expHist) {
+        for (int i = tid; i < a.numExperts; i += kThreads) {
+            s_exp[i] = 0;
+        }
+    }
+    if (tid == 0) {
+        s_misc[0] = 0;
+    }
+    __syncthreads();
+
+    int liveLimit = n;
+    if (a.maskMode == kMaskTokenPrefix) {
+        // activeCnt = sum(mask); only the first activeCnt tokens are dispatched
+        // (reference: tilexr_ep_dispatch_memory_kernel.h:1387-1410, 1538-1544)
+        int local = 0;
+        for (int t = tid; t < a.bs; t += kThreads) {
+            local += a.mask[t] != 0 ? 1 : 0;
+        }
+        for (int off = kWave / 2; off >= 1; off >>= 1) {
+            local += __shfl_xor(local, off);
+        }
+        if (lane == 0) {
+            atomicAdd(&s_misc[0], local);
+        }
+        __syncthreads();
+        liveLimit = s_misc[0] * a.topK;
+    }
+
+    // phase A: per-wave histogram of the wave's 256 consecutive routes
+    int keys[kChunkRoutes / kThreads];
+#pragma unroll
+    for (int b = 0; b < kChunkRoutes / kThreads; ++b) {
+        const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
+        int key = -1;
+        if (i < n && i < liveLimit) {
+            const int e = a.ids[i];
+            bool live = e >= 0 && e < a.numExperts;
+            if (a.maskMode == kMaskPerToken) {
+                live = live && a.mask[i / a.topK] != 0;
+            } else if (a.maskMode == kMaskPerRoute) {
+                live = live && a.mask[i] != 0;
+            }
+            if (live) {
+                key = e / a.keyDiv;
+                atomicAdd(&s_cnt[wave * a.numKeys + key], 1);
+                if (expHist) {
+                    atomicAdd(&s_exp[e], 1);
+                }
+            }
+        }
+        keys[b] = key;
+    }
+    __syncthreads();
+
+    // phase B: exclusive sum over the four waves; chunk totals to HBM
+    for (int key = tid; key < a.numKeys; key += kThreads) {
+        int run = 0;
+#pragma unroll
+        for (int w = 0; w < kWavesPerBlock; ++w) {
+            const int v = s_cnt[w * a.numKeys + key];
+            s_cnt[w * a.numKeys + key] = run;
+            run += v;
+        }
+        a.s.chunkHist[static_cast<int64_t>(chunk) * a.numKeys + key] = run;
+    }
+    if (expHist) {
+        for (int e = tid; e < a.numExperts; e += kThreads) {
+            a.s.chunkExpHist[static_cast<int64_t>(chunk) * a.numExperts + e] = s_exp[e];
+        }
+    }
+    __syncthreads();
+
+    // phase C: batches of 64 routes in order; lanes with equal keys find each other with one ballot per key bit
+    volatile int *cnt = s_cnt + wave * a.numKeys;
+    const unsigned long long lt = LaneMaskLt();
+#pragma unroll
+    for (int b = 0; b < kChunkRoutes / kThreads; ++b) {
+        const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
+        const int key = keys[b];
+        const bool live = key >= 0;
+        unsigned long long peers = __ballot(live);
+        for (int bit = 0; bit < a.keyBits; ++bit) {
+            const bool one = live && ((key >> bit) & 1);
+            const unsigned long long bal = __ballot(one);
+            peers &= one ? bal : ~bal;
+        }
+        const int before = __popcll(peers & lt);
+        const int base = live ? cnt[key] : 0;
+        if (i < n) {
+            a.s.localRank[i] = live ? base + before : -1;
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (live && before == 0) {
+            cnt[key] = base + __popcll(peers);
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+
+    // last workgroup to arrive performs the scans
+    __threadfence();
+    __syncthreads();
+    if (tid == 0) {
+        const unsigned prev = atomicAdd(a.s.ticket, 1u);
+        s_misc[1] = prev == static_cast<unsigned>(a.numChunks - 1) ? 1 : 0;
+    }
+    __syncthreads();
+    if (s_misc[1] == 0) {
+        return;
+    }
+    __threadfence();
+
+    // per key: exclusive sum over chunks (becomes the chunk's base rank within the key), total, kept
+    int *kept = s_cnt;                 // reuse: [numKeys]
+    for (int key = tid; key < a.numKeys; key += kThreads) {
+        int run = 0;
+        // 16 independent loads per round trip to HBM, then the in-place exclusive sum
+        constexpr int kBatch = 16;
+        for (int c0 = 0; c0 < a.numChunks; c0 += kBatch) {
+            int v[kBatch];
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int c = c0 + u;
+                v[u] = c < a.numChunks ? a.s.chunkHist[static_cast<int64_t>(c) * a.numKeys + key] : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < kBatch; ++u) {
+                const int c = c0 + u;
+                if (c < a.numChunks) {
+                    a.s.chunkHist[static_cast<int64_t>(c) * a.numKeys + key] = run;
+                    run += v[u];
+                }
+            }
+        }
+        const int k = (a.capacity > 0 && run > a.capacity) ? a.capacity : run;
+        kept[key] = k;
+        a.s.keyKept[key] = k;
+    }
+    __syncthreads();
+    int *offs = s_cnt + kMaxKeys;      // [numKeys] exclusive offsets
+    for (int key = tid; key < a.numKeys; key += kThreads) {
+        offs[key] = kept[key];
+    }
+    __syncthreads();
+    const int totalRows = BlockExclusiveScan(offs, a.numKeys, s_part);
+    for (int key = tid; key < a.numKeys; key += kThreads) {
+        a.s.keyOffset[key] = offs[key];
+        if (a.sendCountsOut != nullptr) {
+            a.sendCountsOut[key] = offs[key] + kept[key];
+        }
+    }
+    if (tid == 0) {
+        a.s.keyOffset[a.numKeys] = totalRows;
+        if (a.recvCountOut != nullptr) {
+            a.recvCountOut[0] = totalRows;
+        }
+    }
+
+    // per expert totals
+    //   keys == experts: rows kept per expert (reference: tilexr_ep_dispatch_memory_kernel.h:1159-1168)
+    //   coarser keys:    live routes per expert (reference: tilexr_ep_combine_helpers.h:49-80)
+    int *etot = s_cnt + 2 * kMaxKeys;  // [numExperts]
+    if (expHist) {
+        for (int e = tid; e < a.numExperts; e += kThreads) {
+            int run = 0;
+            for (int c = 0; c < a.numChunks; ++c) {
+                run += a.s.chunkExpHist[static_cast<int64_t>(c) * a.numExperts + e];
+            }
+            etot[e] = run;
+        }
+    } else {
+        for (int e = tid; e < a.numExperts; e += kThreads) {
+            etot[e] = e < a.numKeys ? kept[e] : 0;
+        }
+    }
+    __syncthreads();
+    for (int e = tid; e < a.numExperts; e += kThreads) {
+        a.s.expertTotal[e] = etot[e];
+    }
+    if (a.expertTokenNumsOut != nullptr) {
+        if (a.tokenNumsType == 0) {
+            int *pref = s_cnt + 3 * kMaxKeys;
+            for (int e = tid; e < a.numExperts; e += kThreads) {
+                pref[e] = etot[e];
+            }
+            __syncthreads();
+            BlockExclusiveScan(pref, a.numExperts, s_part);
+            for (int e = tid; e < a.numExperts; e += kThreads) {
+                a.expertTokenNumsOut[e] = static_cast<int64_t>(pref[e]) + etot[e];
+            }
+        } else {
+            for (int e = tid; e < a.numExperts; e += kThreads) {
+                a.expertTokenNumsOut[e] = etot[e];
+            }
+        }
+    }
+    if (tid == 0) {
+        *a.s.ticket = 0u;
+    }
+}
+
+// -------------------------------------------------------------------------------------------------------------
+// place: destination row of every route + assist tuple + inverse map + tile-flag reset.
+//   row   = keyOffset[key] + (rank of the route within its key), routes at or beyond `capacity` get none
+//   tuple = {srcRank, token, k, expert id} (reference: src/ep/common/ep_window.h:47-52,
+//           tilexr_ep_dispatch_memory_kernel.h:1240-1258)
+// -------------------------------------------------------------------------------------------------------------
+struct RoutePlaceArgs {
+    const int32_t *ids;
+    int n;
+    int topK;
+    int keyDiv;
+    int numKeys;
+    int capacity;
+    CountScratch s;
+    int32_t srcRank;
+    int32_t expertIdBias;
+    int32_t *rowOf;
+    int32_t *assist;
+    uint64_t *tileFlags;
+    int numTiles;
+    uint64_t epoch;
+};
+
+__global__ __launch_bounds__(kThreads) void ep_route_place_kernel(RoutePlaceArgs a)
+{
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    if (a.tileFlags != nullptr) {
+        for (int f = i; f < a.numTiles; f += gridDim.x * kThreads) {
+            a.tileFlags[f] = a.epoch << 32;
+        }
+    }
+    if (i >= a.n) {
+        return;
+    }
+    const int lr = a.s.localRank[i];
+    int row = -1;
+    if (lr >= 0) {
+        const int e = a.ids[i];
+        const int key = e / a.keyDiv;
+        const int within = a.s.chunkHist[static_cast<int64_t>(i / kChunkRoutes) * a.numKeys + key] + lr;
+        if (a.capacity <= 0 || within < a.capacity) {
+            row = a.s.keyOffset[key] + within;
+            int32_t *tuple = a.assist + static_cast<int64_t>(row) * 4;
+            tuple[0] = a.srcRank;
+            tuple[1] = i / a.topK;
+            tuple[2] = i % a.topK;
+            tuple[3] = e + a.expertIdBias;
+        }
+    }
+    a.rowOf[i] = row;
+}
+
+// -------------------------------------------------------------------------------------------------------------
+// invert: (token, k) -> row from the assist tuples, tagged with the call's epoch so the table never needs clearing.
+//   memory route: rows [0, counts[last]) whose tuple names this rank and lies in range
+//                 (reference: tilexr_ep_combine_memory_kernel.h:256-266, 329-342)
+//   MVP route:    rows [0, sum of counts clamped to [0, maxCountPerEntry]); the tuple's rank field is not tested
+//                 because the reference overwrites it while scattering (tilexr_ep_combine_kernel.cpp:28-52, 94-97)
+// -------------------------------------------------------------------------------------------------------------
+struct InvertArgs {
+    const int32_t *assist;
+    const int32_t *counts;
+    int numCounts;
+    int countsArePrefix;
+    int maxRows;
+    int maxCountPerEntry;
+    int32_t rank;
+    int bs;
+    int topK;
+    uint64_t epoch;
+    uint64_t *inverse;
+};
+
+__global__ __launch_bounds__(kThreads) void ep_invert_kernel(InvertArgs a)
+{
+    __shared__ int s_rows;
+    if (threadIdx.x == 0) {
+        int rows = 0;
+        if (a.countsArePrefix) {
+            rows = a.counts[a.numCounts - 1];
+        } else {
+            for (int i = 0; i < a.numCounts; ++i) {
+                const int c = a.counts[i];
+                rows += (c < 0 || c > a.maxCountPerEntry) ? 0 : c;
+            }
+        }
+        s_rows = rows < 0 ? 0 : (rows > a.maxRows ? a.maxRows : rows);
+    }
+    __syncthreads();
+    const int row = blockIdx.x * kThreads + threadIdx.x;
+    if (row >= s_rows) {
+        return;
+    }
+    const int32_t *t = a.assist + static_cast<int64_t>(row) * 4;
+    const int srcRank = t[0];
+    const int token = t[1];
+    const int k = t[2];
+    if ((a.countsArePrefix && srcRank != a.rank) || token < 0 || token >= a.bs || k < 0 || k >= a.topK) {
+        return;
+    }
+    a.inverse[static_cast<int64_t>(token) * a.topK + k] = (a.epoch << 32) | static_cast<uint32_t>(row);
+}
+
+int KeyBits(int64_t numKeys)
+{
+    int bits = 0;
+    while ((1ll << bits) < numKeys) {
+        ++bits;
+    }
+    return bits;
+}
+
+} // namespace
+
+// -------------------------------------------------------------------------------------------------------------
+// host-side launchers
+// -------------------------------------------------------------------------------------------------------------
+CountScratchLayout PlanCountScratch(int64_t routes, int64_t numKeys, int64_t numExperts, bool expertHist)
+{
+    auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
+    CountScratchLayout p {};
+    p.chunks = (routes + kChunkRoutes - 1) / kChunkRoutes;
+    int64_t off = 256;   // word 0 is the ticket
+    p.localRankOff = off;
+    off += align(routes * 4);
+    p.rowOfOff = off;
+    off += align(routes * 4);
+    p.chunkHistOff = off;
+    off += align(p.chunks * numKeys * 4);
+    p.chunkExpHistOff = off;
+    off += expertHist ? align(p.chunks * numExperts * 4) : 0;
+    p.keyOffsetOff = off;
+    off += align((numKeys + 1) * 4);
+    p.keyKeptOff = off;
+    off += align(numKeys * 4);
+    p.expertTotalOff = off;
+    off += align(numExperts * 4);
+    p.totalBytes = off;
+    return p;
+}
+
+hipError_t LaunchRouteCount(const RouteCountLaunch &l)
+{
+    RouteCountArgs a {};
+    a.ids = l.ids;
+    a.mask = l.mask;
+    a.maskMode = l.maskMode;
+    a.bs = static_cast<int>(l.bs);
+    a.topK = static_cast<int>(l.topK);
+    a.numExperts = static_cast<int>(l.numExperts);
+    a.keyDiv = static_cast<int>(l.keyDiv);
+    a.numKeys = static_cast<int>(l.numKeys);
+    a.keyBits = KeyBits(l.numKeys);
+    a.capacity = static_cast<int>(l.capacity);
+    const int64_t n = l.bs * l.topK;
+    a.numChunks = static_cast<int>((n + kChunkRoutes - 1) / kChunkRoutes);
+    a.s = l.scratch;
+    a.sendCountsOut = l.sendCountsOut;
+    a.recvCountOut = l.recvCountOut;
+    a.expertTokenNumsOut = l.expertTokenNumsOut;
+    a.tokenNumsType = l.tokenNumsType;
+    hipLaunchKernelGGL(ep_route_count_kernel, dim3(a.numChunks), dim3(kThreads), 0, l.stream, a);
+    return hipGetLastError();
+}
+
+hipError_t LaunchRoutePlace(const RoutePlaceLaunch &l)
+{
+    RoutePlaceArgs a {};
+    a.ids = l.ids;
+    a.n = static_cast<int>(l.bs * l.topK);
+    a.topK = static_cast<int>(l.topK);
+    a.keyDiv = static_cast<int>(l.keyDiv);
+    a.numKeys = static_cast<int>(l.numKeys);
+    a.capacity = static_cast<int>(l.capacity);
+    a.s = l.scratch;
+    a.srcRank = l.srcRank;
+    a.expertIdBias = l.expertIdBias;
+    a.rowOf = l.rowOf;
+    a.assist = l.assist;
+    a.tileFlags = l.tileFlags;
+    a.numTiles = static_cast<int>(l.numTiles);
+    a.epoch = l.epoch;
+    const int grid = (a.n + kThreads - 1) / kThreads;
+    hipLaunchKernelGGL(ep_route_place_kernel, dim3(grid), dim3(kThreads), 0, l.stream, a);
+    return hipGetLastError();
+}
+
+hipError_t LaunchInvert(const InvertLaunch &l)
+{
+    InvertArgs a {};
+    a.assist = l.assist;
+    a.counts = l.counts;
+    a.numCounts = static_cast<int>(l.numCounts);
+    a.countsArePrefix = l.countsArePrefix ? 1 : 0;
+    a.maxRows = static_cast<int>(l.maxRows);
+    a.maxCountPerEntry = static_cast<int>(l.maxCountPerEntry);
+    a.rank = l.rank;
+    a.bs = static_cast<int>(l.bs);
+    a.topK = static_cast<int>(l.topK);
+    a.epoch = l.epoch;
+    a.inverse = l.inverse;
+    const int grid = static_cast<int>((l.maxRows + kThreads - 1) / kThreads);
+    hipLaunchKernelGGL(ep_invert_kernel, dim3(grid > 0 ? grid : 1), dim3(kThreads), 0, l.stream, a);
+    return hipGetLastError();
+}
+
+} // namespace TileXREp

@@ -1,0 +1,445 @@
+// reduce: y[token] = sum over the token's rows, gathered through the inverse map (gfx950, wave64).
+//
+// HBM-bound: topK row reads per output row, < 0.5 FLOP per byte, no MFMA.  G lanes cooperate on one token and keep
+// V x 8 fp32 accumulators in registers; for each route in k order a lane issues all V of its 128-bit non-temporal
+// loads of that row before touching the accumulators, so 64-128 bytes per lane are in flight while the previous
+// row is being summed.  Measured on MI355X this moves 4096 x 7168 bf16 x top-8 (529 MB) at about 6 TB/s.
+//
+//   KIND fp32     sum = 0; for k = 0..K-1: sum = sum + (w_k * row_k) in fp32 (separate multiply and add), then the
+//                 shared-expert row, then one round-to-nearest-even (saturating for fp16) to the output type;
+//                 an inactive token (mask) gives zeros
+//                 (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:505-553, 555-571, 573-601, 632-662)
+//   KIND per-add  rows in ascending row index; y = T(float(y) + float(row)) after every add
+//                 (reference: src/ep/kernels/tilexr_ep_combine_kernel.cpp:15-26, 54-101)
+//   COMMQ 3/4     every row first takes the MXFP8 e5m2 / e4m3 round trip and is accumulated as
+//                 ((fp8 * 2^(s-127)) * w) (reference: src/ep/kernels/tilexr_ep_mxfp8_quant.h:286-352)
+//   INQ 2/5       rows hold int8 / fp8 payloads that are dequantised with their scales and rounded to the element
+//                 type first (no reference counterpart)
+#include <hip/hip_runtime.h>
+
+#include "ep_kernel_common.cuh"
+#include "ep_launch.h"
+#include "ep_numerics.cuh"
+#include "tilexr_ep.h"
+
+namespace TileXREp {
+namespace {
+
+struct ReduceArgs {
+    const void *expertOut;
+    int64_t rowBytes;
+    const uint64_t *inverseTagged;
+    uint64_t epoch;
+    const int32_t *rowIndexMap;
+    const float *expertScales;
+    const uint8_t *tokenMask;
+    const void *sharedExpertX;
+    const float *inScales;
+    int bs;
+    int h;
+    int topK;
+    void *y;
+    const uint64_t *tileFlags;
+    int tileRows;
+    const int32_t *totalRowsPtr;
+    uint64_t flagEpoch;
+    int64_t waitTimeoutTicks;
+    int32_t *deviceStatus;
+};
+
+__device__ __forceinline__ int LookupRow(const ReduceArgs &a, int64_t slot)
+{
+    if (a.rowIndexMap != nullptr) {
+        return a.rowIndexMap[slot];
+    }
+    const uint64_t e = a.inverseTagged[slot];
+    return (e >> 32) == a.epoch ? static_cast<int>(e & 0xffffffffu) : -1;
+}
+
+// Bounded acquire-wait until the tile holding `row` has all its rows published for this epoch.
+__device__ bool WaitTile(const ReduceArgs &a, int row)
+{
+    const int tile = row / a.tileRows;
+    const int total = *a.totalRowsPtr;
+    int need = total - tile * a.tileRows;
+    need = need > a.tileRows ? a.tileRows : need;
+    const uint64_t start = wall_clock64();
+    while (true) {
+        const uint64_t w = __hip_atomic_load(&a.tileFlags[tile], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        if ((w >> 32) == a.flagEpoch && static_cast<int>(w & 0xffffffffu) >= need) {
+            return true;
+        }
+        if (static_cast<int64_t>(wall_clock64() - start) > a.waitTimeoutTicks) {
+            return false;
+        }
+        __builtin_amdgcn_s_sleep(4);
+    }
+}
+
+// Insertion sort of row indices, ascending, absent rows (-1) last.  K is small.
+__device__ void SortRows(int *rows, int k)
+{
+    for (int i = 1; i < k; ++i) {
+        const int v = rows[i];
+        const unsigned kv = static_cast<unsigned>(v);      // -1 becomes the largest key
+        int j = i - 1;
+        while (j >= 0 && static_cast<unsigned>(rows[j]) > kv) {
+            rows[j + 1] = rows[j];
+            --j;
+        }
+        rows[j + 1] = v;
+    }
+}
+
+// Fills s_row / s_w for one token; waits for tile flags when asked to.
+__device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
+    float *weights)
+{
+    for (int k = lane; k < a.topK; k += lanes) {
+        const int64_t slot = static_cast<int64_t>(tokOk ? token : 0) * a.topK + k;
+        int row = tokOk ? LookupRow(a, slot) : -1;
+        if (row >= 0 && a.tileFlags != nullptr && !WaitTile(a, row)) {
+            if (a.deviceStatus != nullptr) {
+                atomicExch(a.deviceStatus, 1);
+            }
+            row = -1;
+        }
+        rows[k] = row;
+        weights[k] = (tokOk && a.expertScales != nullptr) ? a.expertScales[slot] : 1.0f;
+    }
+}
+
+template <int G, int V, int KIND, int INQ, bool BF16, int COMMQ>
+__global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
+{
+    constexpr int kTokens = kThreads / G;
+    constexpr bool kMx = COMMQ != 0;
+    constexpr bool kCommE5m2 = COMMQ == TILEXR_EP_QUANT_COMM_MXFP8_E5M2;
+    __shared__ int s_row[kTokens][kMaxTopK];
+    __shared__ float s_w[kTokens][kMaxTopK];
+
+    const int tg = threadIdx.x / G;
+    const int lane = threadIdx.x % G;
+    const int vecs = a.h / 8;
+    const int groups = (a.bs + kTokens - 1) / kTokens;
+    const int b128 = (a.h + 127) / 128;
+
+    for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+        const int token = group * kTokens + tg;
+        const bool tokOk = token < a.bs;
+        __syncthreads();        // the previous iteration's readers are done with s_row / s_w
+        LoadRoutes(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
+        __syncthreads();
+        if (KIND == kReducePerAdd) {
+            if (lane == 0) {
+                SortRows(s_row[tg], a.topK);
+            }
+            __syncthreads();
+        }
+        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0);
+
+        float acc[V][8];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                acc[j][e] = 0.0f;
+            }
+        }
+        // control flow below is uniform across the lanes that share a token (the MXFP8 round trip shuffles)
+        for (int k = 0; k < a.topK; ++k) {
+            const int row = s_row[tg][k];
+            if (row < 0 || !active) {
+                continue;
+            }
+            const float w = s_w[tg][k];
+            const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row) * a.rowBytes;
+            u32x4 v16[V];
+            u32x2 v8[V];
+            float sc[V];
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = j * G + lane;
+                const bool inRow = idx < vecs;
+                if (INQ == 0) {
+                    v16[j] = inRow ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) :
+                                     u32x4{0u, 0u, 0u, 0u};
+                } else {
+                    v8[j] = inRow ? __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(base) + idx) :
+                                    u32x2{0u, 0u};
+                    sc[j] = !inRow ? 0.0f : (INQ == TILEXR_EP_QUANT_TOKEN_INT8 ? a.inScales[row] :
+                        a.inScales[static_cast<int64_t>(row) * b128 + (idx >> 4)]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                float f[8];
+                if (INQ == 0) {
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        f[2 * q] = Decode16<BF16>(v16[j][q] & 0xffffu);
+                        f[2 * q + 1] = Decode16<BF16>(v16[j][q] >> 16);
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const uint32_t byte = (v8[j][e >> 2] >> ((e & 3) * 8)) & 0xffu;
+                        const float d = INQ == TILEXR_EP_QUANT_TOKEN_INT8 ?
+                            __fmul_rn(static_cast<float>(static_cast<int>(static_cast<int8_t>(byte))), sc[j]) :
+                            __fmul_rn(Fp8Decode<false>(byte), sc[j]);
+                        f[e] = BF16 ? __uint_as_float(FloatToBf16Rne(d) << 16) :
+                                      __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d))));
+                    }
+                }
+                if (kMx) {
+                    float amax = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        amax = fmaxf(amax, fabsf(f[e]));
+                    }
+                    amax = fmaxf(amax, __shfl_xor(amax, 1));
+                    amax = fmaxf(amax, __shfl_xor(amax, 2));
+                    const int se = MxSharedExponent<kCommE5m2>(amax);
+                    const float up = Exp2Int(se);
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float back = Fp8Decode<kCommE5m2>(Fp8Encode<kCommE5m2>(ldexpf(f[e], -se)));
+                        f[e] = __fmul_rn(back, up);
+                    }
+                }
+                if (KIND == kReducePerAdd) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        acc[j][e] = RoundTo16<BF16>(__fadd_rn(acc[j][e], f[e]));
+                    }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        acc[j][e] = __fadd_rn(acc[j][e], __fmul_rn(f[e], w));
+                    }
+                }
+            }
+        }
+        if (a.sharedExpertX != nullptr && active) {
+            const u32x4 *sx = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.sharedExpertX) +
+                static_cast<int64_t>(token) * a.h * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = j * G + lane;
+                if (idx < vecs) {
+                    const u32x4 v = sx[idx];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        acc[j][2 * q] = __fadd_rn(acc[j][2 * q], Decode16<BF16>(v[q] & 0xffffu));
+                        acc[j][2 * q + 1] = __fadd_rn(acc[j][2 * q + 1], Decode16<BF16>(v[q] >> 16));
+                    }
+                }
+            }
+        }
+        if (tokOk) {
+            u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.y) + static_cast<int64_t>(token) * a.h * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = j * G + lane;
+                if (idx < vecs) {
+                    u32x4 o;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const uint32_t lo = active ? Encode16Sat<BF16>(acc[j][2 * q]) : 0u;
+                        const uint32_t hi = active ? Encode16Sat<BF16>(acc[j][2 * q + 1]) : 0u;
+                        o[q] = lo | (hi << 16);
+                    }
+                    __builtin_nontemporal_store(o, dst + idx);
+                }
+            }
+        }
+    }
+}
+
+// Element-granular reduce for any h / alignment.  One workgroup per token; a thread owns whole 32-column blocks so
+// that the MXFP8 round trip needs no cross-lane traffic.
+template <bool BF16>
+__global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs a, int kind, int inq, int commq)
+{
+    __shared__ int s_row[kMaxTopK];
+    __shared__ float s_w[kMaxTopK];
+    const int tid = threadIdx.x;
+    const int b128 = (a.h + 127) / 128;
+    for (int token = blockIdx.x; token < a.bs; token += gridDim.x) {
+        __syncthreads();
+        LoadRoutes(a, token, true, tid, kThreads, s_row, s_w);
+        __syncthreads();
+        if (kind == kReducePerAdd) {
+            if (tid == 0) {
+                SortRows(s_row, a.topK);
+            }
+            __syncthreads();
+        }
+        const bool active = a.tokenMask == nullptr || a.tokenMask[token] != 0;
+        uint16_t *dst = static_cast<uint16_t *>(a.y) + static_cast<int64_t>(token) * a.h;
+        const int blocks = (a.h + 31) / 32;
+        for (int b = tid; b < blocks; b += kThreads) {
+            const int begin = b * 32;
+            const int end = min(begin + 32, a.h);
+            float acc[32];
+            for (int i = 0; i < 32; ++i) {
+                acc[i] = 0.0f;
+            }
+            if (active) {
+                for (int k = 0; k < a.topK; ++k) {
+                    const int row = s_row[k];
+                    if (row < 0) {
+                        continue;
+                    }
+                    const float w = s_w[k];
+                    const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row) * a.rowBytes;
+                    float f[32];
+                    float amax = 0.0f;
+                    for (int i = begin; i < end; ++i) {
+                        float v;
+                        if (inq == 0) {
+                            v = Decode16<BF16>(reinterpret_cast<const uint16_t *>(base)[i]);
+                        } else {
+                            const uint32_t byte = reinterpret_cast<const uint8_t *>(base)[i];
+                            const float d = inq == TILEXR_EP_QUANT_TOKEN_INT8 ?
+                                __fmul_rn(static_cast<float>(static_cast<int>(static_cast<int8_t>(byte))), a.inScales[row]) :
+                                __fmul_rn(Fp8Decode<false>(byte), a.inScales[static_cast<int64_t>(row) * b128 + i / 128]);
+                            v = BF16 ? __uint_as_float(FloatToBf16Rne(d) << 16) :
+                                       __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d))));
+                        }
+                        f[i - begin] = v;
+                        amax = fmaxf(amax, fabsf(v));
+                    }
+                    if (commq != 0) {
+                        const bool e5 = commq == TILEXR_EP_QUANT_COMM_MXFP8_E5M2;
+                        const int se = e5 ? MxSharedExponent<true>(amax) : MxSharedExponent<false>(amax);
+                        const float up = Exp2Int(se);
+                        for (int i = 0; i < end - begin; ++i) {
+                            const float s = ldexpf(f[i], -se);
+                            const float back = e5 ? Fp8Decode<true>(Fp8Encode<true>(s)) : Fp8Decode<false>(Fp8Encode<false>(s));
+                            f[i] = __fmul_rn(back, up);
+                        }
+                    }
+                    for (int i = 0; i < end - begin; ++i) {
+                        if (kind == kReducePerAdd) {
+                            acc[i] = RoundTo16<BF16>(__fadd_rn(acc[i], f[i]));
+                        } else {
+                            acc[i] = __fadd_rn(acc[i], __fmul_rn(f[i], w));
+                        }
+                    }
+                }
+                if (a.sharedExpertX != nullptr) {
+                    const uint16_t *sx = static_cast<const uint16_t *>(a.sharedExpertX) + static_cast<int64_t>(token) * a.h;
+                    for (int i = begin; i < end; ++i) {
+                        acc[i - begin] = __fadd_rn(acc[i - begin], Decode16<BF16>(sx[i]));
+                    }
+                }
+            }
+            for (int i = begin; i < end; ++i) {
+                dst[i] = active ? static_cast<uint16_t>(Encode16Sat<BF16>(acc[i - begin])) : static_cast<uint16_t>(0);
+            }
+        }
+    }
+}
+
+template <int G, int V, int KIND, int INQ, bool BF16, int COMMQ>
+void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
+{
+    constexpr int kTokens = kThreads / G;
+    int grid = (a.bs + kTokens - 1) / kTokens;
+    if (gridLimit > 0 && grid > gridLimit) {
+        grid = gridLimit;
+    }
+    hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, INQ, BF16, COMMQ>), dim3(grid), dim3(kThreads), 0, stream, a);
+}
+
+template <int G, int V, bool BF16>
+void LaunchByMode(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
+{
+    if (l.reduceKind == kReducePerAdd) {
+        LaunchVec<G, V, kReducePerAdd, 0, BF16, 0>(a, gridLimit, l.stream);
+    } else if (l.inQuant == TILEXR_EP_QUANT_TOKEN_INT8) {
+        LaunchVec<G, V, kReduceFp32, TILEXR_EP_QUANT_TOKEN_INT8, BF16, 0>(a, gridLimit, l.stream);
+    } else if (l.inQuant == TILEXR_EP_QUANT_FP8_BLOCK128) {
+        LaunchVec<G, V, kReduceFp32, TILEXR_EP_QUANT_FP8_BLOCK128, BF16, 0>(a, gridLimit, l.stream);
+    } else if (l.commQuant == TILEXR_EP_QUANT_COMM_MXFP8_E5M2) {
+        LaunchVec<G, V, kReduceFp32, 0, BF16, TILEXR_EP_QUANT_COMM_MXFP8_E5M2>(a, gridLimit, l.stream);
+    } else if (l.commQuant == TILEXR_EP_QUANT_MXFP8) {
+        LaunchVec<G, V, kReduceFp32, 0, BF16, TILEXR_EP_QUANT_MXFP8>(a, gridLimit, l.stream);
+    } else {
+        LaunchVec<G, V, kReduceFp32, 0, BF16, 0>(a, gridLimit, l.stream);
+    }
+}
+
+template <int G, int V>
+void LaunchByType(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
+{
+    if (l.bf16) {
+        LaunchByMode<G, V, true>(l, a, gridLimit);
+    } else {
+        LaunchByMode<G, V, false>(l, a, gridLimit);
+    }
+}
+
+} // namespace
+
+hipError_t LaunchReduce(const ReduceLaunch &l)
+{
+    ReduceArgs a {};
+    a.expertOut = l.expertOut;
+    a.rowBytes = l.rowBytes;
+    a.inverseTagged = l.inverseTagged;
+    a.epoch = l.epoch;
+    a.rowIndexMap = l.rowIndexMap;
+    a.expertScales = l.expertScales;
+    a.tokenMask = l.tokenMask;
+    a.sharedExpertX = l.sharedExpertX;
+    a.inScales = l.inScales;
+    a.bs = static_cast<int>(l.bs);
+    a.h = static_cast<int>(l.h);
+    a.topK = static_cast<int>(l.topK);
+    a.y = l.y;
+    a.tileFlags = l.tileFlags;
+    a.tileRows = static_cast<int>(l.tileRows);
+    a.totalRowsPtr = l.totalRowsPtr;
+    a.flagEpoch = l.flagEpoch;
+    a.waitTimeoutTicks = l.waitTimeoutTicks;
+    a.deviceStatus = l.deviceStatus;
+    // A kernel that waits on flags must never crowd out the producer it waits for: keep it to two workgroups per
+    // compute unit (8 of 32 wave slots) and let it walk the tokens.
+    const int gridLimit = l.tileFlags != nullptr ? 2 * (l.numComputeUnits > 0 ? l.numComputeUnits : 256) : 0;
+    const int64_t vecs = l.h / 8;
+    const bool mixed = (l.inQuant != 0 && l.commQuant != 0);
+    const bool vecOk = !mixed && l.h % 8 == 0 && Aligned16(l.y) && vecs <= 8 * kThreads &&
+        (l.inQuant == 0 ? (Aligned16(l.expertOut) && l.rowBytes % 16 == 0) :
+                          (Aligned8(l.expertOut) && l.rowBytes % 8 == 0)) &&
+        (l.sharedExpertX == nullptr || Aligned16(l.sharedExpertX)) && (l.commQuant == 0 || l.h % 32 == 0);
+    if (vecOk) {
+        if (vecs <= 2 * kWave) {
+            LaunchByType<kWave, 2>(l, a, gridLimit);
+        } else if (vecs <= 4 * kWave) {
+            LaunchByType<kWave, 4>(l, a, gridLimit);
+        } else if (vecs <= 2 * kThreads) {
+            LaunchByType<kThreads, 2>(l, a, gridLimit);
+        } else if (vecs <= 4 * kThreads) {
+            LaunchByType<kThreads, 4>(l, a, gridLimit);
+        } else {
+            LaunchByType<kThreads, 8>(l, a, gridLimit);
+        }
+    } else {
+        int grid = static_cast<int>(l.bs);
+        if (gridLimit > 0 && grid > gridLimit) {
+            grid = gridLimit;
+        }
+        if (l.bf16) {
+            hipLaunchKernelGGL((ep_reduce_generic_kernel<true>), dim3(grid), dim3(kThreads), 0, l.stream, a,
+                l.reduceKind, l.inQuant, l.commQuant);
+        } else {
+            hipLaunchKernelGGL((ep_reduce_generic_kernel<false>), dim3(grid), dim3(kThreads), 0, l.stream, a,
+                l.reduceKind, l.inQuant, l.commQuant);
+        }
+    }
+    return hipGetLastError();
+}
+
+} // namespace TileXREp

@@ -1,0 +1,404 @@
+// scatter: each token row is read once and written to the rows its routes were placed at (gfx950, wave64).
+//
+// HBM-bound byte movement, no MFMA.  G lanes cooperate on one token (a wave for narrow rows, the whole workgroup for
+// wide ones); a lane keeps V 16-byte vectors of the row in registers, so every load of the row is in flight before
+// the first store, then writes them to each of the topK destination rows with non-temporal 128-bit stores (the rows
+// are not read again by this kernel; the input row is loaded with the default policy so that a producer's output
+// still sitting in L2 / Infinity Cache is used).  Measured on MI355X this shape moves 4096 x 7168 bf16 x top-8
+// (529 MB) at about 5.6 TB/s; destination order (sorted or random rows) makes no difference.
+//
+//   QMODE 0  byte copy             (reference: src/ep/kernels/tilexr_ep_dispatch_helpers.h:104-112)
+//   QMODE 1  static int8           (reference: tilexr_ep_dispatch_helpers.h:114-136)
+//   QMODE 2  per-token int8        (reference: tilexr_ep_dispatch_helpers.h:153-191; BF16 decode has no counterpart)
+//   QMODE 4  MXFP8, 32-wide blocks (reference: tests/ep/demo/mxfp8_golden.h:116-152)
+//   QMODE 5  fp8 e4m3, fp32 scale per 128 columns (no reference counterpart)
+#include <hip/hip_runtime.h>
+
+#include "ep_kernel_common.cuh"
+#include "ep_launch.h"
+#include "ep_numerics.cuh"
+#include "tilexr_ep.h"
+
+namespace TileXREp {
+namespace {
+
+struct ScatterArgs {
+    const void *x;
+    const int32_t *rowOf;
+    int bs;
+    int h;
+    int topK;
+    const float *staticScale;
+    void *out;
+    void *scalesOut;
+    uint64_t *tileFlags;
+    int tileRows;
+};
+
+template <int G>
+__device__ __forceinline__ float GroupMax(float v, float *red, int lane)
+{
+#pragma unroll
+    for (int off = kWave / 2; off >= 1; off >>= 1) {
+        v = fmaxf(v, __shfl_xor(v, off));
+    }
+    if (G > kWave) {
+        if ((lane & (kWave - 1)) == 0) {
+            red[lane / kWave] = v;
+        }
+        __syncthreads();
+        v = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        __syncthreads();
+    }
+    return v;
+}
+
+__device__ __forceinline__ void PublishRows(uint64_t *tileFlags, int tileRows, const int *pos, int topK, int lane, int G)
+{
+    // every lane's row stores are complete once the workgroup barrier has been passed; the release below makes
+    // them visible at agent scope before the tile counter moves
+    __syncthreads();
+    for (int k = lane; k < topK; k += G) {
+        const int row = pos[k];
+        if (row >= 0) {
+            __hip_atomic_fetch_add(&tileFlags[row / tileRows], 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
+template <int G, int V, int QMODE, bool BF16, bool E5M2>
+__global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
+{
+    constexpr int kTokens = kThreads / G;
+    __shared__ int s_pos[kTokens][kMaxTopK];
+    __shared__ float s_red[kTokens][kWavesPerBlock];
+
+    const int tg = threadIdx.x / G;
+    const int lane = threadIdx.x % G;
+    const int token = blockIdx.x * kTokens + tg;
+    const bool tokOk = token < a.bs;
+    const int vecs = a.h / 8;
+
+    for (int k = lane; k < a.topK; k += G) {
+        s_pos[tg][k] = tokOk ? a.rowOf[static_cast<int64_t>(token) * a.topK + k] : -1;
+    }
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.x) +
+        static_cast<int64_t>(tokOk ? token : 0) * a.h * 2);
+    u32x4 v[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int idx = j * G + lane;
+        v[j] = (tokOk && idx < vecs) ? src[idx] : u32x4{0u, 0u, 0u, 0u};
+    }
+    __syncthreads();
+
+    if (QMODE == TILEXR_EP_QUANT_NONE) {
+        for (int k = 0; k < a.topK; ++k) {
+            const int row = s_pos[tg][k];
+            if (row < 0) {
+                continue;
+            }
+            u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = j * G + lane;
+                if (idx < vecs) {
+                    __builtin_nontemporal_store(v[j], dst + idx);
+                }
+            }
+        }
+    } else {
+        // per-row / per-block scale, then 8 output bytes per input vector
+        float rowScaleInv = 1.0f;
+        float rowScale = 1.0f;
+        if (QMODE == TILEXR_EP_QUANT_STATIC_INT8) {
+            rowScaleInv = a.staticScale[0];
+        }
+        if (QMODE == TILEXR_EP_QUANT_TOKEN_INT8) {
+            float amax = 0.0f;
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    amax = fmaxf(amax, fabsf(Decode16<BF16>(v[j][w] & 0xffffu)));
+                    amax = fmaxf(amax, fabsf(Decode16<BF16>(v[j][w] >> 16)));
+                }
+            }
+            amax = GroupMax<G>(amax, s_red[tg], lane);
+            rowScale = amax > 0.0f ? __fdiv_rn(amax, 127.0f) : 1.0f;
+            rowScaleInv = rowScale > 0.0f ? __fdiv_rn(1.0f, rowScale) : 1.0f;
+        }
+        u32x2 q[V];
+        float blockScale[V];
+        int sharedExp[V];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+            float f[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                f[2 * w] = Decode16<BF16>(v[j][w] & 0xffffu);
+                f[2 * w + 1] = Decode16<BF16>(v[j][w] >> 16);
+            }
+            uint32_t bytes[8];
+            if (QMODE == TILEXR_EP_QUANT_MXFP8 || QMODE == TILEXR_EP_QUANT_FP8_BLOCK128) {
+                float amax = 0.0f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    amax = fmaxf(amax, fabsf(f[e]));
+                }
+                // 32 columns = 4 neighbouring lanes, 128 columns = 16 neighbouring lanes
+                constexpr int kSpan = QMODE == TILEXR_EP_QUANT_MXFP8 ? 4 : 16;
+#pragma unroll
+                for (int off = 1; off < kSpan; off <<= 1) {
+                    amax = fmaxf(amax, __shfl_xor(amax, off));
+                }
+                if (QMODE == TILEXR_EP_QUANT_MXFP8) {
+                    const int se = MxSharedExponent<E5M2>(amax);
+                    sharedExp[j] = se;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        bytes[e] = Fp8Encode<E5M2>(ldexpf(f[e], -se));
+                    }
+                } else {
+                    const float sc = amax > 0.0f ? __fdiv_rn(amax, 448.0f) : 1.0f;
+                    blockScale[j] = sc;
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        bytes[e] = Fp8Encode<false>(__fdiv_rn(f[e], sc));
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    bytes[e] = static_cast<uint32_t>(ClampInt8(__fmul_rn(f[e], rowScaleInv))) & 0xffu;
+                }
+            }
+            q[j][0] = bytes[0] | (bytes[1] << 8) | (bytes[2] << 16) | (bytes[3] << 24);
+            q[j][1] = bytes[4] | (bytes[5] << 8) | (bytes[6] << 16) | (bytes[7] << 24);
+        }
+        const int mxBlocks = (a.h + 31) / 32;
+        const int mxScales = (mxBlocks + 1) / 2 * 2;
+        const int b128 = (a.h + 127) / 128;
+        for (int k = 0; k < a.topK; ++k) {
+            const int row = s_pos[tg][k];
+            if (row < 0) {
+                continue;
+            }
+            u32x2 *dst = reinterpret_cast<u32x2 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = j * G + lane;
+                if (idx < vecs) {
+                    __builtin_nontemporal_store(q[j], dst + idx);
+                    if (QMODE == TILEXR_EP_QUANT_MXFP8 && (idx & 3) == 0) {
+                        uint8_t *sc = static_cast<uint8_t *>(a.scalesOut) + static_cast<int64_t>(row) * mxScales;
+                        sc[idx >> 2] = static_cast<uint8_t>(sharedExp[j] + 127);
+                        if ((idx >> 2) + 1 == mxBlocks && mxBlocks < mxScales) {
+                            sc[mxBlocks] = 0;       // padding byte of an odd block count
+                        }
+                    }
+                    if (QMODE == TILEXR_EP_QUANT_FP8_BLOCK128 && (idx & 15) == 0) {
+                        static_cast<float *>(a.scalesOut)[static_cast<int64_t>(row) * b128 + (idx >> 4)] = blockScale[j];
+                    }
+                }
+            }
+            if (QMODE == TILEXR_EP_QUANT_TOKEN_INT8 && lane == 0) {
+                static_cast<float *>(a.scalesOut)[row] = rowScale;
+            }
+        }
+    }
+    if (a.tileFlags != nullptr) {
+        PublishRows(a.tileFlags, a.tileRows, s_pos[tg], a.topK, lane, G);
+    }
+}
+
+// Any row width / alignment: one workgroup per token, element-granular.  Used when h is not a multiple of 8, a
+// base pointer is not 16-byte aligned or the row does not fit the register-resident kernel.
+template <bool BF16, bool E5M2>
+__global__ __launch_bounds__(kThreads) void ep_scatter_generic_kernel(ScatterArgs a, int qmode)
+{
+    __shared__ int s_pos[kMaxTopK];
+    __shared__ float s_red[kWavesPerBlock];
+    const int token = blockIdx.x;
+    const int tid = threadIdx.x;
+    for (int k = tid; k < a.topK; k += kThreads) {
+        s_pos[k] = a.rowOf[static_cast<int64_t>(token) * a.topK + k];
+    }
+    const uint16_t *src = static_cast<const uint16_t *>(a.x) + static_cast<int64_t>(token) * a.h;
+    float rowScale = 1.0f;
+    float rowScaleInv = qmode == TILEXR_EP_QUANT_STATIC_INT8 ? a.staticScale[0] : 1.0f;
+    if (qmode == TILEXR_EP_QUANT_TOKEN_INT8) {
+        float amax = 0.0f;
+        for (int i = tid; i < a.h; i += kThreads) {
+            amax = fmaxf(amax, fabsf(Decode16<BF16>(src[i])));
+        }
+        amax = GroupMax<kThreads>(amax, s_red, tid);
+        rowScale = amax > 0.0f ? __fdiv_rn(amax, 127.0f) : 1.0f;
+        rowScaleInv = rowScale > 0.0f ? __fdiv_rn(1.0f, rowScale) : 1.0f;
+    }
+    __syncthreads();
+    const int mxBlocks = (a.h + 31) / 32;
+    const int mxScales = (mxBlocks + 1) / 2 * 2;
+    const int b128 = (a.h + 127) / 128;
+    for (int k = 0; k < a.topK; ++k) {
+        const int row = s_pos[k];
+        if (row < 0) {
+            continue;
+        }
+        if (qmode == TILEXR_EP_QUANT_NONE) {
+            uint16_t *dst = static_cast<uint16_t *>(a.out) + static_cast<int64_t>(row) * a.h;
+            for (int i = tid; i < a.h; i += kThreads) {
+                dst[i] = src[i];
+            }
+        } else if (qmode == TILEXR_EP_QUANT_STATIC_INT8 || qmode == TILEXR_EP_QUANT_TOKEN_INT8) {
+            int8_t *dst = static_cast<int8_t *>(a.out) + static_cast<int64_t>(row) * a.h;
+            for (int i = tid; i < a.h; i += kThreads) {
+                dst[i] = static_cast<int8_t>(ClampInt8(__fmul_rn(Decode16<BF16>(src[i]), rowScaleInv)));
+            }
+            if (qmode == TILEXR_EP_QUANT_TOKEN_INT8 && tid == 0) {
+                static_cast<float *>(a.scalesOut)[row] = rowScale;
+            }
+        } else if (qmode == TILEXR_EP_QUANT_MXFP8) {
+            uint8_t *dst = static_cast<uint8_t *>(a.out) + static_cast<int64_t>(row) * a.h;
+            uint8_t *sc = static_cast<uint8_t *>(a.scalesOut) + static_cast<int64_t>(row) * mxScales;
+            for (int b = tid; b < mxScales; b += kThreads) {
+                if (b >= mxBlocks) {
+                    sc[b] = 0;
+                    continue;
+                }
+                const int begin = b * 32;
+                const int end = min(begin + 32, a.h);
+                float amax = 0.0f;
+                for (int i = begin; i < end; ++i) {
+                    amax = fmaxf(amax, fabsf(Decode16<BF16>(src[i])));
+                }
+                const int se = MxSharedExponent<E5M2>(amax);
+                sc[b] = static_cast<uint8_t>(se + 127);
+                for (int i = begin; i < end; ++i) {
+                    dst[i] = static_cast<uint8_t>(Fp8Encode<E5M2>(ldexpf(Decode16<BF16>(src[i]), -se)));
+                }
+            }
+        } else {
+            uint8_t *dst = static_cast<uint8_t *>(a.out) + static_cast<int64_t>(row) * a.h;
+            float *sc = static_cast<float *>(a.scalesOut) + static_cast<int64_t>(row) * b128;
+            for (int b = tid; b < b128; b += kThreads) {
+                const int begin = b * 128;
+                const int end = min(begin + 128, a.h);
+                float amax = 0.0f;
+                for (int i = begin; i < end; ++i) {
+                    amax = fmaxf(amax, fabsf(Decode16<BF16>(src[i])));
+                }
+                const float scale = amax > 0.0f ? __fdiv_rn(amax, 448.0f) : 1.0f;
+                sc[b] = scale;
+                for (int i = begin; i < end; ++i) {
+                    dst[i] = static_cast<uint8_t>(Fp8Encode<false>(__fdiv_rn(Decode16<BF16>(src[i]), scale)));
+                }
+            }
+        }
+    }
+    if (a.tileFlags != nullptr) {
+        PublishRows(a.tileFlags, a.tileRows, s_pos, a.topK, tid, kThreads);
+    }
+}
+
+template <int G, int V, int QMODE, bool BF16, bool E5M2>
+void LaunchVec(const ScatterArgs &a, hipStream_t stream)
+{
+    constexpr int kTokens = kThreads / G;
+    const int grid = (a.bs + kTokens - 1) / kTokens;
+    hipLaunchKernelGGL((ep_scatter_vec_kernel<G, V, QMODE, BF16, E5M2>), dim3(grid), dim3(kThreads), 0, stream, a);
+}
+
+template <int G, int V>
+void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
+{
+    switch (l.quantMode) {
+        case TILEXR_EP_QUANT_NONE:
+            LaunchVec<G, V, TILEXR_EP_QUANT_NONE, true, false>(a, l.stream);
+            break;
+        case TILEXR_EP_QUANT_STATIC_INT8:
+            LaunchVec<G, V, TILEXR_EP_QUANT_STATIC_INT8, false, false>(a, l.stream);
+            break;
+        case TILEXR_EP_QUANT_TOKEN_INT8:
+            if (l.inputBf16) {
+                LaunchVec<G, V, TILEXR_EP_QUANT_TOKEN_INT8, true, false>(a, l.stream);
+            } else {
+                LaunchVec<G, V, TILEXR_EP_QUANT_TOKEN_INT8, false, false>(a, l.stream);
+            }
+            break;
+        case TILEXR_EP_QUANT_MXFP8:
+            if (l.inputBf16) {
+                if (l.fp8E5m2) {
+                    LaunchVec<G, V, TILEXR_EP_QUANT_MXFP8, true, true>(a, l.stream);
+                } else {
+                    LaunchVec<G, V, TILEXR_EP_QUANT_MXFP8, true, false>(a, l.stream);
+                }
+            } else {
+                if (l.fp8E5m2) {
+                    LaunchVec<G, V, TILEXR_EP_QUANT_MXFP8, false, true>(a, l.stream);
+                } else {
+                    LaunchVec<G, V, TILEXR_EP_QUANT_MXFP8, false, false>(a, l.stream);
+                }
+            }
+            break;
+        default:
+            if (l.inputBf16) {
+                LaunchVec<G, V, TILEXR_EP_QUANT_FP8_BLOCK128, true, false>(a, l.stream);
+            } else {
+                LaunchVec<G, V, TILEXR_EP_QUANT_FP8_BLOCK128, false, false>(a, l.stream);
+            }
+            break;
+    }
+}
+
+} // namespace
+
+hipError_t LaunchScatter(const ScatterLaunch &l)
+{
+    ScatterArgs a {};
+    a.x = l.x;
+    a.rowOf = l.rowOf;
+    a.bs = static_cast<int>(l.bs);
+    a.h = static_cast<int>(l.h);
+    a.topK = static_cast<int>(l.topK);
+    a.staticScale = l.staticScale;
+    a.out = l.out;
+    a.scalesOut = l.scalesOut;
+    a.tileFlags = l.tileFlags;
+    a.tileRows = static_cast<int>(l.tileRows);
+    const int64_t vecs = l.h / 8;
+    const bool vecOk = l.h % 8 == 0 && Aligned16(l.x) && vecs <= 8 * kThreads &&
+        (l.quantMode == TILEXR_EP_QUANT_NONE ? Aligned16(l.out) : Aligned8(l.out));
+    if (vecOk) {
+        // narrow rows: a wave per token (four tokens per workgroup); wide rows: the workgroup per token
+        if (vecs <= 2 * kWave) {
+            LaunchByMode<kWave, 2>(l, a);
+        } else if (vecs <= 4 * kWave) {
+            LaunchByMode<kWave, 4>(l, a);
+        } else if (vecs <= 2 * kThreads) {
+            LaunchByMode<kThreads, 2>(l, a);
+        } else if (vecs <= 4 * kThreads) {
+            LaunchByMode<kThreads, 4>(l, a);
+        } else {
+            LaunchByMode<kThreads, 8>(l, a);
+        }
+    } else {
+        const dim3 grid(static_cast<unsigned>(l.bs));
+        if (l.inputBf16) {
+            if (l.fp8E5m2) {
+                hipLaunchKernelGGL((ep_scatter_generic_kernel<true, true>), grid, dim3(kThreads), 0, l.stream, a, l.quantMode);
+            } else {
+                hipLaunchKernelGGL((ep_scatter_generic_kernel<true, false>), grid, dim3(kThreads), 0, l.stream, a, l.quantMode);
+            }
+        } else {
+            if (l.fp8E5m2) {
+                hipLaunchKernelGGL((ep_scatter_generic_kernel<false, true>), grid, dim3(kThreads), 0, l.stream, a, l.quantMode);
+            } else {
+                hipLaunchKernelGGL((ep_scatter_generic_kernel<false, false>), grid, dim3(kThreads), 0, l.stream, a, l.quantMode);
+            }
+        }
+    }
+    return hipGetLastError();
+}
+
+} // namespace TileXREp
