@@ -1,0 +1,314 @@
+"""GPU parity for several logical ranks on one device (the reference's 4-rank checker configuration and friends).
+
+Each rank has its own communicator and stream; a rank's outputs are complete once every rank of the world has made
+the call and the rank's stream has been synchronised.  Everything is compared bit-exactly: against the CPU oracle
+on seeded inputs and against the reference checker's own output blobs (tests/golden/checker_fixtures.npz).
+"""
+import hashlib
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from gpu_harness import DEV, alloc_dispatch_outputs, bits16, to_dev
+from oracle import ep as O
+from tilexr_amd import ep
+
+pytestmark = pytest.mark.gpu
+
+FIXTURES = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "checker_fixtures.npz")
+
+
+class World:
+    def __init__(self, ranks):
+        torch.cuda.set_device(0)
+        self.ranks = ranks
+        self.comms = [ep.Comm(ranks, r) for r in range(ranks)]
+        self.streams = [torch.cuda.Stream() for _ in range(ranks)]
+
+    def sync(self):
+        for s in self.streams:
+            s.synchronize()
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        torch.cuda.synchronize()
+        for c in self.comms:
+            c.destroy()
+
+
+def rand_ids(rng, R, bs, K, E, invalid=0.0):
+    ids = np.stack([np.stack([rng.permutation(E)[:K] for _ in range(bs)]) for _ in range(R)]).astype(np.int32)
+    if invalid:
+        bad = rng.random(ids.shape) < invalid
+        ids[bad] = rng.choice([-1, -7, E, E + 5], size=int(bad.sum()))
+    return ids
+
+
+def rand_x(rng, R, bs, h, dtype, scale=1.0):
+    f = (rng.standard_normal((R, bs, h)) * scale).astype(np.float32)
+    t = torch.from_numpy(f).to(torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16)
+    return t.to(DEV), bits16(t)
+
+
+def run_dispatch(world, memory, xt, ids, bs, h, K, E, dtype, order=None, quant=ep.Q_NONE, mask=None,
+                 mask_type=ep.MASK_NONE, nums_type=1, static=None, fp8=None):
+    """Calls every rank (in `order`), returns the per-rank output dicts (device tensors)."""
+    R = world.ranks
+    outs = []
+    for r in range(R):
+        out = alloc_dispatch_outputs(bs, h, K, E, ranks=R, quant=quant)
+        out["counts"] = torch.full((E if memory else R,), -1, dtype=torch.int32, device=DEV)
+        out["tp_counts"] = torch.full((R,), -1, dtype=torch.int32, device=DEV)
+        outs.append(out)
+    dev_ids = [to_dev(ids[r]) for r in range(R)]
+    dev_mask = [None if mask is None else to_dev(mask[r]) for r in range(R)]
+    dev_static = to_dev(static)
+    keep = (dev_ids, dev_mask, dev_static)
+    for r in (order or range(R)):
+        o = outs[r]
+        if memory:
+            st = ep.dispatch_memory_v2(
+                xt[r], dev_ids[r], world.comms[r], bs, h, K, E, o["expand_x"], o["assist"], o["token_nums"],
+                o["counts"], dtype, world.streams[r], active_mask=dev_mask[r], active_mask_type=mask_type,
+                quant_mode=quant, token_nums_type=nums_type, dynamic_scales=o["scales"],
+                expand_x_dtype=fp8 if quant == ep.Q_MXFP8 else ep.DT_RESERVED)
+        else:
+            st = ep.dispatch_v2(
+                xt[r], dev_ids[r], world.comms[r], bs, h, K, E, o["expand_x"], o["assist"], o["token_nums"],
+                o["counts"], dtype if quant == ep.Q_NONE else ep.DT_INT8, world.streams[r],
+                scales=dev_static if quant == ep.Q_STATIC_INT8 else None, active_mask=dev_mask[r], quant_mode=quant,
+                token_nums_type=nums_type, dynamic_scales=o["scales"] if quant == ep.Q_TOKEN_INT8 else None,
+                tp_recv_counts=o["tp_counts"])
+        assert st == 0, f"rank {r}: status {st}"
+    world.sync()
+    del keep
+    return outs
+
+
+def check_rank(out, want, counts_key):
+    n = want["rows"]
+    assert np.array_equal(out["assist"].cpu().numpy()[:n], want["assist"][:n])
+    assert np.array_equal(out["expand_x"].cpu().numpy()[:n], want["expand_x"][:n])
+    assert np.array_equal(out["token_nums"].cpu().numpy(), want["expert_token_nums"])
+    assert np.array_equal(out["counts"].cpu().numpy(), want[counts_key])
+    assert np.all(out["assist"].cpu().numpy()[n:] == -77)
+
+
+MULTI_SHAPES = [(2, 3, 8, 2, 4), (4, 128, 1024, 2, 16), (4, 33, 40, 3, 8), (8, 50, 256, 4, 32), (3, 17, 33, 2, 6),
+                (4, 300, 512, 8, 64)]
+
+
+@pytest.mark.parametrize("shape", MULTI_SHAPES)
+def test_mvp_dispatch_and_combine_across_ranks(shape):
+    R, bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape))
+    ids = rand_ids(rng, R, bs, K, E, invalid=0.1)
+    xt, xb = rand_x(rng, R, bs, h, ep.DT_FP16, scale=3.0)
+    mask = (rng.random((R, bs)) < 0.7).astype(np.uint8)
+    static = np.array([1.5], np.float32)
+    with World(R) as w:
+        for quant in (ep.Q_NONE, ep.Q_STATIC_INT8, ep.Q_TOKEN_INT8):
+            for use_mask, nums_type in ((False, 1), (True, 0)):
+                order = list(rng.permutation(R))
+                outs = run_dispatch(w, False, xt, ids, bs, h, K, E, ep.DT_FP16, order=order, quant=quant,
+                                    mask=mask if use_mask else None, nums_type=nums_type, static=static)
+                case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16, quant_mode=quant, token_nums_type=nums_type)
+                wants = [O.mvp_dispatch(case, r, xb, ids, mask if use_mask else None, static) for r in range(R)]
+                for r in range(R):
+                    check_rank(outs[r], wants[r], "recv_counts")
+                    assert np.array_equal(outs[r]["tp_counts"].cpu().numpy(), wants[r]["recv_counts"])
+                    if quant == ep.Q_TOKEN_INT8:
+                        n = wants[r]["rows"]
+                        assert np.array_equal(outs[r]["scales"].cpu().numpy()[:n, 0], wants[r]["dyn_scales"][:n])
+                if quant != ep.Q_NONE:
+                    continue
+                # combine: expert outputs = some function of the dispatched rows (here: the rows, scaled by rank)
+                ys = [torch.full((bs, h), 7.0, dtype=torch.float16, device=DEV) for _ in range(R)]
+                eo = []
+                for r in range(R):
+                    t = outs[r]["expand_x"].view(torch.float16) * (1.0 + 0.25 * r)
+                    eo.append(t.contiguous())
+                for r in reversed(order):
+                    st = ep.combine_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
+                                       ep.DT_FP16, w.streams[r])
+                    assert st == 0
+                w.sync()
+                eo_np = np.stack([bits16(t) for t in eo])
+                assist_np = np.stack([o["assist"].cpu().numpy() for o in outs])
+                counts_np = np.stack([o["counts"].cpu().numpy() for o in outs])
+                for r in range(R):
+                    want_y = O.mvp_combine(case, r, eo_np, assist_np, counts_np)
+                    assert np.array_equal(bits16(ys[r]), want_y), f"rank {r}"
+
+
+@pytest.mark.parametrize("shape", MULTI_SHAPES)
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+def test_memory_dispatch_and_combine_across_ranks(shape, dtype):
+    R, bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + dtype)
+    ids = rand_ids(rng, R, bs, K, E, invalid=0.1)
+    xt, xb = rand_x(rng, R, bs, h, dtype)
+    tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+    with World(R) as w:
+        for mask_type, nums_type in ((ep.MASK_NONE, 1), (ep.MASK_TOKEN, 0), (ep.MASK_EXPERT, 1)):
+            mask = None
+            if mask_type == ep.MASK_TOKEN:
+                mask = (rng.random((R, bs)) < 0.7).astype(np.uint8)
+            elif mask_type == ep.MASK_EXPERT:
+                mask = (rng.random((R, bs, K)) < 0.7).astype(np.uint8)
+            order = list(rng.permutation(R))
+            outs = run_dispatch(w, True, xt, ids, bs, h, K, E, dtype, order=order, mask=mask, mask_type=mask_type,
+                                nums_type=nums_type)
+            case = O.Case(R, bs, h, K, E, dtype=dtype, mask_type=mask_type, token_nums_type=nums_type)
+            wants = [O.mem_dispatch(case, r, xb, ids, mask) for r in range(R)]
+            for r in range(R):
+                check_rank(outs[r], wants[r], "send_counts")
+            # combine with weights, a token mask and a shared-expert term on some variants
+            weights = rng.random((R, bs, K)).astype(np.float32)
+            tmask = (rng.random((R, bs)) < 0.8).astype(np.uint8) if mask_type == ep.MASK_TOKEN else None
+            shared_t, shared_b = rand_x(rng, R, bs, h, dtype) if mask_type != ep.MASK_EXPERT else (None, None)
+            comm_quant = {ep.MASK_NONE: 0, ep.MASK_TOKEN: 3, ep.MASK_EXPERT: 4}[mask_type]
+            ys = [torch.full((bs, h), 7.0, dtype=tdt, device=DEV) for _ in range(R)]
+            eo = [(outs[r]["expand_x"].view(tdt) * (1.0 + 0.25 * r)).contiguous() for r in range(R)]
+            dev_w = [to_dev(weights[r]) for r in range(R)]
+            dev_m = [None if tmask is None else to_dev(tmask[r]) for r in range(R)]
+            for r in reversed(order):
+                st = ep.combine_memory_v2(
+                    eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r], dtype, w.streams[r],
+                    expert_scales=dev_w[r], active_mask=dev_m[r],
+                    active_mask_type=ep.MASK_TOKEN if tmask is not None else ep.MASK_NONE,
+                    shared_expert_x=None if shared_t is None else shared_t[r], quant_mode=comm_quant)
+                assert st == 0
+            w.sync()
+            eo_np = np.stack([bits16(t) for t in eo])
+            assist_np = np.stack([o["assist"].cpu().numpy() for o in outs])
+            counts_np = np.stack([o["counts"].cpu().numpy() for o in outs])
+            for r in range(R):
+                want_y = O.mem_combine(case, r, eo_np, assist_np, counts_np, expert_scales=weights[r],
+                                       token_mask=None if tmask is None else tmask[r],
+                                       shared_expert_x=None if shared_b is None else shared_b[r],
+                                       comm_quant=comm_quant)
+                assert np.array_equal(bits16(ys[r]), want_y), f"rank {r}"
+
+
+@pytest.mark.parametrize("fp8", [ep.DT_FP8E4M3, ep.DT_FP8E5M2])
+def test_memory_dispatch_mxfp8_across_ranks(fp8):
+    R, bs, h, K, E = 4, 40, 288, 4, 16
+    rng = np.random.default_rng(77 + fp8)
+    ids = rand_ids(rng, R, bs, K, E)
+    xt, xb = rand_x(rng, R, bs, h, ep.DT_BF16, scale=5.0)
+    with World(R) as w:
+        outs = run_dispatch(w, True, xt, ids, bs, h, K, E, ep.DT_BF16, quant=ep.Q_MXFP8, fp8=fp8)
+        case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16, quant_mode=O.Q_MXFP8, out_dtype=fp8)
+        for r in range(R):
+            want = O.mem_dispatch(case, r, xb, ids)
+            check_rank(outs[r], want, "send_counts")
+            n = want["rows"]
+            assert np.array_equal(outs[r]["scales"].cpu().numpy()[:n], want["dyn_scales"][:n])
+
+
+def checker_input(R, bs, h):
+    tt, hh = np.meshgrid(np.arange(bs), np.arange(h), indexing="ij")
+    return np.stack([((0x1000 + r * 0x100 + tt * 0x10 + hh) & 0xffff).astype(np.uint16) for r in range(R)])
+
+
+def test_reference_checker_blobs():
+    """ep_dispatch / ep_combine blobs of the reference's no-NPU checker (tools/checker/src/oracle.cpp:661-708,
+    executor.cpp:471-541) for its default routing, including the 4 x 128 x 1024 top-2 16-expert configuration."""
+    fx = np.load(FIXTURES)
+    for i in range(int(fx["num_cases"][0])):
+        R, bs, h, K, E, dtype = (int(v) for v in fx[f"case{i}_shape"])
+        ids = np.broadcast_to(fx[f"case{i}_ids"], (R, bs, K)).copy()
+        xb = checker_input(R, bs, h)
+        tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+        xt = torch.from_numpy(xb.view(np.int16)).view(tdt).to(DEV)
+        with World(R) as w:
+            outs = run_dispatch(w, False, xt, ids, bs, h, K, E, dtype)
+            ys = []
+            for r in range(R):
+                n = bs * K
+                blob = np.concatenate([
+                    outs[r]["expand_x"].cpu().numpy()[:n].reshape(-1),
+                    np.zeros((R - 1) * n * h * 2, np.uint8),
+                    outs[r]["assist"].cpu().numpy()[:n].reshape(-1).view(np.uint8),
+                    outs[r]["counts"].cpu().numpy().view(np.uint8),
+                    outs[r]["token_nums"].cpu().numpy().view(np.uint8)])
+                if f"case{i}_dispatch_blobs" in fx:
+                    assert np.array_equal(blob, fx[f"case{i}_dispatch_blobs"][r]), f"case {i} rank {r}"
+                else:
+                    digest = np.frombuffer(hashlib.sha256(blob.tobytes()).digest(), np.uint8)
+                    assert np.array_equal(digest, fx[f"case{i}_dispatch_sha256"][r]), f"case {i} rank {r}"
+            # the checker's ep_combine restores every routed row to [token, k]; the library's combine sums them, so
+            # restore is checked through a one-hot trick: keep only the rows of one k and combine
+            for k in range(K):
+                ys = [torch.zeros((bs, h), dtype=tdt, device=DEV) for _ in range(R)]
+                eo = []
+                for r in range(R):
+                    keep = (outs[r]["assist"][:, 2] == k).view(-1, 1)
+                    rows = outs[r]["expand_x"].view(torch.int16)
+                    eo.append(torch.where(keep, rows, torch.zeros_like(rows)).contiguous())
+                for r in range(R):
+                    assert ep.combine_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
+                                         dtype, w.streams[r]) == 0
+                w.sync()
+                for r in range(R):
+                    restored = ys[r].view(torch.int16).cpu().numpy().view(np.uint16)
+                    if f"case{i}_combine_blobs" in fx:
+                        want = fx[f"case{i}_combine_blobs"][r].view(np.uint16).reshape(bs, K, h)[:, k]
+                    else:
+                        want = xb[r]
+                    # x + 0 == x for every finite checker input (all are small positive normals / subnormals)
+                    assert np.array_equal(restored, want), f"case {i} rank {r} k {k}"
+
+
+def test_repeated_exchanges_reuse_staging_safely():
+    """Back-to-back exchanges with different data, then a different shape: the send half of an exchange must wait
+    for the previous exchange's drains."""
+    R, K, E = 4, 4, 16
+    rng = np.random.default_rng(12)
+    with World(R) as w:
+        for bs, h in ((96, 512), (96, 512), (20, 64), (200, 1024)):
+            for memory in (True, False):
+                ids = rand_ids(rng, R, bs, K, E)
+                xt, xb = rand_x(rng, R, bs, h, ep.DT_BF16)
+                first = run_dispatch(w, memory, xt, ids, bs, h, K, E, ep.DT_BF16)
+                ids2 = rand_ids(rng, R, bs, K, E)
+                # no host synchronisation between the calls of the two exchanges
+                second = run_dispatch(w, memory, xt, ids2, bs, h, K, E, ep.DT_BF16, order=[3, 1, 0, 2])
+                case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16)
+                fn = O.mem_dispatch if memory else O.mvp_dispatch
+                key = "send_counts" if memory else "recv_counts"
+                for r in range(R):
+                    check_rank(first[r], fn(case, r, xb, ids), key)
+                    check_rank(second[r], fn(case, r, xb, ids2), key)
+
+
+def test_exchange_protocol_errors():
+    R, bs, h, K, E = 2, 8, 64, 2, 4
+    rng = np.random.default_rng(3)
+    ids = rand_ids(rng, R, bs, K, E)
+    xt, xb = rand_x(rng, R, bs, h, ep.DT_BF16)
+    with World(R) as w:
+        outs = [alloc_dispatch_outputs(bs, h, K, E, ranks=R) for _ in range(R)]
+        counts = [torch.zeros((E,), dtype=torch.int32, device=DEV) for _ in range(R)]
+        dev_ids = [to_dev(ids[r]) for r in range(R)]
+
+        def call(r, bs_=bs):
+            o = outs[r]
+            return ep.dispatch_memory_v2(xt[r], dev_ids[r], w.comms[r], bs_, h, K, E, o["expand_x"], o["assist"],
+                                         o["token_nums"], counts[r], ep.DT_BF16, w.streams[r])
+        assert call(0) == 0
+        assert call(0) == -4            # the same rank twice in one exchange
+        assert call(1, bs_=bs - 1) == -3   # a rank whose shape disagrees with the exchange in flight
+        assert call(1) == 0
+        w.sync()
+        case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16)
+        for r in range(R):
+            want = O.mem_dispatch(case, r, xb, ids)
+            n = want["rows"]
+            assert np.array_equal(outs[r]["expand_x"].cpu().numpy()[:n], want["expand_x"][:n])
+            assert np.array_equal(counts[r].cpu().numpy(), want["send_counts"])

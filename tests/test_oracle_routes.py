@@ -427,3 +427,39 @@ def test_memory_combine_quantised_input_equals_combine_of_dequantised_rows(orc):
                               expert_scales=w, in_quant=mode, in_scales=d["dyn_scales"])
         assert np.array_equal(got, want)
         assert rows > 0
+
+
+# ---------------------------------------------------------------------------------------------
+# committed checker fixtures (usable where the reference sources are absent)
+# ---------------------------------------------------------------------------------------------
+def test_oracle_matches_committed_checker_fixtures(orc):
+    """tests/golden/checker_fixtures.npz holds the reference checker's ep_dispatch / ep_combine blobs
+    (made by tests/golden/make_checker_fixtures.py); the oracle must reproduce them byte for byte."""
+    import hashlib
+    import os
+    fx = np.load(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "checker_fixtures.npz"))
+    assert int(fx["num_cases"][0]) >= 4
+    for i in range(int(fx["num_cases"][0])):
+        R, bs, h, K, E, dtype = (int(v) for v in fx[f"case{i}_shape"])
+        ids = np.broadcast_to(fx[f"case{i}_ids"], (R, bs, K)).copy()
+        tt, hh = np.meshgrid(np.arange(bs), np.arange(h), indexing="ij")
+        x = np.stack([((0x1000 + r * 0x100 + tt * 0x10 + hh) & 0xffff).astype(np.uint16) for r in range(R)])
+        case = O.Case(R, bs, h, K, E, dtype=dtype)
+        for r in range(R):
+            got = orc.mvp_dispatch(case, r, x, ids)
+            n = got["rows"]
+            assert n == bs * K
+            blob = np.concatenate([got["expand_x"][:n].reshape(-1), np.zeros((R - 1) * n * h * 2, np.uint8),
+                                   got["assist"][:n].reshape(-1).view(np.uint8), got["recv_counts"].view(np.uint8),
+                                   got["expert_token_nums"].view(np.uint8)])
+            if f"case{i}_dispatch_blobs" in fx:
+                assert np.array_equal(blob, fx[f"case{i}_dispatch_blobs"][r])
+                restored = fx[f"case{i}_combine_blobs"][r].view(np.uint16).reshape(bs, K, h)
+                assert np.array_equal(restored, np.broadcast_to(x[r][:, None, :], (bs, K, h)))
+            else:
+                digest = np.frombuffer(hashlib.sha256(blob.tobytes()).digest(), np.uint8)
+                assert np.array_equal(digest, fx[f"case{i}_dispatch_sha256"][r])
+                want = np.broadcast_to(x[r][:, None, :], (bs, K, h))
+                digest = np.frombuffer(hashlib.sha256(np.ascontiguousarray(want).tobytes()).digest(), np.uint8)
+                assert np.array_equal(digest, fx[f"case{i}_combine_sha256"][r])
+    assert int(fx["case3_dispatch_events"][0]) == 4148 and int(fx["case3_combine_events"][0]) == 6164

@@ -12,6 +12,7 @@
 #include "ep_context.h"
 #include "ep_host.h"
 #include "ep_launch.h"
+#include "ep_run_common.h"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -22,55 +23,6 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
 namespace {
 
 constexpr int kOk = TileXR::TILEXR_SUCCESS;
-constexpr int64_t kDefaultWaitUs = 2 * 1000 * 1000;
-constexpr int64_t kWallClockTicksPerUs = 100;      // wall_clock64() counts at 100 MHz on CDNA3/CDNA4
-
-int LaunchStatus(hipError_t err, const char *what)
-{
-    if (err == hipSuccess) {
-        return kOk;
-    }
-    // reference: src/ep/host/ep_kernel_launch.cpp:153,177 reports launch failures on stderr and returns MKIRT
-    std::fprintf(stderr, "tilexr-ep: launching %s failed: %s\n", what, hipGetErrorString(err));
-    return TileXR::TILEXR_ERROR_MKIRT;
-}
-
-// Records the caller's timing events (if any) around one kernel launch.
-template <typename Launch>
-int Timed(EpComm *comm, int kernel, hipStream_t stream, const char *what, Launch launch)
-{
-    hipEvent_t start = comm->timing[kernel][0];
-    hipEvent_t stop = comm->timing[kernel][1];
-    if (start != nullptr && hipEventRecord(start, stream) != hipSuccess) {
-        return TileXR::TILEXR_ERROR_INTERNAL;
-    }
-    const int ret = LaunchStatus(launch(), what);
-    if (ret == kOk && stop != nullptr && hipEventRecord(stop, stream) != hipSuccess) {
-        return TileXR::TILEXR_ERROR_INTERNAL;
-    }
-    return ret;
-}
-
-bool WithinKernelLimits(int64_t bs, int64_t h, int64_t topK, int64_t experts)
-{
-    const int64_t intMax = std::numeric_limits<int32_t>::max();
-    return experts <= kMaxKeys && topK <= kMaxTopK && bs <= intMax / topK && h <= intMax / 2 && bs * topK <= intMax / 4;
-}
-
-CountScratch CarveCountScratch(void *base, const CountScratchLayout &plan, bool expertHist)
-{
-    auto at = [base](int64_t off) { return reinterpret_cast<int32_t *>(static_cast<char *>(base) + off); };
-    CountScratch s {};
-    s.ticket = static_cast<uint32_t *>(base);
-    s.localRank = at(plan.localRankOff);
-    s.chunkHist = at(plan.chunkHistOff);
-    s.chunkExpHist = expertHist ? at(plan.chunkExpHistOff) : nullptr;
-    s.keyOffset = at(plan.keyOffsetOff);
-    s.keyKept = at(plan.keyKeptOff);
-    s.expertTotal = at(plan.expertTotalOff);
-    return s;
-}
-
 // ---------------------------------------------------------------------------------------------------------
 // one rank per device: rows go straight from x to expandXOut
 // ---------------------------------------------------------------------------------------------------------

@@ -24,19 +24,18 @@ void ReleaseWorld(EpWorld *world)
     if (world->flagArea != nullptr) {
         (void)hipFree(world->flagArea);
     }
-    for (auto *list : {&world->stageRows, &world->stageAux, &world->combineSlots, &world->combineMeta}) {
-        for (DeviceBuffer &b : *list) {
-            b.Release();
-        }
+    for (DeviceBuffer *b : {&world->stageRows, &world->stageAux, &world->stageCounts, &world->combineSlots,
+             &world->combineMeta}) {
+        b->Release();
     }
-    for (PendingDispatch &p : world->pendingDispatch) {
-        if (p.sent != nullptr) {
-            (void)hipEventDestroy(p.sent);
-        }
-    }
-    for (PendingCombine &p : world->pendingCombine) {
-        if (p.sent != nullptr) {
-            (void)hipEventDestroy(p.sent);
+    for (auto *list : {&world->dispatchEvents, &world->combineEvents}) {
+        for (RankEvents &e : *list) {
+            if (e.sent != nullptr) {
+                (void)hipEventDestroy(e.sent);
+            }
+            if (e.drained != nullptr) {
+                (void)hipEventDestroy(e.drained);
+            }
         }
     }
     delete world;
@@ -49,10 +48,8 @@ EpWorld *CreateWorld(int rankSize)
     world->comms.assign(static_cast<size_t>(rankSize), nullptr);
     world->pendingDispatch.resize(static_cast<size_t>(rankSize));
     world->pendingCombine.resize(static_cast<size_t>(rankSize));
-    world->stageRows.resize(static_cast<size_t>(rankSize));
-    world->stageAux.resize(static_cast<size_t>(rankSize));
-    world->combineSlots.resize(static_cast<size_t>(rankSize));
-    world->combineMeta.resize(static_cast<size_t>(rankSize));
+    world->dispatchEvents.resize(static_cast<size_t>(rankSize));
+    world->combineEvents.resize(static_cast<size_t>(rankSize));
     int device = -1;
     if (hipGetDevice(&device) == hipSuccess) {
         world->device = device;
@@ -179,6 +176,7 @@ int TileXRCommDestroy(TileXRCommPtr comm)
     }
     c->dispatchScratch.Release();
     c->combineScratch.Release();
+    c->drainScratch.Release();
     if (c->dev != nullptr) {
         (void)hipFree(c->dev);
     }

@@ -35,20 +35,38 @@ struct DeviceBuffer {
     void Release();
 };
 
+// What all ranks of one exchange must agree on.
+struct ExchangeShape {
+    int64_t bs = 0;
+    int64_t h = 0;
+    int64_t topK = 0;
+    int64_t experts = 0;
+    int64_t quantMode = 0;
+    int dtype = 0;
+    int outDtype = 0;
+    bool memoryRoute = false;
+    bool operator==(const ExchangeShape &o) const
+    {
+        return bs == o.bs && h == o.h && topK == o.topK && experts == o.experts && quantMode == o.quantMode &&
+            dtype == o.dtype && outDtype == o.outDtype && memoryRoute == o.memoryRoute;
+    }
+};
+
 struct PendingDispatch {
     bool present = false;
     EpDispatchParams params {};
-    bool memoryRoute = false;
-    int64_t magic = 0;
-    hipEvent_t sent = nullptr;
 };
 
 struct PendingCombine {
     bool present = false;
     EpCombineParams params {};
-    bool memoryRoute = false;
-    int64_t magic = 0;
-    hipEvent_t sent = nullptr;
+};
+
+// Per-rank events of the two-half exchange; created on first use, `armed` once recorded.
+struct RankEvents {
+    hipEvent_t sent = nullptr;       // this rank's send half is enqueued
+    hipEvent_t drained = nullptr;    // this rank's drain half is enqueued (staging may be reused after it)
+    bool drainedArmed = false;
 };
 
 struct EpComm;
@@ -63,12 +81,18 @@ struct EpWorld {
     uint8_t *flagArea = nullptr;
     std::mutex mu;
     // multi-rank exchange (rankSize > 1)
+    ExchangeShape dispatchShape {};
+    ExchangeShape combineShape {};
     std::vector<PendingDispatch> pendingDispatch;
     std::vector<PendingCombine> pendingCombine;
-    std::vector<DeviceBuffer> stageRows;      // per source rank: rows grouped by key
-    std::vector<DeviceBuffer> stageAux;       // per source rank: assist tuples + per-row scales
-    std::vector<DeviceBuffer> combineSlots;   // per source rank: [bs, topK] rows returned by the expert ranks
-    std::vector<DeviceBuffer> combineMeta;    // per source rank: [bs, topK] tagged origin of each slot
+    std::vector<RankEvents> dispatchEvents;
+    std::vector<RankEvents> combineEvents;
+    uint64_t combineEpoch = 0;
+    DeviceBuffer stageRows;       // [R] payload rows grouped by key
+    DeviceBuffer stageAux;        // [R] assist tuples + per-row scales
+    DeviceBuffer stageCounts;     // [R] keyOffset + expertTotal
+    DeviceBuffer combineSlots;    // [R] [bs, topK] rows returned by the expert ranks
+    DeviceBuffer combineMeta;     // [R] tagged slot table + order keys
 };
 
 struct EpComm {
@@ -80,6 +104,7 @@ struct EpComm {
     std::atomic<int64_t> nextMagic {1};
     DeviceBuffer dispatchScratch;
     DeviceBuffer combineScratch;
+    DeviceBuffer drainScratch;
     hipEvent_t timing[5][2] = {};     // optional (start, stop) pairs around each kernel, see tilexr_ep.h
     std::mutex mu;
 };

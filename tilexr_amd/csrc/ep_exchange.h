@@ -1,0 +1,88 @@
+// Launch interface of the exchange kernels used when several logical ranks share the device (rankSize > 1).
+//
+// A multi-rank dispatch is two halves.  The source rank's call groups its rows by destination into a staging area
+// (the same count / place / scatter kernels as the single-rank path, writing to staging instead of expandXOut).
+// Once every rank has sent, each destination rank's outputs are assembled ("drained") from all staging areas:
+//   plan   per-segment counts -> count outputs + exclusive offsets, one workgroup
+//   copy   one workgroup per output row: locate its segment, copy row, assist tuple and scales
+// A multi-rank combine is the transpose: every expert rank returns its rows to per-(token, k) slots of the source
+// ranks ("return"), then each source rank runs the ordinary reduce kernel over its slots.
+#ifndef TILEXR_AMD_EP_EXCHANGE_H
+#define TILEXR_AMD_EP_EXCHANGE_H
+
+#include <cstdint>
+
+#include <hip/hip_runtime_api.h>
+
+namespace TileXREp {
+
+// Staging of one world: every per-source area has the same size, so kernels address areas arithmetically.
+struct StageLayout {
+    char *rows;              // [R] x rowsStride bytes: payload rows grouped by key
+    int64_t rowsStride;
+    char *aux;               // [R] x auxStride bytes: assist tuples [n,4] int32, then per-row scales
+    int64_t auxStride;
+    int64_t scalesOffset;    // offset of the scales inside an aux area
+    int32_t *counts;         // [R] x countsStride ints: keyOffset[numKeys+1], expertTotal[E]
+    int64_t countsStride;
+    int64_t expertTotalOffset;   // in ints
+};
+
+struct DrainPlanLaunch {
+    StageLayout stage;
+    int rankSize;
+    int dstRank;
+    int localExperts;
+    bool memoryRoute;        // segments (localExpert, src) with inclusive-sum counts, else (src) with plain counts
+    int32_t *planOffsets;    // [numSeg + 1] exclusive offsets (scratch of the destination rank)
+    int32_t *countsOut;
+    int32_t *tpCountsOut;    // optional mirror of countsOut (MVP route)
+    int64_t *expertTokenNumsOut;
+    int tokenNumsType;
+    hipStream_t stream;
+};
+
+struct DrainCopyLaunch {
+    StageLayout stage;
+    int rankSize;
+    int dstRank;
+    int localExperts;
+    bool memoryRoute;
+    const int32_t *planOffsets;
+    int64_t maxRows;
+    int64_t rowBytes;
+    int64_t scaleBytesPerRow;
+    void *expandXOut;
+    int32_t *assistOut;
+    void *scalesOut;
+    hipStream_t stream;
+};
+
+struct ReturnRowsLaunch {
+    const void *expertOut;
+    const int32_t *assist;
+    const int32_t *counts;
+    int64_t numCounts;
+    bool memoryRoute;
+    int64_t maxCountPerEntry;
+    int64_t maxRows;
+    int64_t rowBytes;
+    int rankSize;
+    int expertRank;          // the calling rank
+    int64_t bs;
+    int64_t topK;
+    uint64_t epoch;
+    char *slots;             // [R] x slotsStride: rows at slot token*topK + k of the source rank
+    int64_t slotsStride;
+    uint64_t *meta;          // [R] x metaStride words: inverse (epoch << 32 | slot), then order keys
+    int64_t metaStride;      // in words
+    hipStream_t stream;
+};
+
+hipError_t LaunchDrainPlan(const DrainPlanLaunch &l);
+hipError_t LaunchDrainCopy(const DrainCopyLaunch &l);
+hipError_t LaunchReturnRows(const ReturnRowsLaunch &l);
+
+} // namespace TileXREp
+
+#endif // TILEXR_AMD_EP_EXCHANGE_H

@@ -1,4 +1,5 @@
-// Kernel launch interface between the host orchestration (api.cpp) and the HIP kernels (ep_kernels.hip).
+// Kernel launch interface between the host orchestration (api.cpp, multi_rank.cpp) and the HIP kernels (ep_count.hip,
+// ep_scatter.hip, ep_reduce.hip).
 //
 // The data path of one dispatch is three launches on the caller's stream:
 //   count   per-chunk stable rank of every route within its key + per-chunk key histogram; the last workgroup
@@ -120,6 +121,7 @@ struct ReduceLaunch {
     const uint64_t *inverseTagged;   // either this (with epoch) ...
     uint64_t epoch;
     const int32_t *rowIndexMap;      // ... or a plain row map (-1 = none)
+    const uint64_t *orderKeys;       // optional, per-add kind: rows are summed in ascending orderKeys[row]
     const float *expertScales;       // optional [bs, topK]
     const uint8_t *tokenMask;        // optional [bs]
     const void *sharedExpertX;       // optional [bs, h]

@@ -31,6 +31,7 @@ struct ReduceArgs {
     const uint64_t *inverseTagged;
     uint64_t epoch;
     const int32_t *rowIndexMap;
+    const uint64_t *orderKeys;
     const float *expertScales;
     const uint8_t *tokenMask;
     const void *sharedExpertX;
@@ -76,9 +77,23 @@ __device__ bool WaitTile(const ReduceArgs &a, int row)
     }
 }
 
-// Insertion sort of row indices, ascending, absent rows (-1) last.  K is small.
-__device__ void SortRows(int *rows, int k)
+// Insertion sort of row indices, absent rows (-1) last.  The order is the row index itself, or -- when rows come
+// from several expert ranks -- the (expert rank, row) key recorded for each slot.  K is small.
+__device__ void SortRows(int *rows, int k, const uint64_t *orderKeys)
 {
+    if (orderKeys != nullptr) {
+        for (int i = 1; i < k; ++i) {
+            const int v = rows[i];
+            const uint64_t kv = v < 0 ? ~0ull : orderKeys[v];
+            int j = i - 1;
+            while (j >= 0 && (rows[j] < 0 ? ~0ull : orderKeys[rows[j]]) > kv) {
+                rows[j + 1] = rows[j];
+                --j;
+            }
+            rows[j + 1] = v;
+        }
+        return;
+    }
     for (int i = 1; i < k; ++i) {
         const int v = rows[i];
         const unsigned kv = static_cast<unsigned>(v);      // -1 becomes the largest key
@@ -132,7 +147,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
         __syncthreads();
         if (KIND == kReducePerAdd) {
             if (lane == 0) {
-                SortRows(s_row[tg], a.topK);
+                SortRows(s_row[tg], a.topK, a.orderKeys);
             }
             __syncthreads();
         }
@@ -271,7 +286,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
         __syncthreads();
         if (kind == kReducePerAdd) {
             if (tid == 0) {
-                SortRows(s_row, a.topK);
+                SortRows(s_row, a.topK, a.orderKeys);
             }
             __syncthreads();
         }
@@ -391,6 +406,7 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     a.inverseTagged = l.inverseTagged;
     a.epoch = l.epoch;
     a.rowIndexMap = l.rowIndexMap;
+    a.orderKeys = l.orderKeys;
     a.expertScales = l.expertScales;
     a.tokenMask = l.tokenMask;
     a.sharedExpertX = l.sharedExpertX;
