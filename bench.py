@@ -21,6 +21,19 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 
 
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch from the committed hardware-counter summary (profiles/hbm_traffic_<workload>.txt, lines
+    `<kernel>_bytes_per_launch = N`), or None when no summary covers this workload."""
+    path = os.path.join(ROOT, "profiles", f"hbm_traffic_{workload}.txt")
+    if not os.path.exists(path):
+        return None
+    for line in open(path):
+        parts = line.split("=")
+        if len(parts) == 2 and parts[0].strip() == f"{kernel}_bytes_per_launch":
+            return int(float(parts[1].strip()))
+    return None
+
+
 def parse():
     p = argparse.ArgumentParser()
     p.add_argument("--gpus", type=int, default=1)
@@ -30,6 +43,11 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-kernel-events", action="store_true",
                    help="do not record per-kernel HIP events inside the timed region")
+    p.add_argument("--event-stride", type=int, default=10,
+                   help="record the per-kernel events on every N-th timed step")
+    p.add_argument("--calibrate-copy", action="store_true",
+                   help="also launch a plain 256 MiB read + 256 MiB write kernel before the warm-up, as the known-size "
+                        "yardstick for hardware-counter runs")
     return p.parse_args()
 
 
@@ -110,30 +128,43 @@ def main():
                                       expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
                                       row_index_map=row_map), "combine")
 
+    if args.calibrate_copy:
+        src = torch.zeros((64 << 20,), dtype=torch.int32, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst)      # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst
+
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()
     kept_rows = int(send_counts[-1].item())
     dispatch_bytes, combine_bytes = workloads.algorithmic_bytes(w, kept_rows, inverse_index=True)
 
-    # per-kernel events: one (start, stop) pair per step for the scatter and the reduce kernel
-    pairs = []
+    # Per-kernel HIP events inside the timed region, on a sample of the steps only: an event record between two
+    # kernels holds the queue for about 5 us on this GPU, so bracketing both kernels on every step would add about
+    # 20 us to a 200 us step.  Every `stride`-th step carries a (start, stop) pair around the scatter and the
+    # reduce kernel; the library records them on the stream the kernels are launched on.
     use_events = not args.no_kernel_events
-    if use_events:
-        pairs = [[(ep.HipEvent(timing=True), ep.HipEvent(timing=True)) for _ in range(args.steps)] for _ in range(2)]
+    stride = max(1, args.event_stride)
+    sampled = [i for i in range(args.steps) if i % stride == 0] if use_events else []
+    pairs = {i: [(ep.HipEvent(timing=True), ep.HipEvent(timing=True)) for _ in range(2)] for i in sampled}
     d_ev = [ep.HipEvent(timing=True) for _ in range(3)]
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(args.steps):
-        if use_events:
-            ep.set_kernel_timing_events(comm, ep.K_SCATTER, *pairs[0][i])
-            ep.set_kernel_timing_events(comm, ep.K_REDUCE, *pairs[1][i])
-        step()
+        if i in pairs:
+            ep.set_kernel_timing_events(comm, ep.K_SCATTER, *pairs[i][0])
+            ep.set_kernel_timing_events(comm, ep.K_REDUCE, *pairs[i][1])
+            step()
+            ep.set_kernel_timing_events(comm, ep.K_SCATTER, None, None)
+            ep.set_kernel_timing_events(comm, ep.K_REDUCE, None, None)
+        else:
+            step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
-    for k in (ep.K_SCATTER, ep.K_REDUCE):
-        ep.set_kernel_timing_events(comm, k, None, None)
 
     # split of one step into its two calls (outside the timed region)
     d_ev[0].record(stream)
@@ -155,16 +186,17 @@ def main():
     roofline = None
     kernels = {}
     if use_events:
-        for name, plist, nbytes in (("scatter", pairs[0], dispatch_bytes), ("reduce", pairs[1], combine_bytes)):
-            times = sorted(a.elapsed_ms(b) * 1e3 for a, b in plist)
+        for which, (name, nbytes) in enumerate((("scatter", dispatch_bytes), ("reduce", combine_bytes))):
+            times = sorted(pairs[i][which][0].elapsed_ms(pairs[i][which][1]) * 1e3 for i in sampled)
             avg = sum(times) / len(times)
             kernels[name] = {"avg_us": round(avg, 2), "min_us": round(times[0], 2), "p50_us": round(times[len(times) // 2], 2),
-                             "max_us": round(times[-1], 2), "algorithmic_bytes": nbytes,
+                             "max_us": round(times[-1], 2), "launches_timed": len(times), "algorithmic_bytes": nbytes,
                              "achieved_GBps": round(nbytes / (avg * 1e-6) / 1e9, 1)}
         dom = "scatter" if kernels["scatter"]["avg_us"] >= kernels["reduce"]["avg_us"] else "reduce"
         roofline = {"bound": "hbm", "kernel": "ep_scatter_vec_kernel" if dom == "scatter" else "ep_reduce_vec_kernel",
                     "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4), "traffic": None,
+                    "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4),
+                    "traffic": measured_traffic(w.name, dom),
                     "avg_launch_us": kernels[dom]["avg_us"], "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
 
     result = {

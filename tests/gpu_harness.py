@@ -8,8 +8,20 @@ from tilexr_amd import ep
 DEV = "cuda:0"
 
 
+_KEEP = []      # device copies made by to_dev(): kernels on side streams may still read them after the call returns
+
+
 def to_dev(a):
-    return None if a is None else torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    if a is None:
+        return None
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(DEV)
+    _KEEP.append(t)
+    return t
+
+
+def release_device_copies():
+    torch.cuda.synchronize()
+    _KEEP.clear()
 
 
 def bits16(t):
@@ -26,7 +38,7 @@ class Session:
         self.stream = torch.cuda.Stream()
 
     def close(self):
-        torch.cuda.synchronize()
+        release_device_copies()
         self.comm.destroy()
 
     def __enter__(self):

@@ -11,7 +11,7 @@ import numpy as np
 import pytest
 import torch
 
-from gpu_harness import DEV, alloc_dispatch_outputs, bits16, to_dev
+from gpu_harness import DEV, alloc_dispatch_outputs, bits16, release_device_copies, to_dev
 from oracle import ep as O
 from tilexr_amd import ep
 
@@ -35,7 +35,7 @@ class World:
         return self
 
     def __exit__(self, *exc):
-        torch.cuda.synchronize()
+        release_device_copies()
         for c in self.comms:
             c.destroy()
 

@@ -26,7 +26,7 @@ def ids_for(rng, bs, K, E, invalid=0.0):
 def x_for(rng, bs, h, dtype, scale=1.0):
     f = (rng.standard_normal((bs, h)) * scale).astype(np.float32)
     t = torch.from_numpy(f).to(torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16)
-    return t, bits16(t)
+    return t.to(DEV), bits16(t)      # the device copy stays alive in the caller's scope while kernels read it
 
 
 def check_dispatch(got, want, rows_key="rows"):
@@ -59,7 +59,7 @@ def test_memory_dispatch_matches_oracle(shape, dtype):
             for nums_type in (0, 1):
                 out = alloc_dispatch_outputs(bs, h, K, E)
                 counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
-                st = ep.dispatch_memory_v2(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                st = ep.dispatch_memory_v2(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
                                            out["token_nums"], counts, dtype, s.stream, active_mask=to_dev(mask),
                                            active_mask_type=mask_type, token_nums_type=nums_type)
                 assert st == 0
@@ -87,7 +87,7 @@ def test_mvp_dispatch_matches_oracle(shape):
                     counts = torch.full((1,), -1, dtype=torch.int32, device=DEV)
                     tp_counts = torch.full((1,), -1, dtype=torch.int32, device=DEV)
                     st = ep.dispatch_v2(
-                        xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"], out["token_nums"],
+                        xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"], out["token_nums"],
                         counts, ep.DT_FP16 if quant == ep.Q_NONE else ep.DT_INT8, s.stream,
                         scales=to_dev(static) if quant == ep.Q_STATIC_INT8 else None,
                         active_mask=to_dev(mask) if use_mask else None, quant_mode=quant, token_nums_type=nums_type,
@@ -116,7 +116,7 @@ def test_simple_entry_points():
             out = alloc_dispatch_outputs(bs, h, K, E)
             counts = torch.zeros((E if memory else 1,), dtype=torch.int32, device=DEV)
             fn = ep.dispatch_memory if memory else ep.dispatch
-            assert fn(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["token_nums"], counts,
+            assert fn(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["token_nums"], counts,
                       out["assist"], ep.DT_BF16, s.stream) == 0
             y = torch.zeros((bs, h), dtype=torch.bfloat16, device=DEV)
             fnc = ep.combine_memory if memory else ep.combine
@@ -151,11 +151,11 @@ def test_quantised_dispatch_matches_oracle(shape, dtype, quant, fp8):
     xb[0, :] = 0                       # an all-zero row
     if h >= 64:
         xb[1, 32:64] = 0               # an all-zero block
-    xt = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16)
+    xt = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16).to(DEV)
     with Session() as s:
         out = alloc_dispatch_outputs(bs, h, K, E, quant=quant)
         counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
-        st, _ = ep.dispatch_memory_ex(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+        st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
                                       out["token_nums"], counts, dtype, s.stream, quant_mode=quant,
                                       dynamic_scales=out["scales"], expand_x_dtype=fp8, row_index_map=out["row_map"])
         assert st == 0
@@ -175,7 +175,7 @@ def test_quantised_dispatch_matches_oracle(shape, dtype, quant, fp8):
         if quant == ep.Q_MXFP8:
             # the reference API takes the same mode through DispatchMemoryV2
             out2 = alloc_dispatch_outputs(bs, h, K, E, quant=quant)
-            st = ep.dispatch_memory_v2(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out2["expand_x"], out2["assist"],
+            st = ep.dispatch_memory_v2(xt, to_dev(ids), s.comm, bs, h, K, E, out2["expand_x"], out2["assist"],
                                        out2["token_nums"], counts, dtype, s.stream, quant_mode=4,
                                        dynamic_scales=out2["scales"], expand_x_dtype=fp8)
             assert st == 0
@@ -193,7 +193,7 @@ def test_capacity_drop_matches_oracle():
     with Session() as s:
         out = alloc_dispatch_outputs(bs, h, K, E)
         counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
-        st, _ = ep.dispatch_memory_ex(xt.to(DEV), to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+        st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
                                       out["token_nums"], counts, ep.DT_BF16, s.stream, expert_capacity=cap,
                                       row_index_map=out["row_map"])
         assert st == 0

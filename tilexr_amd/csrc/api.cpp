@@ -97,18 +97,26 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     place.numTiles = p.tileFlagsOut != nullptr ? (n + p.tileRows - 1) / p.tileRows : 0;
     place.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
     place.stream = stream;
-    ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
-    if (ret != kOk) {
-        return ret;
-    }
-    if (p.metaReadyEvent != nullptr &&
-        hipEventRecord(static_cast<hipEvent_t>(p.metaReadyEvent), stream) != hipSuccess) {
-        return TileXR::TILEXR_ERROR_INTERNAL;
+    // The scatter kernel can resolve the rows of its own tokens; a separate launch is only needed when something
+    // has to be complete before the first row lands (tile flags reset, assist tuples behind metaReadyEvent).
+    const bool separatePlace = p.tileFlagsOut != nullptr || p.metaReadyEvent != nullptr;
+    if (separatePlace) {
+        ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
+        if (ret != kOk) {
+            return ret;
+        }
+        if (p.metaReadyEvent != nullptr &&
+            hipEventRecord(static_cast<hipEvent_t>(p.metaReadyEvent), stream) != hipSuccess) {
+            return TileXR::TILEXR_ERROR_INTERNAL;
+        }
+    } else {
+        place.rowOf = p.rowIndexMapOut;      // only written when the caller asked for the map
     }
 
     ScatterLaunch scatter {};
     scatter.x = p.x;
     scatter.rowOf = rowOf;
+    scatter.fusedPlace = separatePlace ? nullptr : &place;
     scatter.bs = p.bs;
     scatter.h = p.h;
     scatter.topK = p.topK;

@@ -10,6 +10,7 @@
 #include "ep_block_scan.cuh"
 #include "ep_kernel_common.cuh"
 #include "ep_launch.h"
+#include "ep_place.cuh"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -268,23 +269,12 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
 }
 
 // -------------------------------------------------------------------------------------------------------------
-// place: destination row of every route + assist tuple + inverse map + tile-flag reset.
-//   row   = keyOffset[key] + (rank of the route within its key), routes at or beyond `capacity` get none
-//   tuple = {srcRank, token, k, expert id} (reference: src/ep/common/ep_window.h:47-52,
-//           tilexr_ep_dispatch_memory_kernel.h:1240-1258)
+// place (stand-alone): destination row of every route + assist tuple + inverse map + tile-flag reset.  Used when
+// something must be complete before the scatter starts (tile flags reset, a metadata-ready event) or when the
+// rows go to a staging area; otherwise the scatter kernel resolves the rows of its own tokens (ep_place.cuh).
 // -------------------------------------------------------------------------------------------------------------
 struct RoutePlaceArgs {
-    const int32_t *ids;
-    int n;
-    int topK;
-    int keyDiv;
-    int numKeys;
-    int capacity;
-    CountScratch s;
-    int32_t srcRank;
-    int32_t expertIdBias;
-    int32_t *rowOf;
-    int32_t *assist;
+    PlaceArgs p;
     uint64_t *tileFlags;
     int numTiles;
     uint64_t epoch;
@@ -298,25 +288,9 @@ __global__ __launch_bounds__(kThreads) void ep_route_place_kernel(RoutePlaceArgs
             a.tileFlags[f] = a.epoch << 32;
         }
     }
-    if (i >= a.n) {
-        return;
+    if (i < a.p.n) {
+        PlaceRoute(a.p, i);
     }
-    const int lr = a.s.localRank[i];
-    int row = -1;
-    if (lr >= 0) {
-        const int e = a.ids[i];
-        const int key = e / a.keyDiv;
-        const int within = a.s.chunkHist[static_cast<int64_t>(i / kChunkRoutes) * a.numKeys + key] + lr;
-        if (a.capacity <= 0 || within < a.capacity) {
-            row = a.s.keyOffset[key] + within;
-            int32_t *tuple = a.assist + static_cast<int64_t>(row) * 4;
-            tuple[0] = a.srcRank;
-            tuple[1] = i / a.topK;
-            tuple[2] = i % a.topK;
-            tuple[3] = e + a.expertIdBias;
-        }
-    }
-    a.rowOf[i] = row;
 }
 
 // -------------------------------------------------------------------------------------------------------------
@@ -435,22 +409,12 @@ hipError_t LaunchRouteCount(const RouteCountLaunch &l)
 hipError_t LaunchRoutePlace(const RoutePlaceLaunch &l)
 {
     RoutePlaceArgs a {};
-    a.ids = l.ids;
-    a.n = static_cast<int>(l.bs * l.topK);
-    a.topK = static_cast<int>(l.topK);
-    a.keyDiv = static_cast<int>(l.keyDiv);
-    a.numKeys = static_cast<int>(l.numKeys);
-    a.capacity = static_cast<int>(l.capacity);
-    a.s = l.scratch;
-    a.srcRank = l.srcRank;
-    a.expertIdBias = l.expertIdBias;
-    a.rowOf = l.rowOf;
-    a.assist = l.assist;
+    a.p = MakePlaceArgs(l);
     a.tileFlags = l.tileFlags;
     a.numTiles = static_cast<int>(l.numTiles);
     a.epoch = l.epoch;
-    const int grid = (a.n + kThreads - 1) / kThreads;
-    hipLaunchKernelGGL(ep_route_place_kernel, dim3(grid), dim3(kThreads), 0, l.stream, a);
+    const int grid = (a.p.n + kThreads - 1) / kThreads;
+    hipLaunchKernelGGL(ep_route_place_kernel, dim3(grid > 0 ? grid : 1), dim3(kThreads), 0, l.stream, a);
     return hipGetLastError();
 }
 

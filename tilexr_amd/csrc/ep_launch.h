@@ -4,7 +4,8 @@
 // The data path of one dispatch is three launches on the caller's stream:
 //   count   per-chunk stable rank of every route within its key + per-chunk key histogram; the last workgroup
 //           to finish scans the histograms into per-chunk bases, per-key offsets and the count outputs
-//   place   destination row of every route, assist tuples, inverse row map, tile-flag reset
+//   place   destination row of every route, assist tuples, inverse row map, tile-flag reset (folded into the
+//           scatter launch when nothing has to be complete before the scatter starts)
 //   scatter token rows read once and written to their topK destination rows (optionally quantised)
 // and of one combine two launches:
 //   invert  (skipped when the caller supplies the row map) row -> (token, k) inverse from the assist tuples
@@ -80,7 +81,8 @@ struct RoutePlaceLaunch {
 
 struct ScatterLaunch {
     const void *x;
-    const int32_t *rowOf;
+    const int32_t *rowOf;            // rows resolved by an earlier place launch, unless ...
+    const RoutePlaceLaunch *fusedPlace;  // ... this is set: the scatter resolves them itself (rowOf output optional)
     int64_t bs;
     int64_t h;
     int64_t topK;

@@ -17,6 +17,7 @@
 #include "ep_kernel_common.cuh"
 #include "ep_launch.h"
 #include "ep_numerics.cuh"
+#include "ep_place.cuh"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -25,6 +26,7 @@ namespace {
 struct ScatterArgs {
     const void *x;
     const int32_t *rowOf;
+    PlaceArgs place;             // place.ids != nullptr: resolve the rows here instead of reading rowOf
     int bs;
     int h;
     int topK;
@@ -34,6 +36,11 @@ struct ScatterArgs {
     uint64_t *tileFlags;
     int tileRows;
 };
+
+__device__ __forceinline__ int RowOfRoute(const ScatterArgs &a, int route)
+{
+    return a.place.ids != nullptr ? PlaceRoute(a.place, route) : a.rowOf[route];
+}
 
 template <int G>
 __device__ __forceinline__ float GroupMax(float v, float *red, int lane)
@@ -80,7 +87,7 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
     const int vecs = a.h / 8;
 
     for (int k = lane; k < a.topK; k += G) {
-        s_pos[tg][k] = tokOk ? a.rowOf[static_cast<int64_t>(token) * a.topK + k] : -1;
+        s_pos[tg][k] = tokOk ? RowOfRoute(a, token * a.topK + k) : -1;
     }
     const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.x) +
         static_cast<int64_t>(tokOk ? token : 0) * a.h * 2);
@@ -222,7 +229,7 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_generic_kernel(ScatterArg
     const int token = blockIdx.x;
     const int tid = threadIdx.x;
     for (int k = tid; k < a.topK; k += kThreads) {
-        s_pos[k] = a.rowOf[static_cast<int64_t>(token) * a.topK + k];
+        s_pos[k] = RowOfRoute(a, token * a.topK + k);
     }
     const uint16_t *src = static_cast<const uint16_t *>(a.x) + static_cast<int64_t>(token) * a.h;
     float rowScale = 1.0f;
@@ -358,6 +365,9 @@ hipError_t LaunchScatter(const ScatterLaunch &l)
     ScatterArgs a {};
     a.x = l.x;
     a.rowOf = l.rowOf;
+    if (l.fusedPlace != nullptr) {
+        a.place = MakePlaceArgs(*l.fusedPlace);
+    }
     a.bs = static_cast<int>(l.bs);
     a.h = static_cast<int>(l.h);
     a.topK = static_cast<int>(l.topK);
