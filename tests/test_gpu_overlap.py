@@ -1,0 +1,109 @@
+"""Tile readiness flags: combine on one stream consuming rows while dispatch on another stream is still writing them,
+and the bounded wait that ends a combine whose producer never shows up.
+
+No kernel here is allowed to wait forever: the flag wait has a wall-clock bound and reports through a device word.
+"""
+import numpy as np
+import pytest
+import torch
+
+from gpu_harness import DEV, Session, alloc_dispatch_outputs, bits16, to_dev
+from oracle import ep as O
+from tilexr_amd import ep
+
+pytestmark = pytest.mark.gpu
+
+
+def routing(rng, bs, K, E):
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(bs)]).astype(np.int32)
+    w = rng.random((bs, K)).astype(np.float32)
+    return ids, w
+
+
+@pytest.mark.parametrize("shape,tile_rows", [((64, 256, 4, 16), 8), ((2048, 2048, 8, 64), 128), ((777, 1024, 6, 32), 100)])
+def test_combine_overlapped_with_dispatch_through_tile_flags(shape, tile_rows):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape))
+    n = bs * K
+    tiles = (n + tile_rows - 1) // tile_rows
+    with Session() as s:
+        side = torch.cuda.Stream()
+        flags = torch.zeros((tiles,), dtype=torch.int64, device=DEV)     # never cleared between rounds
+        status = torch.zeros((1,), dtype=torch.int32, device=DEV)
+        meta_ready = ep.HipEvent()
+        epochs = []
+        for round_ in range(4):
+            ids, w = routing(rng, bs, K, E)
+            x = torch.from_numpy(rng.standard_normal((bs, h)).astype(np.float32)).to(torch.bfloat16)
+            xb = bits16(x)
+            d_x, d_ids, d_w = x.to(DEV), to_dev(ids), to_dev(w)
+            out = alloc_dispatch_outputs(bs, h, K, E)
+            counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+            y = torch.full((bs, h), 3.0, dtype=torch.bfloat16, device=DEV)
+            torch.cuda.synchronize()
+            st, epoch = ep.dispatch_memory_ex(d_x, d_ids, s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                              out["token_nums"], counts, ep.DT_BF16, s.stream,
+                                              row_index_map=out["row_map"], tile_flags=flags, tile_rows=tile_rows,
+                                              meta_ready_event=meta_ready.value)
+            assert st == 0 and epoch > 0
+            epochs.append(epoch)
+            # the consumer may start once counts, row map and the re-armed flag words are enqueued
+            meta_ready.wait_on(side)
+            st = ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, side,
+                                      expert_scales=d_w, row_index_map=out["row_map"], tile_flags=flags,
+                                      tile_rows=tile_rows, flag_epoch=epoch, wait_timeout_us=5_000_000,
+                                      device_status=status)
+            assert st == 0
+            s.sync()
+            side.synchronize()
+            assert status.item() == 0
+            case = O.Case(1, bs, h, K, E, token_nums_type=1)
+            want = O.mem_dispatch(case, 0, xb[None], ids[None])
+            assert np.array_equal(out["expand_x"].cpu().numpy(), want["expand_x"])
+            wy = O.mem_combine(case, 0, want["expand_x"].view(np.uint16)[None], want["assist"][None],
+                               want["send_counts"][None], expert_scales=w)
+            assert np.array_equal(bits16(y), wy)
+            # every tile ends at (epoch << 32) | rows in the tile
+            f = flags.cpu().numpy().astype(np.uint64)
+            rows_in_tile = np.minimum(tile_rows, n - np.arange(tiles) * tile_rows)
+            assert np.array_equal(f >> np.uint64(32), np.full(tiles, epoch, np.uint64))
+            assert np.array_equal(f & np.uint64(0xffffffff), rows_in_tile.astype(np.uint64))
+        assert epochs == sorted(set(epochs))
+        meta_ready.destroy()
+
+
+def test_flag_wait_expires_instead_of_hanging():
+    bs, h, K, E = 256, 512, 4, 16
+    rng = np.random.default_rng(9)
+    ids, w = routing(rng, bs, K, E)
+    x = torch.from_numpy(rng.standard_normal((bs, h)).astype(np.float32)).to(torch.bfloat16)
+    with Session() as s:
+        d_x, d_ids = x.to(DEV), to_dev(ids)
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        st, _ = ep.dispatch_memory_ex(d_x, d_ids, s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, ep.DT_BF16, s.stream, row_index_map=out["row_map"])
+        assert st == 0
+        s.sync()
+        tile_rows = 32
+        flags = torch.zeros(((bs * K + tile_rows - 1) // tile_rows,), dtype=torch.int64, device=DEV)   # nobody sets them
+        status = torch.zeros((1,), dtype=torch.int32, device=DEV)
+        y = torch.full((bs, h), 3.0, dtype=torch.bfloat16, device=DEV)
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        with torch.cuda.stream(s.stream):
+            start.record()
+            st = ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16,
+                                      s.stream, row_index_map=out["row_map"], tile_flags=flags, tile_rows=tile_rows,
+                                      flag_epoch=4242, wait_timeout_us=2000, device_status=status)
+            stop.record()
+        assert st == 0
+        s.sync()
+        assert status.item() == 1                       # reported, not hung
+        assert start.elapsed_time(stop) < 500.0          # milliseconds: about one timeout, not one per tile
+        # rows whose tile never became ready contribute nothing
+        assert np.all(bits16(y) == 0)
+    # a bad timeout is rejected on the host
+    with Session() as s:
+        st = ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream,
+                                  tile_flags=flags, tile_rows=0)
+        assert st == ep.ERR_PARA_CHECK_FAIL

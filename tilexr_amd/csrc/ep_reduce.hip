@@ -73,6 +73,12 @@ __device__ bool WaitTile(const ReduceArgs &a, int row)
         if (static_cast<int64_t>(wall_clock64() - start) > a.waitTimeoutTicks) {
             return false;
         }
+        // once one wait of the launch has expired the producer is taken to be gone: later waits give up at once,
+        // so a launch whose flags never arrive ends after about one timeout, not one per tile
+        if (a.deviceStatus != nullptr &&
+            __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+            return false;
+        }
         __builtin_amdgcn_s_sleep(4);
     }
 }
