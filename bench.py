@@ -43,6 +43,10 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-kernel-events", action="store_true",
                    help="do not record per-kernel HIP events inside the timed region")
+    p.add_argument("--overlap", action="store_true",
+                   help="run combine on a second stream, consuming tiles through readiness flags while dispatch is "
+                        "still writing rows")
+    p.add_argument("--tile-rows", type=int, default=256)
     p.add_argument("--event-stride", type=int, default=10,
                    help="record the per-kernel events on every N-th timed step")
     p.add_argument("--calibrate-copy", action="store_true",
@@ -119,7 +123,13 @@ def main():
     elif quant == ep.Q_FP8_BLOCK128:
         scales = torch.empty((rows_max, (h + 127) // 128), dtype=torch.float32, device=dev)
 
-    def step():
+    side = torch.cuda.Stream()
+    tiles = (rows_max + args.tile_rows - 1) // args.tile_rows
+    flags = torch.zeros((tiles,), dtype=torch.int64, device=dev)
+    status = torch.zeros((1,), dtype=torch.int32, device=dev)
+    meta_ready, combined = ep.HipEvent(), ep.HipEvent()
+
+    def step_serial():
         st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
                                       ep.DT_BF16, stream, quant_mode=quant, expert_capacity=w.capacity,
                                       dynamic_scales=scales, row_index_map=row_map)
@@ -127,6 +137,24 @@ def main():
         ep.check(ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
                                       expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
                                       row_index_map=row_map), "combine")
+
+    def step_overlapped():
+        # dispatch on `stream` publishes tiles; combine on `side` starts once the metadata is enqueued and reduces
+        # tokens as their tiles land; the next dispatch waits until this combine has read the rows
+        st, epoch = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
+                                          ep.DT_BF16, stream, quant_mode=quant, expert_capacity=w.capacity,
+                                          dynamic_scales=scales, row_index_map=row_map, tile_flags=flags,
+                                          tile_rows=args.tile_rows, meta_ready_event=meta_ready.value)
+        ep.check(st, "dispatch")
+        meta_ready.wait_on(side)
+        ep.check(ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, side,
+                                      expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
+                                      row_index_map=row_map, tile_flags=flags, tile_rows=args.tile_rows,
+                                      flag_epoch=epoch, device_status=status), "combine")
+        combined.record(side)
+        combined.wait_on(stream)
+
+    step = step_overlapped if args.overlap else step_serial
 
     if args.calibrate_copy:
         src = torch.zeros((64 << 20,), dtype=torch.int32, device=dev)
@@ -166,7 +194,11 @@ def main():
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
 
-    # split of one step into its two calls (outside the timed region)
+    if args.overlap and status.item() != 0:
+        print("a tile-flag wait expired during the run", file=sys.stderr)
+        sys.exit(1)
+
+    # split of one step into its two calls, run back to back on one stream (outside the timed region)
     d_ev[0].record(stream)
     st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts, ep.DT_BF16,
                                   stream, quant_mode=quant, expert_capacity=w.capacity, dynamic_scales=scales,
@@ -205,7 +237,8 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "us_per_layer": round(ms_per_step * 1e3, 2),
         "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": dict(workloads.describe(w, ids), kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+        "config": dict(workloads.describe(w, ids), schedule="overlapped via tile flags" if args.overlap else "serial",
+                       kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
         "roofline": roofline, "kernels": kernels,
     }

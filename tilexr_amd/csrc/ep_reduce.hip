@@ -57,7 +57,9 @@ __device__ __forceinline__ int LookupRow(const ReduceArgs &a, int64_t slot)
     return (e >> 32) == a.epoch ? static_cast<int>(e & 0xffffffffu) : -1;
 }
 
-// Bounded acquire-wait until the tile holding `row` has all its rows published for this epoch.
+// Bounded wait until the tile holding `row` has all its rows published for this epoch.  The poll itself is a relaxed
+// device-scope load (no cache maintenance per iteration -- an acquire in the loop would invalidate this XCD's L2 on
+// every spin and starve the producer); the caller issues one acquire fence after all its waits have succeeded.
 __device__ bool WaitTile(const ReduceArgs &a, int row)
 {
     const int tile = row / a.tileRows;
@@ -66,7 +68,7 @@ __device__ bool WaitTile(const ReduceArgs &a, int row)
     need = need > a.tileRows ? a.tileRows : need;
     const uint64_t start = wall_clock64();
     while (true) {
-        const uint64_t w = __hip_atomic_load(&a.tileFlags[tile], __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT);
+        const uint64_t w = __hip_atomic_load(&a.tileFlags[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if ((w >> 32) == a.flagEpoch && static_cast<int>(w & 0xffffffffu) >= need) {
             return true;
         }
@@ -79,7 +81,7 @@ __device__ bool WaitTile(const ReduceArgs &a, int row)
             __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
             return false;
         }
-        __builtin_amdgcn_s_sleep(4);
+        __builtin_amdgcn_s_sleep(16);
     }
 }
 
@@ -127,6 +129,11 @@ __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool 
         }
         rows[k] = row;
         weights[k] = (tokOk && a.expertScales != nullptr) ? a.expertScales[slot] : 1.0f;
+    }
+    if (a.tileFlags != nullptr && lane < a.topK) {
+        // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
+        // workgroup after the barrier that follows) are at least as new as the flag values seen above
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
 }
 

@@ -62,13 +62,16 @@ __device__ __forceinline__ float GroupMax(float v, float *red, int lane)
 
 __device__ __forceinline__ void PublishRows(uint64_t *tileFlags, int tileRows, const int *pos, int topK, int lane, int G)
 {
-    // every lane's row stores are complete once the workgroup barrier has been passed; the release below makes
-    // them visible at agent scope before the tile counter moves
+    // every lane's row stores have been issued once the workgroup barrier has been passed; one release fence per
+    // lane that publishes (not one per row) makes them visible at device scope before the tile counters move
     __syncthreads();
-    for (int k = lane; k < topK; k += G) {
-        const int row = pos[k];
-        if (row >= 0) {
-            __hip_atomic_fetch_add(&tileFlags[row / tileRows], 1ull, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    if (lane < topK) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        for (int k = lane; k < topK; k += G) {
+            const int row = pos[k];
+            if (row >= 0) {
+                __hip_atomic_fetch_add(&tileFlags[row / tileRows], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
         }
     }
 }
