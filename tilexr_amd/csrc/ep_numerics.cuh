@@ -1,8 +1,11 @@
 // Device-side element conversions shared by the scatter and reduce kernels (gfx950, wave64).
 //
 // Every routine is written so that its result is a pure function of the input bits: separate multiplies and adds
-// (the build uses -ffp-contract=off and the explicit *_rn intrinsics), software fp8 encoders instead of the
-// hardware converts, and saturation made explicit.  That is what lets the parity tests demand bit equality.
+// (the build uses -ffp-contract=off and the explicit *_rn intrinsics) and saturation made explicit.  That is what
+// lets the parity tests demand bit equality.  Hardware converts are used only where an exhaustive comparison on
+// gfx950 showed them equal to the software codec: v_cvt_pk_bf16_f32 (all 2^32 inputs, NaNs included),
+// v_cvt_pk_f32_fp8 (all codes except the sign of NaN code 0x7f) and v_cvt_pk_fp8_f32 (all finite |x| < 464; beyond
+// that the hardware returns NaN where this codec saturates, so inputs are clamped first and NaNs patched).
 //   int8 rounding      reference: src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:183-193
 //   MXFP8 / fp8 codec  reference: tests/ep/demo/mxfp8_golden.h:45-152
 //   output casts       reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:595 (CAST_RINT, saturating)
@@ -26,14 +29,19 @@ __device__ __forceinline__ float Decode16(uint32_t bits16)
     return __half2float(__ushort_as_half(static_cast<unsigned short>(bits16)));
 }
 
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+
+// Two fp32 -> two bf16 (round to nearest even, NaN -> (bits >> 16) | 0x40), packed lo | hi << 16.
+__device__ __forceinline__ uint32_t FloatPairToBf16Rne(float lo, float hi)
+{
+    const f32x2 f = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, bf16x2));
+}
+
 __device__ __forceinline__ uint32_t FloatToBf16Rne(float v)
 {
-    uint32_t u = __float_as_uint(v);
-    if ((u & 0x7fffffffu) > 0x7f800000u) {
-        return (u >> 16) | 0x0040u;
-    }
-    u += 0x7fffu + ((u >> 16) & 1u);
-    return u >> 16;
+    return FloatPairToBf16Rne(v, 0.0f) & 0xffffu;
 }
 
 // IEEE round-to-nearest-even; overflow becomes infinity.
@@ -57,6 +65,13 @@ template <bool BF16>
 __device__ __forceinline__ uint32_t Encode16Sat(float v)
 {
     return BF16 ? FloatToBf16Rne(v) : FloatToHalfRneSat(v);
+}
+
+// Two values -> packed 16-bit elements (lo | hi << 16), fp16 saturating as above.
+template <bool BF16>
+__device__ __forceinline__ uint32_t EncodePair16Sat(float lo, float hi)
+{
+    return BF16 ? FloatPairToBf16Rne(lo, hi) : (FloatToHalfRneSat(lo) | (FloatToHalfRneSat(hi) << 16));
 }
 
 // Round an fp32 value to the 16-bit element type and return it as fp32 again (IEEE, non-saturating).
@@ -139,6 +154,46 @@ __device__ __forceinline__ float Fp8Decode(uint32_t code)
         return __uint_as_float(sign | 0x7fc00000u);
     }
     return __uint_as_float(sign | ((exp + 127u - kBias) << 23) | (man << (23 - kMantBits)));
+}
+
+// e4m3 code of x with round-to-nearest-even and saturation to +-448; NaN -> sign | 0x7f.  Same function as
+// Fp8Encode<false>, through the hardware convert.
+__device__ __forceinline__ uint32_t Fp8E4m3EncodePairSat(float lo, float hi)
+{
+    const float clo = __builtin_amdgcn_fmed3f(lo, -448.0f, 448.0f);
+    const float chi = __builtin_amdgcn_fmed3f(hi, -448.0f, 448.0f);
+    uint32_t code = static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(clo, chi, 0, false)) & 0xffffu;
+    if (lo != lo) {
+        code = (code & 0xff00u) | ((__float_as_uint(lo) >> 24) & 0x80u) | 0x7fu;
+    }
+    if (hi != hi) {
+        code = (code & 0x00ffu) | ((((__float_as_uint(hi) >> 24) & 0x80u) | 0x7fu) << 8);
+    }
+    return code;
+}
+
+// True when one of the four e4m3 codes in `word` is a NaN code (0x7f / 0xff).
+__device__ __forceinline__ bool Fp8E4m3WordHasNan(uint32_t word)
+{
+    return (((word & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u) != 0u;
+}
+
+// Four e4m3 codes -> four fp32, same values as Fp8Decode<false> (NaN codes take the software path).
+__device__ __forceinline__ void Fp8E4m3DecodeWord(uint32_t word, float *out)
+{
+    if (Fp8E4m3WordHasNan(word)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            out[i] = Fp8Decode<false>((word >> (8 * i)) & 0xffu);
+        }
+        return;
+    }
+    const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), false);
+    const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), true);
+    out[0] = lo[0];
+    out[1] = lo[1];
+    out[2] = hi[0];
+    out[3] = hi[1];
 }
 
 // Shared exponent of an MXFP8 block: clamp(floor(log2 amax) - emax, -127, 127); all-zero block -> -127.

@@ -137,7 +137,7 @@ __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool 
     }
 }
 
-template <int G, int V, int KIND, int INQ, bool BF16, int COMMQ>
+template <int G, int V, int KIND, bool BF16, int COMMQ>
 __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 {
     constexpr int kTokens = kThreads / G;
@@ -150,7 +150,6 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
     const int lane = threadIdx.x % G;
     const int vecs = a.h / 8;
     const int groups = (a.bs + kTokens - 1) / kTokens;
-    const int b128 = (a.h + 127) / 128;
 
     for (int group = blockIdx.x; group < groups; group += gridDim.x) {
         const int token = group * kTokens + tg;
@@ -183,41 +182,19 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             const float w = s_w[tg][k];
             const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row) * a.rowBytes;
             u32x4 v16[V];
-            u32x2 v8[V];
-            float sc[V];
 #pragma unroll
             for (int j = 0; j < V; ++j) {
                 const int idx = j * G + lane;
-                const bool inRow = idx < vecs;
-                if (INQ == 0) {
-                    v16[j] = inRow ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) :
-                                     u32x4{0u, 0u, 0u, 0u};
-                } else {
-                    v8[j] = inRow ? __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(base) + idx) :
-                                    u32x2{0u, 0u};
-                    sc[j] = !inRow ? 0.0f : (INQ == TILEXR_EP_QUANT_TOKEN_INT8 ? a.inScales[row] :
-                        a.inScales[static_cast<int64_t>(row) * b128 + (idx >> 4)]);
-                }
+                v16[j] = idx < vecs ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) :
+                                      u32x4{0u, 0u, 0u, 0u};
             }
 #pragma unroll
             for (int j = 0; j < V; ++j) {
                 float f[8];
-                if (INQ == 0) {
 #pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        f[2 * q] = Decode16<BF16>(v16[j][q] & 0xffffu);
-                        f[2 * q + 1] = Decode16<BF16>(v16[j][q] >> 16);
-                    }
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const uint32_t byte = (v8[j][e >> 2] >> ((e & 3) * 8)) & 0xffu;
-                        const float d = INQ == TILEXR_EP_QUANT_TOKEN_INT8 ?
-                            __fmul_rn(static_cast<float>(static_cast<int>(static_cast<int8_t>(byte))), sc[j]) :
-                            __fmul_rn(Fp8Decode<false>(byte), sc[j]);
-                        f[e] = BF16 ? __uint_as_float(FloatToBf16Rne(d) << 16) :
-                                      __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d))));
-                    }
+                for (int q = 0; q < 4; ++q) {
+                    f[2 * q] = Decode16<BF16>(v16[j][q] & 0xffffu);
+                    f[2 * q + 1] = Decode16<BF16>(v16[j][q] >> 16);
                 }
                 if (kMx) {
                     float amax = 0.0f;
@@ -273,11 +250,146 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                     u32x4 o;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        const uint32_t lo = active ? Encode16Sat<BF16>(acc[j][2 * q]) : 0u;
-                        const uint32_t hi = active ? Encode16Sat<BF16>(acc[j][2 * q + 1]) : 0u;
-                        o[q] = lo | (hi << 16);
+                        o[q] = active ? EncodePair16Sat<BF16>(acc[j][2 * q], acc[j][2 * q + 1]) : 0u;
                     }
                     __builtin_nontemporal_store(o, dst + idx);
+                }
+            }
+        }
+    }
+}
+
+// Quantised expert output: int8 rows with one fp32 scale per row, or fp8 e4m3 rows with one fp32 scale per 128
+// columns.  Each value is dequantised, rounded to the output element type, then accumulated exactly like an ordinary
+// row (fp32, k order, separate multiply and add).  Rows are a quarter the bytes of bf16 rows, so a lane owns 16
+// consecutive columns per vector (one 16-byte load) and KB rows are kept in flight at once.
+template <int G, int V, int INQ, bool BF16>
+__global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
+{
+    constexpr int kTokens = kThreads / G;
+    constexpr int KB = V >= 4 ? 2 : 4;
+    __shared__ int s_row[kTokens][kMaxTopK];
+    __shared__ float s_w[kTokens][kMaxTopK];
+
+    const int tg = threadIdx.x / G;
+    const int lane = threadIdx.x % G;
+    const int vecs = a.h / 16;
+    const int groups = (a.bs + kTokens - 1) / kTokens;
+    const int b128 = (a.h + 127) / 128;
+
+    for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+        const int token = group * kTokens + tg;
+        const bool tokOk = token < a.bs;
+        __syncthreads();
+        LoadRoutes(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
+        __syncthreads();
+        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0);
+
+        float acc[V][16];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                acc[j][e] = 0.0f;
+            }
+        }
+        for (int k0 = 0; k0 < a.topK; k0 += KB) {
+            u32x4 q[KB][V];
+            float sc[KB][V];
+            int rowOfK[KB];
+#pragma unroll
+            for (int u = 0; u < KB; ++u) {
+                const int k = k0 + u;
+                const int row = (k < a.topK && active) ? s_row[tg][k] : -1;
+                rowOfK[u] = row;
+                const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const int idx = j * G + lane;
+                    const bool live = row >= 0 && idx < vecs;
+                    q[u][j] = live ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) :
+                                     u32x4{0u, 0u, 0u, 0u};
+                    sc[u][j] = !live ? 0.0f : (INQ == TILEXR_EP_QUANT_TOKEN_INT8 ? a.inScales[row] :
+                        a.inScales[static_cast<int64_t>(row) * b128 + (idx >> 3)]);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < KB; ++u) {
+                if (rowOfK[u] < 0) {
+                    continue;                       // uniform across the lanes of a token
+                }
+                const float w = s_w[tg][k0 + u];
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        const uint32_t word = q[u][j][d];
+                        float f[4];
+                        if (INQ == TILEXR_EP_QUANT_TOKEN_INT8) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                f[e] = static_cast<float>(static_cast<int>(static_cast<int8_t>((word >> (8 * e)) & 0xffu)));
+                            }
+                        } else {
+                            Fp8E4m3DecodeWord(word, f);
+                        }
+#pragma unroll
+                        for (int e = 0; e < 4; e += 2) {
+                            const float d0 = __fmul_rn(f[e], sc[u][j]);
+                            const float d1 = __fmul_rn(f[e + 1], sc[u][j]);
+                            float r0;
+                            float r1;
+                            if (BF16) {
+                                const uint32_t packed = FloatPairToBf16Rne(d0, d1);
+                                r0 = __uint_as_float(packed << 16);
+                                r1 = __uint_as_float(packed & 0xffff0000u);
+                            } else {
+                                r0 = __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d0))));
+                                r1 = __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d1))));
+                            }
+                            acc[j][4 * d + e] = __fadd_rn(acc[j][4 * d + e], __fmul_rn(r0, w));
+                            acc[j][4 * d + e + 1] = __fadd_rn(acc[j][4 * d + e + 1], __fmul_rn(r1, w));
+                        }
+                    }
+                }
+            }
+        }
+        if (a.sharedExpertX != nullptr && active) {
+            const u32x4 *sx = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.sharedExpertX) +
+                static_cast<int64_t>(token) * a.h * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = j * G + lane;
+                if (idx < vecs) {
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const u32x4 v = sx[idx * 2 + half];
+#pragma unroll
+                        for (int q2 = 0; q2 < 4; ++q2) {
+                            float &lo = acc[j][half * 8 + 2 * q2];
+                            float &hi = acc[j][half * 8 + 2 * q2 + 1];
+                            lo = __fadd_rn(lo, Decode16<BF16>(v[q2] & 0xffffu));
+                            hi = __fadd_rn(hi, Decode16<BF16>(v[q2] >> 16));
+                        }
+                    }
+                }
+            }
+        }
+        if (tokOk) {
+            u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.y) + static_cast<int64_t>(token) * a.h * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = j * G + lane;
+                if (idx < vecs) {
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        u32x4 o;
+#pragma unroll
+                        for (int q2 = 0; q2 < 4; ++q2) {
+                            o[q2] = active ? EncodePair16Sat<BF16>(acc[j][half * 8 + 2 * q2], acc[j][half * 8 + 2 * q2 + 1]) : 0u;
+                        }
+                        __builtin_nontemporal_store(o, dst + idx * 2 + half);
+                    }
                 }
             }
         }
@@ -370,7 +482,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
     }
 }
 
-template <int G, int V, int KIND, int INQ, bool BF16, int COMMQ>
+template <int G, int V, int KIND, bool BF16, int COMMQ>
 void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
 {
     constexpr int kTokens = kThreads / G;
@@ -378,24 +490,20 @@ void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
     if (gridLimit > 0 && grid > gridLimit) {
         grid = gridLimit;
     }
-    hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, INQ, BF16, COMMQ>), dim3(grid), dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ>), dim3(grid), dim3(kThreads), 0, stream, a);
 }
 
 template <int G, int V, bool BF16>
 void LaunchByMode(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
 {
     if (l.reduceKind == kReducePerAdd) {
-        LaunchVec<G, V, kReducePerAdd, 0, BF16, 0>(a, gridLimit, l.stream);
-    } else if (l.inQuant == TILEXR_EP_QUANT_TOKEN_INT8) {
-        LaunchVec<G, V, kReduceFp32, TILEXR_EP_QUANT_TOKEN_INT8, BF16, 0>(a, gridLimit, l.stream);
-    } else if (l.inQuant == TILEXR_EP_QUANT_FP8_BLOCK128) {
-        LaunchVec<G, V, kReduceFp32, TILEXR_EP_QUANT_FP8_BLOCK128, BF16, 0>(a, gridLimit, l.stream);
+        LaunchVec<G, V, kReducePerAdd, BF16, 0>(a, gridLimit, l.stream);
     } else if (l.commQuant == TILEXR_EP_QUANT_COMM_MXFP8_E5M2) {
-        LaunchVec<G, V, kReduceFp32, 0, BF16, TILEXR_EP_QUANT_COMM_MXFP8_E5M2>(a, gridLimit, l.stream);
+        LaunchVec<G, V, kReduceFp32, BF16, TILEXR_EP_QUANT_COMM_MXFP8_E5M2>(a, gridLimit, l.stream);
     } else if (l.commQuant == TILEXR_EP_QUANT_MXFP8) {
-        LaunchVec<G, V, kReduceFp32, 0, BF16, TILEXR_EP_QUANT_MXFP8>(a, gridLimit, l.stream);
+        LaunchVec<G, V, kReduceFp32, BF16, TILEXR_EP_QUANT_MXFP8>(a, gridLimit, l.stream);
     } else {
-        LaunchVec<G, V, kReduceFp32, 0, BF16, 0>(a, gridLimit, l.stream);
+        LaunchVec<G, V, kReduceFp32, BF16, 0>(a, gridLimit, l.stream);
     }
 }
 
@@ -406,6 +514,31 @@ void LaunchByType(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
         LaunchByMode<G, V, true>(l, a, gridLimit);
     } else {
         LaunchByMode<G, V, false>(l, a, gridLimit);
+    }
+}
+
+template <int G, int V>
+void LaunchQuant(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
+{
+    constexpr int kTokens = kThreads / G;
+    int grid = (a.bs + kTokens - 1) / kTokens;
+    if (gridLimit > 0 && grid > gridLimit) {
+        grid = gridLimit;
+    }
+    const dim3 g(grid);
+    const dim3 b(kThreads);
+    if (l.inQuant == TILEXR_EP_QUANT_TOKEN_INT8) {
+        if (l.bf16) {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_TOKEN_INT8, true>), g, b, 0, l.stream, a);
+        } else {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_TOKEN_INT8, false>), g, b, 0, l.stream, a);
+        }
+    } else {
+        if (l.bf16) {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_FP8_BLOCK128, true>), g, b, 0, l.stream, a);
+        } else {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_FP8_BLOCK128, false>), g, b, 0, l.stream, a);
+        }
     }
 }
 
@@ -438,12 +571,26 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     // compute unit (8 of 32 wave slots) and let it walk the tokens.
     const int gridLimit = l.tileFlags != nullptr ? 2 * (l.numComputeUnits > 0 ? l.numComputeUnits : 256) : 0;
     const int64_t vecs = l.h / 8;
-    const bool mixed = (l.inQuant != 0 && l.commQuant != 0);
-    const bool vecOk = !mixed && l.h % 8 == 0 && Aligned16(l.y) && vecs <= 8 * kThreads &&
-        (l.inQuant == 0 ? (Aligned16(l.expertOut) && l.rowBytes % 16 == 0) :
-                          (Aligned8(l.expertOut) && l.rowBytes % 8 == 0)) &&
+    const bool plain = l.inQuant == 0 && l.h % 8 == 0 && Aligned16(l.y) && vecs <= 8 * kThreads &&
+        Aligned16(l.expertOut) && l.rowBytes % 16 == 0 &&
         (l.sharedExpertX == nullptr || Aligned16(l.sharedExpertX)) && (l.commQuant == 0 || l.h % 32 == 0);
-    if (vecOk) {
+    const int64_t qvecs = l.h / 16;
+    const bool quant = l.inQuant != 0 && l.commQuant == 0 && l.reduceKind == kReduceFp32 && l.h % 16 == 0 &&
+        qvecs <= 4 * kThreads && Aligned16(l.y) && Aligned16(l.expertOut) && l.rowBytes % 16 == 0 &&
+        (l.sharedExpertX == nullptr || Aligned16(l.sharedExpertX));
+    if (quant) {
+        if (qvecs <= kWave) {
+            LaunchQuant<kWave, 1>(l, a, gridLimit);
+        } else if (qvecs <= 2 * kWave) {
+            LaunchQuant<2 * kWave, 1>(l, a, gridLimit);
+        } else if (qvecs <= kThreads) {
+            LaunchQuant<kThreads, 1>(l, a, gridLimit);
+        } else if (qvecs <= 2 * kThreads) {
+            LaunchQuant<kThreads, 2>(l, a, gridLimit);
+        } else {
+            LaunchQuant<kThreads, 4>(l, a, gridLimit);
+        }
+    } else if (plain) {
         if (vecs <= 2 * kWave) {
             LaunchByType<kWave, 2>(l, a, gridLimit);
         } else if (vecs <= 4 * kWave) {

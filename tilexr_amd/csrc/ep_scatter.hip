@@ -173,8 +173,10 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
                     const float sc = amax > 0.0f ? __fdiv_rn(amax, 448.0f) : 1.0f;
                     blockScale[j] = sc;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        bytes[e] = Fp8Encode<false>(__fdiv_rn(f[e], sc));
+                    for (int e = 0; e < 8; e += 2) {
+                        const uint32_t pair = Fp8E4m3EncodePairSat(__fdiv_rn(f[e], sc), __fdiv_rn(f[e + 1], sc));
+                        bytes[e] = pair & 0xffu;
+                        bytes[e + 1] = pair >> 8;
                     }
                 }
             } else {
