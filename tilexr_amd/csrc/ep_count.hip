@@ -51,8 +51,11 @@ struct RouteCountArgs {
     int tokenNumsType;
 };
 
+// BPW = batches of 64 routes per wave: a workgroup counts 256 * BPW consecutive routes.
+template <int BPW>
 __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs a)
 {
+    constexpr int kChunkRoutes = kThreads * BPW;
     __shared__ int s_cnt[kWavesPerBlock * kMaxKeys];
     __shared__ int s_exp[kMaxKeys];
     __shared__ int s_part[kThreads];
@@ -96,29 +99,57 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
         liveLimit = s_misc[0] * a.topK;
     }
 
-    // phase A: per-wave histogram of the wave's 256 consecutive routes
-    int keys[kChunkRoutes / kThreads];
+    // phase A: load the wave's 64 * BPW consecutive routes (all loads in flight together), decide liveness and key
+    int keys[BPW];
+    {
+        int e[BPW];
+        int m[BPW];
 #pragma unroll
-    for (int b = 0; b < kChunkRoutes / kThreads; ++b) {
-        const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
-        int key = -1;
-        if (i < n && i < liveLimit) {
-            const int e = a.ids[i];
-            bool live = e >= 0 && e < a.numExperts;
+        for (int b = 0; b < BPW; ++b) {
+            const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
+            const bool inRange = i < n && i < liveLimit;
+            e[b] = inRange ? a.ids[i] : -1;
+            m[b] = 1;
             if (a.maskMode == kMaskPerToken) {
-                live = live && a.mask[i / a.topK] != 0;
+                m[b] = inRange ? a.mask[i / a.topK] : 0;
             } else if (a.maskMode == kMaskPerRoute) {
-                live = live && a.mask[i] != 0;
-            }
-            if (live) {
-                key = e / a.keyDiv;
-                atomicAdd(&s_cnt[wave * a.numKeys + key], 1);
-                if (expHist) {
-                    atomicAdd(&s_exp[e], 1);
-                }
+                m[b] = inRange ? a.mask[i] : 0;
             }
         }
-        keys[b] = key;
+#pragma unroll
+        for (int b = 0; b < BPW; ++b) {
+            const bool live = e[b] >= 0 && e[b] < a.numExperts && m[b] != 0;
+            keys[b] = live ? (a.keyDiv == 1 ? e[b] : e[b] / a.keyDiv) : -1;
+            if (expHist && live) {
+                atomicAdd(&s_exp[e[b]], 1);
+            }
+        }
+    }
+    // lanes of a batch with equal keys find each other with one ballot per key bit; the bit loop is outermost so
+    // that the BPW batches give independent instruction streams
+    unsigned long long peers[BPW];
+#pragma unroll
+    for (int b = 0; b < BPW; ++b) {
+        peers[b] = __ballot(keys[b] >= 0);
+    }
+    for (int bit = 0; bit < a.keyBits; ++bit) {
+#pragma unroll
+        for (int b = 0; b < BPW; ++b) {
+            const bool one = keys[b] >= 0 && ((keys[b] >> bit) & 1);
+            const unsigned long long bal = __ballot(one);
+            peers[b] &= one ? bal : ~bal;
+        }
+    }
+    const unsigned long long lt = LaneMaskLt();
+    int packed[BPW];            // lanes of the same key before this one | lanes of the same key << 8
+#pragma unroll
+    for (int b = 0; b < BPW; ++b) {
+        const int before = __popcll(peers[b] & lt);
+        const int same = __popcll(peers[b]);
+        packed[b] = before | (same << 8);
+        if (keys[b] >= 0 && before == 0) {
+            atomicAdd(&s_cnt[wave * a.numKeys + keys[b]], same);      // one LDS atomic per distinct key of a batch
+        }
     }
     __syncthreads();
 
@@ -140,40 +171,39 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     }
     __syncthreads();
 
-    // phase C: batches of 64 routes in order; lanes with equal keys find each other with one ballot per key bit
+    // phase C: batches in order; the running count of a key within the wave lives in LDS (a wave's LDS operations
+    // execute in program order, the barriers only stop the compiler from reordering them)
     volatile int *cnt = s_cnt + wave * a.numKeys;
-    const unsigned long long lt = LaneMaskLt();
 #pragma unroll
-    for (int b = 0; b < kChunkRoutes / kThreads; ++b) {
-        const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
+    for (int b = 0; b < BPW; ++b) {
         const int key = keys[b];
         const bool live = key >= 0;
-        unsigned long long peers = __ballot(live);
-        for (int bit = 0; bit < a.keyBits; ++bit) {
-            const bool one = live && ((key >> bit) & 1);
-            const unsigned long long bal = __ballot(one);
-            peers &= one ? bal : ~bal;
-        }
-        const int before = __popcll(peers & lt);
+        const int before = packed[b] & 0xff;
         const int base = live ? cnt[key] : 0;
-        if (i < n) {
-            a.s.localRank[i] = live ? base + before : -1;
-        }
         __builtin_amdgcn_wave_barrier();
         if (live && before == 0) {
-            cnt[key] = base + __popcll(peers);
+            cnt[key] = base + (packed[b] >> 8);
         }
         __builtin_amdgcn_wave_barrier();
+        packed[b] = live ? base + before : -1;
     }
 
-    // last workgroup to arrive performs the scans
+    // The last workgroup to arrive performs the scans.  Only the chunk histograms (stored in phase B, long since
+    // on their way) have to be visible to it, so the ticket is taken before the rank stores are issued.
     __threadfence();
     __syncthreads();
     if (tid == 0) {
         const unsigned prev = atomicAdd(a.s.ticket, 1u);
         s_misc[1] = prev == static_cast<unsigned>(a.numChunks - 1) ? 1 : 0;
     }
-    __syncthreads();
+#pragma unroll
+    for (int b = 0; b < BPW; ++b) {
+        const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
+        if (i < n) {
+            a.s.localRank[i] = packed[b];
+        }
+    }
+    LdsBarrier();
     if (s_misc[1] == 0) {
         return;
     }
@@ -183,8 +213,8 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     int *kept = s_cnt;                 // reuse: [numKeys]
     for (int key = tid; key < a.numKeys; key += kThreads) {
         int run = 0;
-        // 16 independent loads per round trip to HBM, then the in-place exclusive sum
-        constexpr int kBatch = 16;
+        // the loads of a batch are independent: one round trip per 32 chunks
+        constexpr int kBatch = 32;
         for (int c0 = 0; c0 < a.numChunks; c0 += kBatch) {
             int v[kBatch];
 #pragma unroll
@@ -205,12 +235,12 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
         kept[key] = k;
         a.s.keyKept[key] = k;
     }
-    __syncthreads();
+    LdsBarrier();
     int *offs = s_cnt + kMaxKeys;      // [numKeys] exclusive offsets
     for (int key = tid; key < a.numKeys; key += kThreads) {
         offs[key] = kept[key];
     }
-    __syncthreads();
+    LdsBarrier();
     const int totalRows = BlockExclusiveScan(offs, a.numKeys, s_part);
     for (int key = tid; key < a.numKeys; key += kThreads) {
         a.s.keyOffset[key] = offs[key];
@@ -242,17 +272,22 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
             etot[e] = e < a.numKeys ? kept[e] : 0;
         }
     }
-    __syncthreads();
+    LdsBarrier();
     for (int e = tid; e < a.numExperts; e += kThreads) {
         a.s.expertTotal[e] = etot[e];
     }
     if (a.expertTokenNumsOut != nullptr) {
-        if (a.tokenNumsType == 0) {
+        if (a.tokenNumsType == 0 && !expHist) {
+            // keys are experts: the inclusive prefix sum is the one already computed for the counts output
+            for (int e = tid; e < a.numExperts; e += kThreads) {
+                a.expertTokenNumsOut[e] = e < a.numKeys ? static_cast<int64_t>(offs[e]) + kept[e] : totalRows;
+            }
+        } else if (a.tokenNumsType == 0) {
             int *pref = s_cnt + 3 * kMaxKeys;
             for (int e = tid; e < a.numExperts; e += kThreads) {
                 pref[e] = etot[e];
             }
-            __syncthreads();
+            LdsBarrier();
             BlockExclusiveScan(pref, a.numExperts, s_part);
             for (int e = tid; e < a.numExperts; e += kThreads) {
                 a.expertTokenNumsOut[e] = static_cast<int64_t>(pref[e]) + etot[e];
@@ -362,7 +397,11 @@ CountScratchLayout PlanCountScratch(int64_t routes, int64_t numKeys, int64_t num
 {
     auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
     CountScratchLayout p {};
-    p.chunks = (routes + kChunkRoutes - 1) / kChunkRoutes;
+    p.chunkShift = kMinChunkShift;
+    while (p.chunkShift < kMaxChunkShift && ((routes + (1ll << p.chunkShift) - 1) >> p.chunkShift) > kTargetChunks) {
+        ++p.chunkShift;
+    }
+    p.chunks = (routes + (1ll << p.chunkShift) - 1) >> p.chunkShift;
     int64_t off = 256;   // word 0 is the ticket
     p.localRankOff = off;
     off += align(routes * 4);
@@ -396,13 +435,30 @@ hipError_t LaunchRouteCount(const RouteCountLaunch &l)
     a.keyBits = KeyBits(l.numKeys);
     a.capacity = static_cast<int>(l.capacity);
     const int64_t n = l.bs * l.topK;
-    a.numChunks = static_cast<int>((n + kChunkRoutes - 1) / kChunkRoutes);
+    const int shift = l.scratch.chunkShift;
+    a.numChunks = static_cast<int>((n + (1ll << shift) - 1) >> shift);
     a.s = l.scratch;
     a.sendCountsOut = l.sendCountsOut;
     a.recvCountOut = l.recvCountOut;
     a.expertTokenNumsOut = l.expertTokenNumsOut;
     a.tokenNumsType = l.tokenNumsType;
-    hipLaunchKernelGGL(ep_route_count_kernel, dim3(a.numChunks), dim3(kThreads), 0, l.stream, a);
+    const dim3 grid(static_cast<unsigned>(a.numChunks > 0 ? a.numChunks : 1));
+    switch (shift) {
+        case 10:
+            hipLaunchKernelGGL(ep_route_count_kernel<4>, grid, dim3(kThreads), 0, l.stream, a);
+            break;
+        case 11:
+            hipLaunchKernelGGL(ep_route_count_kernel<8>, grid, dim3(kThreads), 0, l.stream, a);
+            break;
+        case 12:
+            hipLaunchKernelGGL(ep_route_count_kernel<16>, grid, dim3(kThreads), 0, l.stream, a);
+            break;
+        case 13:
+            hipLaunchKernelGGL(ep_route_count_kernel<32>, grid, dim3(kThreads), 0, l.stream, a);
+            break;
+        default:
+            return hipErrorInvalidValue;
+    }
     return hipGetLastError();
 }
 

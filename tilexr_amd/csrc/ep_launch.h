@@ -21,7 +21,9 @@
 
 namespace TileXREp {
 
-constexpr int kChunkRoutes = 1024;      // routes handled by one counting workgroup
+constexpr int kMinChunkShift = 10;      // a counting workgroup handles 2^shift routes: 1024 ...
+constexpr int kMaxChunkShift = 13;      // ... up to 8192, chosen so that about kTargetChunks workgroups run
+constexpr int kTargetChunks = 64;       // (the last one to finish scans one histogram row per chunk)
 constexpr int kMaxKeys = 2048;          // keys (experts) the counting kernel's LDS tables hold
 constexpr int kMaxTopK = 64;
 
@@ -33,6 +35,7 @@ enum MaskMode : int {
 };
 
 struct CountScratch {
+    int chunkShift;         // log2 of the routes per counting workgroup
     uint32_t *ticket;       // 1 word, zero between launches
     int32_t *localRank;     // [n]  rank of the route within (chunk, key); -1 when the route is not live
     int32_t *chunkHist;     // [chunks, numKeys] in: counts; out: exclusive sum over earlier chunks
@@ -154,6 +157,7 @@ hipError_t LaunchReduce(const ReduceLaunch &l);
 
 // Bytes of CountScratch arrays for a problem (used by the host to carve one allocation).
 struct CountScratchLayout {
+    int chunkShift;
     int64_t chunks;
     int64_t localRankOff, chunkHistOff, chunkExpHistOff, keyOffsetOff, keyKeptOff, expertTotalOff, rowOfOff;
     int64_t totalBytes;

@@ -19,6 +19,7 @@ struct PlaceArgs {
     const int32_t *localRank;    // [n] rank within (chunk, key), -1 = not live
     const int32_t *chunkBase;    // [chunks, numKeys] routes of the key in earlier chunks
     const int32_t *keyOffset;    // [numKeys + 1]
+    int chunkShift;
     int n;
     int topK;
     int keyDiv;
@@ -37,6 +38,7 @@ inline PlaceArgs MakePlaceArgs(const RoutePlaceLaunch &l)
     a.localRank = l.scratch.localRank;
     a.chunkBase = l.scratch.chunkHist;
     a.keyOffset = l.scratch.keyOffset;
+    a.chunkShift = l.scratch.chunkShift;
     a.n = static_cast<int>(l.bs * l.topK);
     a.topK = static_cast<int>(l.topK);
     a.keyDiv = static_cast<int>(l.keyDiv);
@@ -57,7 +59,7 @@ __device__ __forceinline__ int PlaceRoute(const PlaceArgs &a, int i)
     if (lr >= 0) {
         const int e = a.ids[i];
         const int key = a.keyDiv == 1 ? e : e / a.keyDiv;
-        const int within = a.chunkBase[static_cast<int64_t>(i / kChunkRoutes) * a.numKeys + key] + lr;
+        const int within = a.chunkBase[static_cast<int64_t>(i >> a.chunkShift) * a.numKeys + key] + lr;
         if (a.capacity <= 0 || within < a.capacity) {
             row = a.keyOffset[key] + within;
             int32_t *tuple = a.assist + static_cast<int64_t>(row) * 4;

@@ -40,6 +40,7 @@ struct ReduceArgs {
     int h;
     int topK;
     void *y;
+    int colSlices;                   // slices a row is cut into (vec kernel, wide rows), else 1
     const uint64_t *tileFlags;
     int tileRows;
     const int32_t *totalRowsPtr;
@@ -148,12 +149,19 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 
     const int tg = threadIdx.x / G;
     const int lane = threadIdx.x % G;
+    constexpr int KB = V <= 2 ? 4 : (V <= 4 ? 2 : 1);      // rows in flight per lane
     const int vecs = a.h / 8;
-    const int groups = (a.bs + kTokens - 1) / kTokens;
+    // a unit is one token, or -- for wide rows -- one slice of G * V vectors of a token
+    const int units = a.bs * a.colSlices;
+    // the launch may use fewer waves per workgroup than kThreads / kWave (single-wave workgroups for sliced rows)
+    const int unitsPerGroup = static_cast<int>(blockDim.x) / G;
+    const int groups = (units + unitsPerGroup - 1) / unitsPerGroup;
 
     for (int group = blockIdx.x; group < groups; group += gridDim.x) {
-        const int token = group * kTokens + tg;
-        const bool tokOk = token < a.bs;
+        const int unit = group * unitsPerGroup + tg;
+        const bool tokOk = unit < units;
+        const int token = unit / a.colSlices;
+        const int colBase = (unit % a.colSlices) * (G * V);
         __syncthreads();        // the previous iteration's readers are done with s_row / s_w
         LoadRoutes(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
         __syncthreads();
@@ -174,53 +182,62 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             }
         }
         // control flow below is uniform across the lanes that share a token (the MXFP8 round trip shuffles)
-        for (int k = 0; k < a.topK; ++k) {
-            const int row = s_row[tg][k];
-            if (row < 0 || !active) {
-                continue;
-            }
-            const float w = s_w[tg][k];
-            const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row) * a.rowBytes;
-            u32x4 v16[V];
+        for (int k0 = 0; k0 < a.topK; k0 += KB) {
+            u32x4 v16[KB][V];
+            int rowOfK[KB];
 #pragma unroll
-            for (int j = 0; j < V; ++j) {
-                const int idx = j * G + lane;
-                v16[j] = idx < vecs ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) :
-                                      u32x4{0u, 0u, 0u, 0u};
-            }
+            for (int u = 0; u < KB; ++u) {
+                const int k = k0 + u;
+                const int row = (k < a.topK && active) ? s_row[tg][k] : -1;
+                rowOfK[u] = row;
+                const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
 #pragma unroll
-            for (int j = 0; j < V; ++j) {
-                float f[8];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    f[2 * q] = Decode16<BF16>(v16[j][q] & 0xffffu);
-                    f[2 * q + 1] = Decode16<BF16>(v16[j][q] >> 16);
+                for (int j = 0; j < V; ++j) {
+                    const int idx = colBase + j * G + lane;
+                    v16[u][j] = (row >= 0 && idx < vecs) ?
+                        __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) : u32x4{0u, 0u, 0u, 0u};
                 }
-                if (kMx) {
-                    float amax = 0.0f;
+            }
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        amax = fmaxf(amax, fabsf(f[e]));
-                    }
-                    amax = fmaxf(amax, __shfl_xor(amax, 1));
-                    amax = fmaxf(amax, __shfl_xor(amax, 2));
-                    const int se = MxSharedExponent<kCommE5m2>(amax);
-                    const float up = Exp2Int(se);
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        const float back = Fp8Decode<kCommE5m2>(Fp8Encode<kCommE5m2>(ldexpf(f[e], -se)));
-                        f[e] = __fmul_rn(back, up);
-                    }
+            for (int u = 0; u < KB; ++u) {
+                if (rowOfK[u] < 0) {
+                    continue;
                 }
-                if (KIND == kReducePerAdd) {
+                const float w = s_w[tg][k0 + u];
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        acc[j][e] = RoundTo16<BF16>(__fadd_rn(acc[j][e], f[e]));
+                for (int j = 0; j < V; ++j) {
+                    float f[8];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        f[2 * q] = Decode16<BF16>(v16[u][j][q] & 0xffffu);
+                        f[2 * q + 1] = Decode16<BF16>(v16[u][j][q] >> 16);
                     }
-                } else {
+                    if (kMx) {
+                        float amax = 0.0f;
 #pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        acc[j][e] = __fadd_rn(acc[j][e], __fmul_rn(f[e], w));
+                        for (int e = 0; e < 8; ++e) {
+                            amax = fmaxf(amax, fabsf(f[e]));
+                        }
+                        amax = fmaxf(amax, __shfl_xor(amax, 1));
+                        amax = fmaxf(amax, __shfl_xor(amax, 2));
+                        const int se = MxSharedExponent<kCommE5m2>(amax);
+                        const float up = Exp2Int(se);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float back = Fp8Decode<kCommE5m2>(Fp8Encode<kCommE5m2>(ldexpf(f[e], -se)));
+                            f[e] = __fmul_rn(back, up);
+                        }
+                    }
+                    if (KIND == kReducePerAdd) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            acc[j][e] = RoundTo16<BF16>(__fadd_rn(acc[j][e], f[e]));
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            acc[j][e] = __fadd_rn(acc[j][e], __fmul_rn(f[e], w));
+                        }
                     }
                 }
             }
@@ -230,7 +247,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                 static_cast<int64_t>(token) * a.h * 2);
 #pragma unroll
             for (int j = 0; j < V; ++j) {
-                const int idx = j * G + lane;
+                const int idx = colBase + j * G + lane;
                 if (idx < vecs) {
                     const u32x4 v = sx[idx];
 #pragma unroll
@@ -245,7 +262,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.y) + static_cast<int64_t>(token) * a.h * 2);
 #pragma unroll
             for (int j = 0; j < V; ++j) {
-                const int idx = j * G + lane;
+                const int idx = colBase + j * G + lane;
                 if (idx < vecs) {
                     u32x4 o;
 #pragma unroll
@@ -485,12 +502,15 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
 template <int G, int V, int KIND, bool BF16, int COMMQ>
 void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
 {
-    constexpr int kTokens = kThreads / G;
-    int grid = (a.bs + kTokens - 1) / kTokens;
-    if (gridLimit > 0 && grid > gridLimit) {
-        grid = gridLimit;
+    // sliced rows: one wave per workgroup, so that no wave waits at a barrier for another slice's rows
+    const int threads = a.colSlices > 1 ? G : kThreads;
+    const int perGroup = threads / G;
+    const int64_t units = static_cast<int64_t>(a.bs) * a.colSlices;
+    int grid = static_cast<int>((units + perGroup - 1) / perGroup);
+    if (gridLimit > 0 && grid > gridLimit * (kThreads / threads)) {
+        grid = gridLimit * (kThreads / threads);
     }
-    hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ>), dim3(grid), dim3(kThreads), 0, stream, a);
+    hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ>), dim3(grid), dim3(threads), 0, stream, a);
 }
 
 template <int G, int V, bool BF16>
@@ -567,6 +587,7 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     a.flagEpoch = l.flagEpoch;
     a.waitTimeoutTicks = l.waitTimeoutTicks;
     a.deviceStatus = l.deviceStatus;
+    a.colSlices = 1;
     // A kernel that waits on flags must never crowd out the producer it waits for: keep it to two workgroups per
     // compute unit (8 of 32 wave slots) and let it walk the tokens.
     const int gridLimit = l.tileFlags != nullptr ? 2 * (l.numComputeUnits > 0 ? l.numComputeUnits : 256) : 0;
@@ -591,16 +612,16 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
             LaunchQuant<kThreads, 4>(l, a, gridLimit);
         }
     } else if (plain) {
+        // a wave per token for narrow rows; wide rows are cut into slices of 128 vectors, one wave each (many small
+        // independent waves with four rows in flight each reach the highest gather bandwidth here)
+        a.colSlices = 1;
         if (vecs <= 2 * kWave) {
             LaunchByType<kWave, 2>(l, a, gridLimit);
         } else if (vecs <= 4 * kWave) {
             LaunchByType<kWave, 4>(l, a, gridLimit);
-        } else if (vecs <= 2 * kThreads) {
-            LaunchByType<kThreads, 2>(l, a, gridLimit);
-        } else if (vecs <= 4 * kThreads) {
-            LaunchByType<kThreads, 4>(l, a, gridLimit);
         } else {
-            LaunchByType<kThreads, 8>(l, a, gridLimit);
+            a.colSlices = static_cast<int>((vecs + 2 * kWave - 1) / (2 * kWave));
+            LaunchByType<kWave, 2>(l, a, gridLimit);
         }
     } else {
         int grid = static_cast<int>(l.bs);

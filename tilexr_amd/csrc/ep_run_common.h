@@ -51,6 +51,7 @@ inline CountScratch CarveCountScratch(void *base, const CountScratchLayout &plan
 {
     auto at = [base](int64_t off) { return reinterpret_cast<int32_t *>(static_cast<char *>(base) + off); };
     CountScratch s {};
+    s.chunkShift = plan.chunkShift;
     s.ticket = static_cast<uint32_t *>(base);
     s.localRank = at(plan.localRankOff);
     s.chunkHist = at(plan.chunkHistOff);
