@@ -46,7 +46,10 @@ def parse():
     p.add_argument("--overlap", action="store_true",
                    help="run combine on a second stream, consuming tiles through readiness flags while dispatch is "
                         "still writing rows")
-    p.add_argument("--tile-rows", type=int, default=256)
+    p.add_argument("--tile-rows", type=int, default=64)
+    p.add_argument("--no-overlap-leg", action="store_true",
+                   help="skip the extra, separately timed run of the other schedule that is reported under "
+                        "config.other_schedule")
     p.add_argument("--event-stride", type=int, default=10,
                    help="record the per-kernel events on every N-th timed step")
     p.add_argument("--calibrate-copy", action="store_true",
@@ -211,6 +214,27 @@ def main():
     dispatch_us = d_ev[0].elapsed_ms(d_ev[1]) * 1e3
     combine_us = d_ev[1].elapsed_ms(d_ev[2]) * 1e3
 
+    # the other schedule (overlapped when the timed one is serial, and the other way round), timed on its own after
+    # the main region so that both are on record; it is not part of `value`
+    other = None
+    if not args.no_overlap_leg:
+        other_step = step_serial if args.overlap else step_overlapped
+        other_steps = max(10, args.steps // 2)
+        for _ in range(5):
+            other_step()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(other_steps):
+            other_step()
+        torch.cuda.synchronize()
+        other_us = (time.perf_counter() - t1) / other_steps * 1e6
+        if status.item() != 0:
+            print("a tile-flag wait expired during the run", file=sys.stderr)
+            sys.exit(1)
+        other = {"schedule": "serial" if args.overlap else "overlapped via tile flags", "tile_rows": args.tile_rows,
+                 "steps": other_steps, "us_per_layer": round(other_us, 2),
+                 "GBps": round((dispatch_bytes + combine_bytes) / (other_us * 1e-6) / 1e9, 1)}
+
     ms_per_step = elapsed / args.steps * 1e3
     total_bytes = dispatch_bytes + combine_bytes
     gbps = total_bytes / (ms_per_step * 1e-3) / 1e9
@@ -238,7 +262,7 @@ def main():
         "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": dict(workloads.describe(w, ids), schedule="overlapped via tile flags" if args.overlap else "serial",
-                       kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+                       other_schedule=other, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
         "roofline": roofline, "kernels": kernels,
     }

@@ -128,8 +128,10 @@ struct TileXREpDispatchExOptions {
     int64_t activeMaskType;
     bool *xActiveMask;
     int32_t *rowIndexMapOut;      // optional [bs, topK]: row of each route in expandXOut, -1 when it has none
-    uint64_t *tileFlagsOut;       // optional readiness words, one per `tileRows` rows of expandXOut:
-                                  //      (epoch << 32) | rows landed, release-published at agent scope
+    uint64_t *tileFlagsOut;       // optional readiness words, one per `tileRows` rows of expandXOut: a word
+                                  //      becomes (epoch << 32) | rows in the tile, in one store, once every row of
+                                  //      the tile (payload and scales) is complete in memory for every compute
+                                  //      unit; until then it holds whatever an earlier epoch left (never cleared)
     int64_t tileRows;
     int64_t *epochOut;            // optional host pointer: receives the epoch the flags are tagged with
     void *metaReadyEvent;         // optional hipEvent_t recorded on `stream` once counts, assist tuples,
@@ -154,7 +156,10 @@ struct TileXREpCombineExOptions {
     bool *xActiveMask;
     void *sharedExpertX;          // optional [bs, h]
     const int32_t *rowIndexMap;   // optional [bs, topK] from dispatch: skips rebuilding the inverse map
-    const uint64_t *tileFlags;    // optional: wait (acquire, agent scope) for the tiles of each row read
+    const uint64_t *tileFlags;    // optional: before a row is read, wait until the upper half of its tile's word
+                                  //      equals flagEpoch; the rows are then read from memory, not from a cache.
+                                  //      A producer other than the dispatch above (an expert stage) completes its
+                                  //      rows with a release at agent scope, then stores the word
     int64_t tileRows;
     int64_t flagEpoch;            // epoch the producer tags its flag words with
     int64_t waitTimeoutUs;        // bound of every flag wait; 0 = library default (2 s)

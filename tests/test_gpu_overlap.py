@@ -72,6 +72,59 @@ def test_combine_overlapped_with_dispatch_through_tile_flags(shape, tile_rows):
         meta_ready.destroy()
 
 
+@pytest.mark.parametrize("quant", ["none", "int8", "fp8_block128"])
+def test_overlap_on_reused_buffers_never_reads_a_previous_round(quant):
+    """The same output buffers carry five different layers in a row, the consumer starts as early as it can and the
+    tiles are small, so rows are read a moment after another compute unit wrote them: a row served from a cache that
+    still holds the previous layer, or read before its stores have landed, shows up as a bit difference."""
+    bs, h, K, E, tile_rows = 4096, 2048, 8, 64, 8
+    qmode = {"none": ep.Q_NONE, "int8": ep.Q_TOKEN_INT8, "fp8_block128": ep.Q_FP8_BLOCK128}[quant]
+    oq = {"none": O.Q_NONE, "int8": O.Q_TOKEN_INT8, "fp8_block128": O.Q_FP8_BLOCK128}[quant]
+    rng = np.random.default_rng(4242 + qmode)
+    n = bs * K
+    tiles = (n + tile_rows - 1) // tile_rows
+    with Session() as s:
+        side = torch.cuda.Stream()
+        flags = torch.zeros((tiles,), dtype=torch.int64, device=DEV)
+        status = torch.zeros((1,), dtype=torch.int32, device=DEV)
+        meta_ready, consumed = ep.HipEvent(), ep.HipEvent()
+        out = alloc_dispatch_outputs(bs, h, K, E, quant=qmode)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        y = torch.zeros((bs, h), dtype=torch.bfloat16, device=DEV)
+        for round_ in range(5):
+            ids, w = routing(rng, bs, K, E)
+            x = torch.from_numpy((rng.standard_normal((bs, h)) * (1 + round_)).astype(np.float32)).to(torch.bfloat16)
+            xb = bits16(x)
+            d_x, d_ids, d_w = x.to(DEV), to_dev(ids), to_dev(w)
+            torch.cuda.synchronize()
+            st, epoch = ep.dispatch_memory_ex(d_x, d_ids, s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                              out["token_nums"], counts, ep.DT_BF16, s.stream, quant_mode=qmode,
+                                              dynamic_scales=out["scales"], row_index_map=out["row_map"],
+                                              tile_flags=flags, tile_rows=tile_rows, meta_ready_event=meta_ready.value)
+            assert st == 0
+            meta_ready.wait_on(side)
+            st = ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, side,
+                                      expert_out_quant_mode=qmode, expert_out_scales=out["scales"], expert_scales=d_w,
+                                      row_index_map=out["row_map"], tile_flags=flags, tile_rows=tile_rows,
+                                      flag_epoch=epoch, wait_timeout_us=5_000_000, device_status=status)
+            assert st == 0
+            consumed.record(side)
+            consumed.wait_on(s.stream)
+            s.sync()
+            side.synchronize()
+            assert status.item() == 0
+            case = O.Case(1, bs, h, K, E, dtype=O.DT_BF16, quant_mode=oq, token_nums_type=1)
+            want = O.mem_dispatch(case, 0, xb[None], ids[None])
+            assert np.array_equal(out["expand_x"].cpu().numpy(), want["expand_x"]), f"round {round_}"
+            eo = want["expand_x"][None] if oq else want["expand_x"].view(np.uint16)[None]
+            wy = O.mem_combine(O.Case(1, bs, h, K, E, dtype=O.DT_BF16), 0, eo, want["assist"][None],
+                               want["send_counts"][None], expert_scales=w, in_quant=oq,
+                               in_scales=want["dyn_scales"] if oq else None)
+            assert np.array_equal(bits16(y), wy), f"round {round_}"
+        meta_ready.destroy()
+        consumed.destroy()
+
+
 def test_flag_wait_expires_instead_of_hanging():
     bs, h, K, E = 256, 512, 4, 16
     rng = np.random.default_rng(9)

@@ -93,12 +93,9 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     place.expertIdBias = static_cast<int32_t>(p.sharedExpertNum);
     place.rowOf = rowOf;
     place.assist = p.assistInfoForCombineOut;
-    place.tileFlags = p.tileFlagsOut;
-    place.numTiles = p.tileFlagsOut != nullptr ? (n + p.tileRows - 1) / p.tileRows : 0;
-    place.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
     place.stream = stream;
-    // The scatter kernel can resolve the rows of its own tokens; a separate launch is only needed when something
-    // has to be complete before the first row lands (tile flags reset, assist tuples behind metaReadyEvent).
+    // The scatter kernel can resolve the rows of its own tokens; a separate launch is only needed when the row map
+    // and the assist tuples have to be complete before the first row lands (readiness flags, metaReadyEvent).
     const bool separatePlace = p.tileFlagsOut != nullptr || p.metaReadyEvent != nullptr;
     if (separatePlace) {
         ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
@@ -130,6 +127,15 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     scatter.scalesOut = p.dynamicScalesOut;
     scatter.tileFlags = p.tileFlagsOut;
     scatter.tileRows = p.tileRows;
+    scatter.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
+    scatter.totalRowsPtr = scratch.keyOffset + numKeys;
+    if (p.tileFlagsOut != nullptr && p.tileRows > 1) {
+        const int64_t tiles = (n + p.tileRows - 1) / p.tileRows;
+        if (!comm->tileCounters.Reserve(static_cast<size_t>(tiles) * sizeof(uint32_t), true)) {
+            return TileXR::TILEXR_ERROR_INTERNAL;
+        }
+        scatter.tileCounters = static_cast<uint32_t *>(comm->tileCounters.ptr);
+    }
     scatter.stream = stream;
     return Timed(comm, kKernelScatter, stream, "scatter", [&] { return LaunchScatter(scatter); });
 }
@@ -189,7 +195,6 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     red.y = p.yOut;
     red.tileFlags = p.tileFlags;
     red.tileRows = p.tileRows;
-    red.totalRowsPtr = p.epRecvCounts + (p.moeExpertNum - 1);
     red.flagEpoch = static_cast<uint64_t>(p.flagEpoch) & 0xffffffffull;
     red.waitTimeoutTicks = (p.waitTimeoutUs > 0 ? p.waitTimeoutUs : kDefaultWaitUs) * kWallClockTicksPerUs;
     red.deviceStatus = p.deviceStatusOut;

@@ -177,6 +177,7 @@ int TileXRCommDestroy(TileXRCommPtr comm)
     c->dispatchScratch.Release();
     c->combineScratch.Release();
     c->drainScratch.Release();
+    c->tileCounters.Release();
     if (c->dev != nullptr) {
         (void)hipFree(c->dev);
     }

@@ -105,6 +105,7 @@ struct EpComm {
     DeviceBuffer dispatchScratch;
     DeviceBuffer combineScratch;
     DeviceBuffer drainScratch;
+    DeviceBuffer tileCounters;        // rows landed per readiness tile; all zero whenever no dispatch is in flight
     hipEvent_t timing[5][2] = {};     // optional (start, stop) pairs around each kernel, see tilexr_ep.h
     std::mutex mu;
 };

@@ -304,25 +304,17 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
 }
 
 // -------------------------------------------------------------------------------------------------------------
-// place (stand-alone): destination row of every route + assist tuple + inverse map + tile-flag reset.  Used when
-// something must be complete before the scatter starts (tile flags reset, a metadata-ready event) or when the
-// rows go to a staging area; otherwise the scatter kernel resolves the rows of its own tokens (ep_place.cuh).
+// place (stand-alone): destination row of every route + assist tuple + inverse map.  Used when they must be complete
+// before the first row lands (readiness flags, a metadata-ready event) or when the rows go to a staging area;
+// otherwise the scatter kernel resolves the rows of its own tokens (ep_place.cuh).
 // -------------------------------------------------------------------------------------------------------------
 struct RoutePlaceArgs {
     PlaceArgs p;
-    uint64_t *tileFlags;
-    int numTiles;
-    uint64_t epoch;
 };
 
 __global__ __launch_bounds__(kThreads) void ep_route_place_kernel(RoutePlaceArgs a)
 {
     const int i = blockIdx.x * kThreads + threadIdx.x;
-    if (a.tileFlags != nullptr) {
-        for (int f = i; f < a.numTiles; f += gridDim.x * kThreads) {
-            a.tileFlags[f] = a.epoch << 32;
-        }
-    }
     if (i < a.p.n) {
         PlaceRoute(a.p, i);
     }
@@ -466,9 +458,6 @@ hipError_t LaunchRoutePlace(const RoutePlaceLaunch &l)
 {
     RoutePlaceArgs a {};
     a.p = MakePlaceArgs(l);
-    a.tileFlags = l.tileFlags;
-    a.numTiles = static_cast<int>(l.numTiles);
-    a.epoch = l.epoch;
     const int grid = (a.p.n + kThreads - 1) / kThreads;
     hipLaunchKernelGGL(ep_route_place_kernel, dim3(grid > 0 ? grid : 1), dim3(kThreads), 0, l.stream, a);
     return hipGetLastError();

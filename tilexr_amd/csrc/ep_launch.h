@@ -4,8 +4,8 @@
 // The data path of one dispatch is three launches on the caller's stream:
 //   count   per-chunk stable rank of every route within its key + per-chunk key histogram; the last workgroup
 //           to finish scans the histograms into per-chunk bases, per-key offsets and the count outputs
-//   place   destination row of every route, assist tuples, inverse row map, tile-flag reset (folded into the
-//           scatter launch when nothing has to be complete before the scatter starts)
+//   place   destination row of every route, assist tuples, inverse row map (folded into the scatter launch when
+//           nothing has to be complete before the scatter starts)
 //   scatter token rows read once and written to their topK destination rows (optionally quantised)
 // and of one combine two launches:
 //   invert  (skipped when the caller supplies the row map) row -> (token, k) inverse from the assist tuples
@@ -76,9 +76,6 @@ struct RoutePlaceLaunch {
     int32_t expertIdBias;        // added to the id stored in the assist tuple (shared experts shift ids)
     int32_t *rowOf;              // [n] out
     int32_t *assist;             // [rows, 4] out
-    uint64_t *tileFlags;         // optional
-    int64_t numTiles;
-    uint64_t epoch;
     hipStream_t stream;
 };
 
@@ -95,8 +92,16 @@ struct ScatterLaunch {
     const float *staticScale;
     void *out;                   // rows of h*2 bytes (mode 0) or h bytes
     void *scalesOut;             // fp32 [rows] (2), u8 [rows, mxScaleCount] (4), fp32 [rows, ceil(h/128)] (5)
-    uint64_t *tileFlags;         // optional: +1 (release, agent scope) on the row's tile after each row
+    // Optional readiness words, one per `tileRows` rows: (epoch << 32) | rows in the tile, stored once, by whoever
+    // lands the tile's last row, after every row of the tile is complete in memory.  Landed rows are counted in
+    // `tileCounters` (library scratch, all zero between launches), never in the words consumers poll: a poll of a
+    // word that atomics are hitting holds those atomics up (measured: 20 000 polls slow the scatter from 95 to
+    // 215 us), a poll of a word that is stored once costs the producer nothing.
+    uint64_t *tileFlags;
+    uint32_t *tileCounters;      // [ceil(rows / tileRows)], unused when tileRows == 1
     int64_t tileRows;
+    uint64_t epoch;
+    const int32_t *totalRowsPtr; // device word: rows kept by this dispatch (size of the last tile)
     hipStream_t stream;
 };
 
@@ -139,9 +144,8 @@ struct ReduceLaunch {
     int64_t h;
     int64_t topK;
     void *y;
-    const uint64_t *tileFlags;       // optional
+    const uint64_t *tileFlags;       // optional: a tile is ready once the upper half of its word equals flagEpoch
     int64_t tileRows;
-    const int32_t *totalRowsPtr;     // device word holding the number of valid rows (for the last tile's size)
     uint64_t flagEpoch;
     int64_t waitTimeoutTicks;        // in wall_clock64 ticks
     int32_t *deviceStatus;

@@ -43,7 +43,6 @@ struct ReduceArgs {
     int colSlices;                   // slices a row is cut into (vec kernel, wide rows), else 1
     const uint64_t *tileFlags;
     int tileRows;
-    const int32_t *totalRowsPtr;
     uint64_t flagEpoch;
     int64_t waitTimeoutTicks;
     int32_t *deviceStatus;
@@ -58,19 +57,20 @@ __device__ __forceinline__ int LookupRow(const ReduceArgs &a, int64_t slot)
     return (e >> 32) == a.epoch ? static_cast<int>(e & 0xffffffffu) : -1;
 }
 
-// Bounded wait until the tile holding `row` has all its rows published for this epoch.  The poll itself is a relaxed
+// Bounded wait until the tile holding `row` has been published for this epoch (its word carries the epoch).  The poll itself is a relaxed
 // device-scope load (no cache maintenance per iteration -- an acquire in the loop would invalidate this XCD's L2 on
-// every spin and starve the producer); the caller issues one acquire fence after all its waits have succeeded.
+// every spin and starve the producer).  What the caller reads afterwards must not come from a stale L2 line: the
+// register-resident kernels read published rows with agent-scope loads, which are served from memory; the
+// element-granular kernel issues one acquire fence after all its waits have succeeded.
 __device__ bool WaitTile(const ReduceArgs &a, int row)
 {
     const int tile = row / a.tileRows;
-    const int total = *a.totalRowsPtr;
-    int need = total - tile * a.tileRows;
-    need = need > a.tileRows ? a.tileRows : need;
     const uint64_t start = wall_clock64();
+    // every poll is a round trip to memory (agent scope): the gap between polls doubles up to about 3 us
+    int backoff = 0;
     while (true) {
         const uint64_t w = __hip_atomic_load(&a.tileFlags[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((w >> 32) == a.flagEpoch && static_cast<int>(w & 0xffffffffu) >= need) {
+        if ((w >> 32) == a.flagEpoch) {
             return true;
         }
         if (static_cast<int64_t>(wall_clock64() - start) > a.waitTimeoutTicks) {
@@ -82,7 +82,14 @@ __device__ bool WaitTile(const ReduceArgs &a, int row)
             __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
             return false;
         }
-        __builtin_amdgcn_s_sleep(16);
+        switch (backoff) {                  // s_sleep takes an immediate: 64 clocks per unit
+            case 0: __builtin_amdgcn_s_sleep(8); break;
+            case 1: __builtin_amdgcn_s_sleep(16); break;
+            case 2: __builtin_amdgcn_s_sleep(32); break;
+            case 3: __builtin_amdgcn_s_sleep(64); break;
+            default: __builtin_amdgcn_s_sleep(127); break;
+        }
+        backoff += backoff < 4 ? 1 : 0;
     }
 }
 
@@ -115,7 +122,29 @@ __device__ void SortRows(int *rows, int k, const uint64_t *orderKeys)
     }
 }
 
+// Row loads of the register-resident kernels.  FL = false: non-temporal loads.  FL = true (rows published through
+// readiness flags, possibly a moment ago by a workgroup on another XCD): agent-scope loads, served from memory, so
+// that no acquire fence (an invalidate of this XCD's whole L2) is needed per token.
+template <bool FL>
+__device__ __forceinline__ u32x4 RowLoad(const char *rowBase, __amdgpu_buffer_rsrc_t rsrc, int byteOffset)
+{
+    if (FL) {
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc, byteOffset, 0, kAuxAgentScope);
+    }
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(rowBase + byteOffset));
+}
+
+template <bool FL>
+__device__ __forceinline__ float ScaleLoad(const float *p)
+{
+    if (FL) {
+        return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return *p;
+}
+
 // Fills s_row / s_w for one token; waits for tile flags when asked to.
+template <bool FENCE>
 __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
     float *weights)
 {
@@ -131,14 +160,14 @@ __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool 
         rows[k] = row;
         weights[k] = (tokOk && a.expertScales != nullptr) ? a.expertScales[slot] : 1.0f;
     }
-    if (a.tileFlags != nullptr && lane < a.topK) {
+    if (FENCE && a.tileFlags != nullptr && lane < a.topK) {
         // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
         // workgroup after the barrier that follows) are at least as new as the flag values seen above
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
 }
 
-template <int G, int V, int KIND, bool BF16, int COMMQ>
+template <int G, int V, int KIND, bool BF16, int COMMQ, bool FL>
 __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 {
     constexpr int kTokens = kThreads / G;
@@ -163,7 +192,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
         const int token = unit / a.colSlices;
         const int colBase = (unit % a.colSlices) * (G * V);
         __syncthreads();        // the previous iteration's readers are done with s_row / s_w
-        LoadRoutes(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
+        LoadRoutes<false>(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
         __syncthreads();
         if (KIND == kReducePerAdd) {
             if (lane == 0) {
@@ -188,14 +217,15 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 #pragma unroll
             for (int u = 0; u < KB; ++u) {
                 const int k = k0 + u;
-                const int row = (k < a.topK && active) ? s_row[tg][k] : -1;
+                // the lanes of a wave share one token, so the row is wave-uniform
+                const int row = __builtin_amdgcn_readfirstlane((k < a.topK && active) ? s_row[tg][k] : -1);
                 rowOfK[u] = row;
                 const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
+                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
                     const int idx = colBase + j * G + lane;
-                    v16[u][j] = (row >= 0 && idx < vecs) ?
-                        __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) : u32x4{0u, 0u, 0u, 0u};
+                    v16[u][j] = (row >= 0 && idx < vecs) ? RowLoad<FL>(base, rsrc, idx * 16) : u32x4{0u, 0u, 0u, 0u};
                 }
             }
 #pragma unroll
@@ -280,7 +310,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 // columns.  Each value is dequantised, rounded to the output element type, then accumulated exactly like an ordinary
 // row (fp32, k order, separate multiply and add).  Rows are a quarter the bytes of bf16 rows, so a lane owns 16
 // consecutive columns per vector (one 16-byte load) and KB rows are kept in flight at once.
-template <int G, int V, int INQ, bool BF16>
+template <int G, int V, int INQ, bool BF16, bool FL>
 __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
 {
     constexpr int kTokens = kThreads / G;
@@ -298,7 +328,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
         const int token = group * kTokens + tg;
         const bool tokOk = token < a.bs;
         __syncthreads();
-        LoadRoutes(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
+        LoadRoutes<false>(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
         __syncthreads();
         const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0);
 
@@ -317,17 +347,17 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
 #pragma unroll
             for (int u = 0; u < KB; ++u) {
                 const int k = k0 + u;
-                const int row = (k < a.topK && active) ? s_row[tg][k] : -1;
+                const int row = __builtin_amdgcn_readfirstlane((k < a.topK && active) ? s_row[tg][k] : -1);
                 rowOfK[u] = row;
                 const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
+                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
                     const int idx = j * G + lane;
                     const bool live = row >= 0 && idx < vecs;
-                    q[u][j] = live ? __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(base) + idx) :
-                                     u32x4{0u, 0u, 0u, 0u};
-                    sc[u][j] = !live ? 0.0f : (INQ == TILEXR_EP_QUANT_TOKEN_INT8 ? a.inScales[row] :
-                        a.inScales[static_cast<int64_t>(row) * b128 + (idx >> 3)]);
+                    q[u][j] = live ? RowLoad<FL>(base, rsrc, idx * 16) : u32x4{0u, 0u, 0u, 0u};
+                    sc[u][j] = !live ? 0.0f : (INQ == TILEXR_EP_QUANT_TOKEN_INT8 ? ScaleLoad<FL>(a.inScales + row) :
+                        ScaleLoad<FL>(a.inScales + static_cast<int64_t>(row) * b128 + (idx >> 3)));
                 }
             }
 #pragma unroll
@@ -424,7 +454,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
     const int b128 = (a.h + 127) / 128;
     for (int token = blockIdx.x; token < a.bs; token += gridDim.x) {
         __syncthreads();
-        LoadRoutes(a, token, true, tid, kThreads, s_row, s_w);
+        LoadRoutes<true>(a, token, true, tid, kThreads, s_row, s_w);
         __syncthreads();
         if (kind == kReducePerAdd) {
             if (tid == 0) {
@@ -502,6 +532,15 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
 template <int G, int V, int KIND, bool BF16, int COMMQ>
 void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
 {
+    if constexpr (G == kThreads) {
+        // whole-workgroup tokens are only used for rows published through readiness flags
+        int grid = a.bs;
+        if (gridLimit > 0 && grid > gridLimit) {
+            grid = gridLimit;
+        }
+        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, true>), dim3(grid), dim3(kThreads), 0, stream, a);
+        return;
+    }
     // sliced rows: one wave per workgroup, so that no wave waits at a barrier for another slice's rows
     const int threads = a.colSlices > 1 ? G : kThreads;
     const int perGroup = threads / G;
@@ -510,7 +549,11 @@ void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
     if (gridLimit > 0 && grid > gridLimit * (kThreads / threads)) {
         grid = gridLimit * (kThreads / threads);
     }
-    hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ>), dim3(grid), dim3(threads), 0, stream, a);
+    if (a.tileFlags != nullptr) {
+        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, true>), dim3(grid), dim3(threads), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, false>), dim3(grid), dim3(threads), 0, stream, a);
+    }
 }
 
 template <int G, int V, bool BF16>
@@ -537,6 +580,24 @@ void LaunchByType(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
     }
 }
 
+template <int G, int V, int INQ>
+void LaunchQuantKernel(const ReduceLaunch &l, const ReduceArgs &a, dim3 g, dim3 b)
+{
+    if (l.bf16) {
+        if (a.tileFlags != nullptr) {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, INQ, true, true>), g, b, 0, l.stream, a);
+        } else {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, INQ, true, false>), g, b, 0, l.stream, a);
+        }
+    } else {
+        if (a.tileFlags != nullptr) {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, INQ, false, true>), g, b, 0, l.stream, a);
+        } else {
+            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, INQ, false, false>), g, b, 0, l.stream, a);
+        }
+    }
+}
+
 template <int G, int V>
 void LaunchQuant(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
 {
@@ -548,17 +609,9 @@ void LaunchQuant(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
     const dim3 g(grid);
     const dim3 b(kThreads);
     if (l.inQuant == TILEXR_EP_QUANT_TOKEN_INT8) {
-        if (l.bf16) {
-            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_TOKEN_INT8, true>), g, b, 0, l.stream, a);
-        } else {
-            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_TOKEN_INT8, false>), g, b, 0, l.stream, a);
-        }
+        LaunchQuantKernel<G, V, TILEXR_EP_QUANT_TOKEN_INT8>(l, a, g, b);
     } else {
-        if (l.bf16) {
-            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_FP8_BLOCK128, true>), g, b, 0, l.stream, a);
-        } else {
-            hipLaunchKernelGGL((ep_reduce_quant_kernel<G, V, TILEXR_EP_QUANT_FP8_BLOCK128, false>), g, b, 0, l.stream, a);
-        }
+        LaunchQuantKernel<G, V, TILEXR_EP_QUANT_FP8_BLOCK128>(l, a, g, b);
     }
 }
 
@@ -583,13 +636,13 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     a.y = l.y;
     a.tileFlags = l.tileFlags;
     a.tileRows = static_cast<int>(l.tileRows);
-    a.totalRowsPtr = l.totalRowsPtr;
     a.flagEpoch = l.flagEpoch;
     a.waitTimeoutTicks = l.waitTimeoutTicks;
     a.deviceStatus = l.deviceStatus;
     a.colSlices = 1;
-    // A kernel that waits on flags must never crowd out the producer it waits for: keep it to two workgroups per
-    // compute unit (8 of 32 wave slots) and let it walk the tokens.
+    // A kernel that waits on flags must never crowd out the producer it waits for: its waiting waves keep their
+    // registers, and with three or more of these workgroups per compute unit a producer workgroup no longer fits
+    // beside them (measured: flag waits expire at six).  Two workgroups per compute unit walk the tokens.
     const int gridLimit = l.tileFlags != nullptr ? 2 * (l.numComputeUnits > 0 ? l.numComputeUnits : 256) : 0;
     const int64_t vecs = l.h / 8;
     const bool plain = l.inQuant == 0 && l.h % 8 == 0 && Aligned16(l.y) && vecs <= 8 * kThreads &&
@@ -619,6 +672,16 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
             LaunchByType<kWave, 2>(l, a, gridLimit);
         } else if (vecs <= 4 * kWave) {
             LaunchByType<kWave, 4>(l, a, gridLimit);
+        } else if (a.tileFlags != nullptr) {
+            // readiness flags: one workgroup per token, so that one wave polls the token's tiles instead of one per
+            // slice (waiters on a hot flag word slow down the producer's atomics on it)
+            if (vecs <= 2 * kThreads) {
+                LaunchByType<kThreads, 2>(l, a, gridLimit);
+            } else if (vecs <= 4 * kThreads) {
+                LaunchByType<kThreads, 4>(l, a, gridLimit);
+            } else {
+                LaunchByType<kThreads, 8>(l, a, gridLimit);
+            }
         } else {
             a.colSlices = static_cast<int>((vecs + 2 * kWave - 1) / (2 * kWave));
             LaunchByType<kWave, 2>(l, a, gridLimit);

@@ -34,7 +34,10 @@ struct ScatterArgs {
     void *out;
     void *scalesOut;
     uint64_t *tileFlags;
+    uint32_t *tileCounters;
     int tileRows;
+    uint64_t epoch;
+    const int32_t *totalRowsPtr;
 };
 
 __device__ __forceinline__ int RowOfRoute(const ScatterArgs &a, int route)
@@ -60,17 +63,78 @@ __device__ __forceinline__ float GroupMax(float v, float *red, int lane)
     return v;
 }
 
-__device__ __forceinline__ void PublishRows(uint64_t *tileFlags, int tileRows, const int *pos, int topK, int lane, int G)
+// Row stores of the register-resident kernels.  WT = false: non-temporal stores (the rows are not read again by this
+// kernel).  WT = true: agent-scope write-through stores, used when readiness flags are published: such a store is
+// complete for every XCD once the issuing wave's vmcnt is zero, so publishing needs no L2 write-back.
+template <bool WT>
+__device__ __forceinline__ void RowStore(const u32x4 &v, char *rowBase, __amdgpu_buffer_rsrc_t rsrc, int byteOffset)
 {
-    // every lane's row stores have been issued once the workgroup barrier has been passed; one release fence per
-    // lane that publishes (not one per row) makes them visible at device scope before the tile counters move
-    __syncthreads();
-    if (lane < topK) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-        for (int k = lane; k < topK; k += G) {
+    if (WT) {
+        __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, byteOffset, 0, kAuxAgentScope);
+    } else {
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(rowBase + byteOffset));
+    }
+}
+
+template <bool WT>
+__device__ __forceinline__ void RowStore(const u32x2 &v, char *rowBase, __amdgpu_buffer_rsrc_t rsrc, int byteOffset)
+{
+    if (WT) {
+        __builtin_amdgcn_raw_buffer_store_b64(v, rsrc, byteOffset, 0, kAuxAgentScope);
+    } else {
+        __builtin_nontemporal_store(v, reinterpret_cast<u32x2 *>(rowBase + byteOffset));
+    }
+}
+
+template <bool WT, typename T>
+__device__ __forceinline__ void ScalarStore(T *p, T v)
+{
+    if (WT) {
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    } else {
+        *p = v;
+    }
+}
+
+// Counts one landed row; whoever lands the last row of a tile stores the tile's readiness word (and leaves the counter
+// at zero for the next dispatch).  The caller has made the row complete in memory first, so has every earlier counter
+// of the tile, and the atomics on one counter are totally ordered: when the last one returns, all rows of the tile are
+// in memory.  The words consumers poll are only ever stored to, never hit by atomics.
+__device__ __forceinline__ void PublishRow(const ScatterArgs &a, int row)
+{
+    const int tile = row / a.tileRows;
+    int rowsInTile = 1;
+    if (a.tileRows > 1) {
+        const int left = *a.totalRowsPtr - tile * a.tileRows;
+        rowsInTile = left < a.tileRows ? left : a.tileRows;
+        const uint32_t before = __hip_atomic_fetch_add(&a.tileCounters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (static_cast<int>(before) + 1 != rowsInTile) {
+            return;
+        }
+        __hip_atomic_store(&a.tileCounters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __hip_atomic_store(&a.tileFlags[tile], (a.epoch << 32) | static_cast<uint32_t>(rowsInTile), __ATOMIC_RELAXED,
+        __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Publishes the rows of one token.  Each wave waits for its own stores and the barrier collects the waves.
+// WT = true: the rows were written through and are then complete.  WT = false: the rows may still sit dirty in this
+// XCD's L2 and one release fence per publishing wave writes them back (slow under load; element-granular fallback only).
+template <bool WT>
+__device__ __forceinline__ void PublishRows(const ScatterArgs &a, const int *pos, int lane, int G)
+{
+    WaitOwnStores();
+    if (G > kWave) {
+        __syncthreads();
+    }
+    if (lane < a.topK) {
+        if (!WT) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+        }
+        for (int k = lane; k < a.topK; k += G) {
             const int row = pos[k];
             if (row >= 0) {
-                __hip_atomic_fetch_add(&tileFlags[row / tileRows], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                PublishRow(a, row);
             }
         }
     }
@@ -82,7 +146,7 @@ __device__ __forceinline__ void PublishRows(uint64_t *tileFlags, int tileRows, c
 // times.  One row per workgroup keeps every wave at V stores in flight, which this memory system rewards: measured
 // 89 us against 93 us for "one workgroup writes all topK rows" on 4096 x 7168 x top-8, and 132 us when the
 // workgroups of a token are spread over the XCDs.
-template <int V>
+template <int V, bool WT>
 __global__ __launch_bounds__(kThreads) void ep_scatter_route_kernel(ScatterArgs a)
 {
     constexpr int kXcds = 8;
@@ -107,28 +171,29 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_route_kernel(ScatterArgs 
         v[i] = idx < vecs ? src[idx] : u32x4{0u, 0u, 0u, 0u};
     }
     __syncthreads();
-    const int row = s_row;
+    const int row = __builtin_amdgcn_readfirstlane(s_row);
     if (row < 0) {
         return;
     }
-    u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2);
+    char *dst = static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2;
+    const __amdgpu_buffer_rsrc_t rsrc = RowResource(dst, vecs * 16);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
         const int idx = i * kThreads + lane;
         if (idx < vecs) {
-            __builtin_nontemporal_store(v[i], dst + idx);
+            RowStore<WT>(v[i], dst, rsrc, idx * 16);
         }
     }
-    if (a.tileFlags != nullptr) {
+    if (WT && a.tileFlags != nullptr) {
+        WaitOwnStores();
         __syncthreads();
         if (lane == 0) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-            __hip_atomic_fetch_add(&a.tileFlags[row / a.tileRows], 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            PublishRow(a, row);
         }
     }
 }
 
-template <int G, int V, int QMODE, bool BF16, bool E5M2>
+template <int G, int V, int QMODE, bool BF16, bool E5M2, bool WT>
 __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
 {
     constexpr int kTokens = kThreads / G;
@@ -156,16 +221,18 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
 
     if (QMODE == TILEXR_EP_QUANT_NONE) {
         for (int k = 0; k < a.topK; ++k) {
-            const int row = s_pos[tg][k];
+            // the lanes of a wave share one token, so the row is wave-uniform
+            const int row = __builtin_amdgcn_readfirstlane(s_pos[tg][k]);
             if (row < 0) {
                 continue;
             }
-            u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2);
+            char *dst = static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2;
+            const __amdgpu_buffer_rsrc_t rsrc = RowResource(dst, vecs * 16);
 #pragma unroll
             for (int j = 0; j < V; ++j) {
                 const int idx = j * G + lane;
                 if (idx < vecs) {
-                    __builtin_nontemporal_store(v[j], dst + idx);
+                    RowStore<WT>(v[j], dst, rsrc, idx * 16);
                 }
             }
         }
@@ -244,35 +311,37 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
         const int mxScales = (mxBlocks + 1) / 2 * 2;
         const int b128 = (a.h + 127) / 128;
         for (int k = 0; k < a.topK; ++k) {
-            const int row = s_pos[tg][k];
+            const int row = __builtin_amdgcn_readfirstlane(s_pos[tg][k]);
             if (row < 0) {
                 continue;
             }
-            u32x2 *dst = reinterpret_cast<u32x2 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h);
+            char *dst = static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h;
+            const __amdgpu_buffer_rsrc_t rsrc = RowResource(dst, vecs * 8);
 #pragma unroll
             for (int j = 0; j < V; ++j) {
                 const int idx = j * G + lane;
                 if (idx < vecs) {
-                    __builtin_nontemporal_store(q[j], dst + idx);
+                    RowStore<WT>(q[j], dst, rsrc, idx * 8);
                     if (QMODE == TILEXR_EP_QUANT_MXFP8 && (idx & 3) == 0) {
                         uint8_t *sc = static_cast<uint8_t *>(a.scalesOut) + static_cast<int64_t>(row) * mxScales;
-                        sc[idx >> 2] = static_cast<uint8_t>(sharedExp[j] + 127);
+                        ScalarStore<WT>(sc + (idx >> 2), static_cast<uint8_t>(sharedExp[j] + 127));
                         if ((idx >> 2) + 1 == mxBlocks && mxBlocks < mxScales) {
-                            sc[mxBlocks] = 0;       // padding byte of an odd block count
+                            ScalarStore<WT>(sc + mxBlocks, static_cast<uint8_t>(0));    // padding byte of an odd block count
                         }
                     }
                     if (QMODE == TILEXR_EP_QUANT_FP8_BLOCK128 && (idx & 15) == 0) {
-                        static_cast<float *>(a.scalesOut)[static_cast<int64_t>(row) * b128 + (idx >> 4)] = blockScale[j];
+                        ScalarStore<WT>(static_cast<float *>(a.scalesOut) + static_cast<int64_t>(row) * b128 + (idx >> 4),
+                            blockScale[j]);
                     }
                 }
             }
             if (QMODE == TILEXR_EP_QUANT_TOKEN_INT8 && lane == 0) {
-                static_cast<float *>(a.scalesOut)[row] = rowScale;
+                ScalarStore<WT>(static_cast<float *>(a.scalesOut) + row, rowScale);
             }
         }
     }
-    if (a.tileFlags != nullptr) {
-        PublishRows(a.tileFlags, a.tileRows, s_pos[tg], a.topK, lane, G);
+    if (WT && a.tileFlags != nullptr) {
+        PublishRows<true>(a, s_pos[tg], lane, G);
     }
 }
 
@@ -361,8 +430,14 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_generic_kernel(ScatterArg
         }
     }
     if (a.tileFlags != nullptr) {
-        PublishRows(a.tileFlags, a.tileRows, s_pos, a.topK, tid, kThreads);
+        PublishRows<false>(a, s_pos, tid, kThreads);
     }
+}
+
+// Rows move with write-through stores when readiness flags are published (see RowStore).
+inline bool WriteThrough(const ScatterArgs &a)
+{
+    return a.tileFlags != nullptr;
 }
 
 template <int G, int V, int QMODE, bool BF16, bool E5M2>
@@ -370,7 +445,11 @@ void LaunchVec(const ScatterArgs &a, hipStream_t stream)
 {
     constexpr int kTokens = kThreads / G;
     const int grid = (a.bs + kTokens - 1) / kTokens;
-    hipLaunchKernelGGL((ep_scatter_vec_kernel<G, V, QMODE, BF16, E5M2>), dim3(grid), dim3(kThreads), 0, stream, a);
+    if (WriteThrough(a)) {
+        hipLaunchKernelGGL((ep_scatter_vec_kernel<G, V, QMODE, BF16, E5M2, true>), dim3(grid), dim3(kThreads), 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((ep_scatter_vec_kernel<G, V, QMODE, BF16, E5M2, false>), dim3(grid), dim3(kThreads), 0, stream, a);
+    }
 }
 
 template <int G, int V>
@@ -381,9 +460,12 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
             // small batches are latency-bound and gain nothing from the extra workgroups
             if (G == kThreads && a.topK > 1 && a.bs >= 1024 &&
                 static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK <= 0x7fffffff) {
-                const int64_t blocks = static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK;
-                hipLaunchKernelGGL((ep_scatter_route_kernel<V>), dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0,
-                    l.stream, a);
+                const dim3 blocks(static_cast<unsigned>(static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK));
+                if (WriteThrough(a)) {
+                    hipLaunchKernelGGL((ep_scatter_route_kernel<V, true>), blocks, dim3(kThreads), 0, l.stream, a);
+                } else {
+                    hipLaunchKernelGGL((ep_scatter_route_kernel<V, false>), blocks, dim3(kThreads), 0, l.stream, a);
+                }
             } else {
                 LaunchVec<G, V, TILEXR_EP_QUANT_NONE, true, false>(a, l.stream);
             }
@@ -440,7 +522,10 @@ hipError_t LaunchScatter(const ScatterLaunch &l)
     a.out = l.out;
     a.scalesOut = l.scalesOut;
     a.tileFlags = l.tileFlags;
+    a.tileCounters = l.tileCounters;
     a.tileRows = static_cast<int>(l.tileRows);
+    a.epoch = l.epoch;
+    a.totalRowsPtr = l.totalRowsPtr;
     const int64_t vecs = l.h / 8;
     const bool vecOk = l.h % 8 == 0 && Aligned16(l.x) && vecs <= 8 * kThreads &&
         (l.quantMode == TILEXR_EP_QUANT_NONE ? Aligned16(l.out) : Aligned8(l.out));

@@ -240,7 +240,6 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     place.expertIdBias = 0;
     place.rowOf = rowOf;
     place.assist = reinterpret_cast<int32_t *>(myAux);
-    place.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
     place.stream = stream;
     ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
     if (ret != kOk) {
