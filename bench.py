@@ -196,6 +196,7 @@ def main():
             step()
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - t0
+    kernel_names = {"scatter": ep.last_kernel_name(comm, ep.K_SCATTER), "reduce": ep.last_kernel_name(comm, ep.K_REDUCE)}
 
     if args.overlap and status.item() != 0:
         print("a tile-flag wait expired during the run", file=sys.stderr)
@@ -249,7 +250,7 @@ def main():
                              "max_us": round(times[-1], 2), "launches_timed": len(times), "algorithmic_bytes": nbytes,
                              "achieved_GBps": round(nbytes / (avg * 1e-6) / 1e9, 1)}
         dom = "scatter" if kernels["scatter"]["avg_us"] >= kernels["reduce"]["avg_us"] else "reduce"
-        roofline = {"bound": "hbm", "kernel": "ep_scatter_vec_kernel" if dom == "scatter" else "ep_reduce_vec_kernel",
+        roofline = {"bound": "hbm", "kernel": kernel_names[dom],
                     "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                     "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4),
                     "traffic": measured_traffic(w.name, dom),

@@ -178,6 +178,11 @@ int TileXRMoeEpCombineMemoryEx(void *expertOut, int32_t *assistInfoForCombine, i
 // the stream of the call.  Pass null events to clear.  Kernel ids: 0 count, 1 place, 2 scatter, 3 invert, 4 reduce.
 int TileXREpSetKernelTimingEvents(TileXRCommPtr comm, int kernel, void *startEvent, void *stopEvent);
 
+// Measurement aid without a reference counterpart: name of the kernel template the last call on `comm` launched
+// for a kernel id (the data kernels have several templates, chosen by row width, alignment and payload type), so
+// that a harness can match its event timings with a profiler's per-kernel rows.  Null before the first launch.
+const char *TileXREpLastKernelName(TileXRCommPtr comm, int kernel);
+
 // Library build identification ("tilexr-ep gfx950 <abi version>").
 const char *TileXREpVersion(void);
 

@@ -129,13 +129,14 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     scatter.tileRows = p.tileRows;
     scatter.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
     scatter.totalRowsPtr = scratch.keyOffset + numKeys;
-    if (p.tileFlagsOut != nullptr && p.tileRows > 1) {
+    if (p.tileFlagsOut != nullptr) {
         const int64_t tiles = (n + p.tileRows - 1) / p.tileRows;
         if (!comm->tileCounters.Reserve(static_cast<size_t>(tiles) * sizeof(uint32_t), true)) {
             return TileXR::TILEXR_ERROR_INTERNAL;
         }
         scatter.tileCounters = static_cast<uint32_t *>(comm->tileCounters.ptr);
     }
+    scatter.kernelNameOut = &comm->lastKernel[kKernelScatter];
     scatter.stream = stream;
     return Timed(comm, kKernelScatter, stream, "scatter", [&] { return LaunchScatter(scatter); });
 }
@@ -199,6 +200,7 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     red.waitTimeoutTicks = (p.waitTimeoutUs > 0 ? p.waitTimeoutUs : kDefaultWaitUs) * kWallClockTicksPerUs;
     red.deviceStatus = p.deviceStatusOut;
     red.numComputeUnits = comm->world->numComputeUnits;
+    red.kernelNameOut = &comm->lastKernel[kKernelReduce];
     red.stream = stream;
     return Timed(comm, kKernelReduce, stream, "reduce", [&] { return LaunchReduce(red); });
 }
@@ -397,6 +399,18 @@ int TileXREpSetKernelTimingEvents(TileXRCommPtr comm, int kernel, void *startEve
     c->timing[kernel][0] = static_cast<hipEvent_t>(startEvent);
     c->timing[kernel][1] = static_cast<hipEvent_t>(stopEvent);
     return TileXR::TILEXR_SUCCESS;
+}
+
+const char *TileXREpLastKernelName(TileXRCommPtr comm, int kernel)
+{
+    EpComm *c = LookupComm(comm);
+    if (c == nullptr || kernel < 0 || kernel > kKernelReduce) {
+        return nullptr;
+    }
+    static const char *const fixed[5] = {"ep_route_count_kernel", "ep_route_place_kernel", nullptr, "ep_invert_kernel",
+        nullptr};
+    std::lock_guard<std::mutex> lock(c->mu);
+    return fixed[kernel] != nullptr ? fixed[kernel] : c->lastKernel[kernel];
 }
 
 int TileXRMoeEpDispatchV2(void *x, int32_t *expertIds, void *scales, bool *xActiveMask, void *expertScales,

@@ -107,6 +107,7 @@ struct EpComm {
     DeviceBuffer drainScratch;
     DeviceBuffer tileCounters;        // rows landed per readiness tile; all zero whenever no dispatch is in flight
     hipEvent_t timing[5][2] = {};     // optional (start, stop) pairs around each kernel, see tilexr_ep.h
+    const char *lastKernel[5] = {};   // name of the kernel template last launched for each kernel id
     std::mutex mu;
 };
 

@@ -98,10 +98,11 @@ struct ScatterLaunch {
     // word that atomics are hitting holds those atomics up (measured: 20 000 polls slow the scatter from 95 to
     // 215 us), a poll of a word that is stored once costs the producer nothing.
     uint64_t *tileFlags;
-    uint32_t *tileCounters;      // [ceil(rows / tileRows)], unused when tileRows == 1
+    uint32_t *tileCounters;      // [ceil(rows / tileRows)]
     int64_t tileRows;
     uint64_t epoch;
     const int32_t *totalRowsPtr; // device word: rows kept by this dispatch (size of the last tile)
+    const char **kernelNameOut;  // optional: receives the name of the kernel template that was launched
     hipStream_t stream;
 };
 
@@ -150,6 +151,7 @@ struct ReduceLaunch {
     int64_t waitTimeoutTicks;        // in wall_clock64 ticks
     int32_t *deviceStatus;
     int numComputeUnits;
+    const char **kernelNameOut;      // optional: receives the name of the kernel template that was launched
     hipStream_t stream;
 };
 

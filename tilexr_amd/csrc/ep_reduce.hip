@@ -652,6 +652,9 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     const bool quant = l.inQuant != 0 && l.commQuant == 0 && l.reduceKind == kReduceFp32 && l.h % 16 == 0 &&
         qvecs <= 4 * kThreads && Aligned16(l.y) && Aligned16(l.expertOut) && l.rowBytes % 16 == 0 &&
         (l.sharedExpertX == nullptr || Aligned16(l.sharedExpertX));
+    if (l.kernelNameOut != nullptr) {
+        *l.kernelNameOut = quant ? "ep_reduce_quant_kernel" : (plain ? "ep_reduce_vec_kernel" : "ep_reduce_generic_kernel");
+    }
     if (quant) {
         if (qvecs <= kWave) {
             LaunchQuant<kWave, 1>(l, a, gridLimit);

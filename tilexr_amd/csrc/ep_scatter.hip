@@ -38,6 +38,7 @@ struct ScatterArgs {
     int tileRows;
     uint64_t epoch;
     const int32_t *totalRowsPtr;
+    int colSlices;               // route kernel: workgroups a row is cut into
 };
 
 __device__ __forceinline__ int RowOfRoute(const ScatterArgs &a, int route)
@@ -100,15 +101,16 @@ __device__ __forceinline__ void ScalarStore(T *p, T v)
 // at zero for the next dispatch).  The caller has made the row complete in memory first, so has every earlier counter
 // of the tile, and the atomics on one counter are totally ordered: when the last one returns, all rows of the tile are
 // in memory.  The words consumers poll are only ever stored to, never hit by atomics.
-__device__ __forceinline__ void PublishRow(const ScatterArgs &a, int row)
+// `parts` callers publish each row (the slices a row is cut into).
+__device__ __forceinline__ void PublishRow(const ScatterArgs &a, int row, int parts)
 {
     const int tile = row / a.tileRows;
     int rowsInTile = 1;
-    if (a.tileRows > 1) {
+    if (a.tileRows > 1 || parts > 1) {
         const int left = *a.totalRowsPtr - tile * a.tileRows;
         rowsInTile = left < a.tileRows ? left : a.tileRows;
         const uint32_t before = __hip_atomic_fetch_add(&a.tileCounters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (static_cast<int>(before) + 1 != rowsInTile) {
+        if (static_cast<int>(before) + 1 != rowsInTile * parts) {
             return;
         }
         __hip_atomic_store(&a.tileCounters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -134,27 +136,31 @@ __device__ __forceinline__ void PublishRows(const ScatterArgs &a, const int *pos
         for (int k = lane; k < a.topK; k += G) {
             const int row = pos[k];
             if (row >= 0) {
-                PublishRow(a, row);
+                PublishRow(a, row, 1);
             }
         }
     }
 }
 
-// Plain copy of wide rows, one workgroup per route: the workgroup loads its token's row and writes the one destination
-// row of route (token, k).  The topK workgroups of a token are given block indices that the dispatcher places on the
-// same XCD (block b runs on XCD b % 8), so the row comes from HBM once and from that XCD's L2 the other topK - 1
-// times.  One row per workgroup keeps every wave at V stores in flight, which this memory system rewards: measured
-// 89 us against 93 us for "one workgroup writes all topK rows" on 4096 x 7168 x top-8, and 132 us when the
-// workgroups of a token are spread over the XCDs.
-template <int V, bool WT>
-__global__ __launch_bounds__(kThreads) void ep_scatter_route_kernel(ScatterArgs a)
+// Plain copy of wide rows, one workgroup per (route, slice of 512 vectors): the workgroup loads its part of the token's
+// row and writes it to the destination row of route (token, k).  The workgroups of a token are given block indices that
+// the dispatcher places on the same XCD (block b runs on XCD b % 8), so the row comes from HBM once and from that
+// XCD's L2 the other topK - 1 times.  Two 16-byte loads then two 16-byte stores per lane is what this memory system
+// rewards, whatever the workgroup size: measured on 4096 x 7168 x top-8, 83-85 us with two vectors per lane (128 to
+// 448 lanes per workgroup), 92-95 us with three to fourteen, 105-130 us with one; 93 us for "one workgroup writes all
+// topK rows", and 132 us when the workgroups of a token are spread over the XCDs.
+constexpr int kRouteVecs = 2;
+template <int THREADS, int V, bool WT>
+__global__ __launch_bounds__(THREADS) void ep_scatter_route_kernel(ScatterArgs a)
 {
     constexpr int kXcds = 8;
     __shared__ int s_row;
     const int xcd = blockIdx.x % kXcds;
     const int j = blockIdx.x / kXcds;
-    const int token = (j / a.topK) * kXcds + xcd;
-    const int k = j % a.topK;
+    const int perToken = a.topK * a.colSlices;
+    const int token = (j / perToken) * kXcds + xcd;
+    const int k = (j % perToken) / a.colSlices;
+    const int colBase = ((j % perToken) % a.colSlices) * (V * THREADS);
     if (token >= a.bs) {
         return;
     }
@@ -167,7 +173,7 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_route_kernel(ScatterArgs 
     u32x4 v[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-        const int idx = i * kThreads + lane;
+        const int idx = colBase + i * THREADS + lane;
         v[i] = idx < vecs ? src[idx] : u32x4{0u, 0u, 0u, 0u};
     }
     __syncthreads();
@@ -179,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_route_kernel(ScatterArgs 
     const __amdgpu_buffer_rsrc_t rsrc = RowResource(dst, vecs * 16);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-        const int idx = i * kThreads + lane;
+        const int idx = colBase + i * THREADS + lane;
         if (idx < vecs) {
             RowStore<WT>(v[i], dst, rsrc, idx * 16);
         }
@@ -188,7 +194,7 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_route_kernel(ScatterArgs 
         WaitOwnStores();
         __syncthreads();
         if (lane == 0) {
-            PublishRow(a, row);
+            PublishRow(a, row, a.colSlices);
         }
     }
 }
@@ -459,12 +465,17 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
         case TILEXR_EP_QUANT_NONE:
             // small batches are latency-bound and gain nothing from the extra workgroups
             if (G == kThreads && a.topK > 1 && a.bs >= 1024 &&
-                static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK <= 0x7fffffff) {
-                const dim3 blocks(static_cast<unsigned>(static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK));
+                static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK * a.colSlices <= 0x7fffffff) {
+                const dim3 blocks(static_cast<unsigned>(static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK * a.colSlices));
+                if (l.kernelNameOut != nullptr) {
+                    *l.kernelNameOut = "ep_scatter_route_kernel";
+                }
                 if (WriteThrough(a)) {
-                    hipLaunchKernelGGL((ep_scatter_route_kernel<V, true>), blocks, dim3(kThreads), 0, l.stream, a);
+                    hipLaunchKernelGGL((ep_scatter_route_kernel<kThreads, kRouteVecs, true>), blocks, dim3(kThreads), 0,
+                        l.stream, a);
                 } else {
-                    hipLaunchKernelGGL((ep_scatter_route_kernel<V, false>), blocks, dim3(kThreads), 0, l.stream, a);
+                    hipLaunchKernelGGL((ep_scatter_route_kernel<kThreads, kRouteVecs, false>), blocks, dim3(kThreads), 0,
+                        l.stream, a);
                 }
             } else {
                 LaunchVec<G, V, TILEXR_EP_QUANT_NONE, true, false>(a, l.stream);
@@ -526,9 +537,13 @@ hipError_t LaunchScatter(const ScatterLaunch &l)
     a.tileRows = static_cast<int>(l.tileRows);
     a.epoch = l.epoch;
     a.totalRowsPtr = l.totalRowsPtr;
+    a.colSlices = static_cast<int>((l.h / 8 + kRouteVecs * kThreads - 1) / (kRouteVecs * kThreads));
     const int64_t vecs = l.h / 8;
     const bool vecOk = l.h % 8 == 0 && Aligned16(l.x) && vecs <= 8 * kThreads &&
         (l.quantMode == TILEXR_EP_QUANT_NONE ? Aligned16(l.out) : Aligned8(l.out));
+    if (l.kernelNameOut != nullptr) {
+        *l.kernelNameOut = vecOk ? "ep_scatter_vec_kernel" : "ep_scatter_generic_kernel";
+    }
     if (vecOk) {
         // narrow rows: a wave per token (four tokens per workgroup); wide rows: the workgroup per token
         if (vecs <= 2 * kWave) {

@@ -23,6 +23,7 @@ EXPORTS = (
     "TileXRMoeEpDispatch", "TileXRMoeEpDispatchV2", "TileXRMoeEpDispatchMemory", "TileXRMoeEpDispatchMemoryV2",
     "TileXRMoeEpCombine", "TileXRMoeEpCombineV2", "TileXRMoeEpCombineMemory", "TileXRMoeEpCombineMemoryV2",
     "TileXRMoeEpDispatchMemoryEx", "TileXRMoeEpCombineMemoryEx", "TileXREpVersion", "TileXREpSetKernelTimingEvents",
+    "TileXREpLastKernelName",
     "TileXRCommInitRankLocal", "TileXRCommDestroy", "TileXRGetCommArgsHost", "TileXRGetCommArgsDev",
     "TileXRCommNextMagic",
 )
@@ -72,6 +73,8 @@ def lib():
         _lib = C.CDLL(LIB_PATH)
         i64, vp, i32 = C.c_int64, C.c_void_p, C.c_int
         _lib.TileXREpVersion.restype = C.c_char_p
+        _lib.TileXREpLastKernelName.restype = C.c_char_p
+        _lib.TileXREpLastKernelName.argtypes = [C.c_void_p, C.c_int]
         _lib.TileXRCommInitRankLocal.argtypes = [i32, i32, C.POINTER(vp)]
         _lib.TileXRCommDestroy.argtypes = [vp]
         _lib.TileXRCommNextMagic.argtypes = [vp, C.POINTER(i64)]
@@ -94,7 +97,7 @@ def lib():
         _lib.TileXREpSetKernelTimingEvents.argtypes = [vp, i32, vp, vp]
         for name in EXPORTS:
             fn = getattr(_lib, name)
-            if name != "TileXREpVersion":
+            if name not in ("TileXREpVersion", "TileXREpLastKernelName"):
                 fn.restype = C.c_int
     return _lib
 
@@ -272,6 +275,11 @@ K_COUNT, K_PLACE, K_SCATTER, K_INVERT, K_REDUCE = range(5)
 def set_kernel_timing_events(comm, kernel, start=None, stop=None):
     return lib().TileXREpSetKernelTimingEvents(_h(comm), kernel, start.handle if start else None,
                                                stop.handle if stop else None)
+
+
+def last_kernel_name(comm, kernel):
+    name = lib().TileXREpLastKernelName(_h(comm), kernel)
+    return name.decode() if name else None
 
 
 # ---- HIP events for the dispatch/combine overlap (hipEvent_t handles usable with the C ABI) ---------------
