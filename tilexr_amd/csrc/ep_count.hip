@@ -2,7 +2,7 @@
 //
 // They turn the [bs, topK] expert-id table into destinations without moving a single payload byte:
 //   count   stable rank of every live route within its key + histograms; the last workgroup scans them
-//   place   destination row of every route, assist tuples, inverse map, tile-flag reset
+//   place   destination row of every route, assist tuples, inverse map
 //   invert  (combine side) row -> (token, k) inverse rebuilt from assist tuples
 // All integer work; the reference behaviour each kernel restates is cited at the kernel.
 #include <hip/hip_runtime.h>
@@ -58,6 +58,7 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     constexpr int kChunkRoutes = kThreads * BPW;
     __shared__ int s_cnt[kWavesPerBlock * kMaxKeys];
     __shared__ int s_exp[kMaxKeys];
+    __shared__ int s_tot[kMaxKeys];     // single-chunk launches: the chunk's (= the launch's) routes per key
     __shared__ int s_part[kThreads];
     __shared__ int s_misc[4];
 
@@ -162,11 +163,21 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
             s_cnt[w * a.numKeys + key] = run;
             run += v;
         }
-        a.s.chunkHist[static_cast<int64_t>(chunk) * a.numKeys + key] = run;
+        if (a.numChunks == 1) {
+            // the only chunk: its totals stay in LDS, its base within every key is zero, nobody has to be waited for
+            s_tot[key] = run;
+            a.s.chunkHist[key] = 0;
+            continue;
+        }
+        // written through (agent scope): complete for the scanning workgroup, on whatever XCD it runs, once this
+        // wave's stores have drained, with no write-back of the L2
+        __hip_atomic_store(&a.s.chunkHist[static_cast<int64_t>(chunk) * a.numKeys + key], run, __ATOMIC_RELAXED,
+            __HIP_MEMORY_SCOPE_AGENT);
     }
-    if (expHist) {
+    if (expHist && a.numChunks > 1) {
         for (int e = tid; e < a.numExperts; e += kThreads) {
-            a.s.chunkExpHist[static_cast<int64_t>(chunk) * a.numExperts + e] = s_exp[e];
+            __hip_atomic_store(&a.s.chunkExpHist[static_cast<int64_t>(chunk) * a.numExperts + e], s_exp[e],
+                __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     __syncthreads();
@@ -189,12 +200,16 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     }
 
     // The last workgroup to arrive performs the scans.  Only the chunk histograms (stored in phase B, long since
-    // on their way) have to be visible to it, so the ticket is taken before the rank stores are issued.
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned prev = atomicAdd(a.s.ticket, 1u);
-        s_misc[1] = prev == static_cast<unsigned>(a.numChunks - 1) ? 1 : 0;
+    // on their way) have to be complete for it, so the ticket is taken before the rank stores are issued.
+    if (a.numChunks > 1) {
+        WaitOwnStores();
+        __syncthreads();
+        if (tid == 0) {
+            const unsigned prev = atomicAdd(a.s.ticket, 1u);
+            s_misc[1] = prev == static_cast<unsigned>(a.numChunks - 1) ? 1 : 0;
+        }
+    } else if (tid == 0) {
+        s_misc[1] = 1;
     }
 #pragma unroll
     for (int b = 0; b < BPW; ++b) {
@@ -207,20 +222,20 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     if (s_misc[1] == 0) {
         return;
     }
-    __threadfence();
 
     // per key: exclusive sum over chunks (becomes the chunk's base rank within the key), total, kept
     int *kept = s_cnt;                 // reuse: [numKeys]
     for (int key = tid; key < a.numKeys; key += kThreads) {
-        int run = 0;
+        int run = a.numChunks == 1 ? s_tot[key] : 0;
         // the loads of a batch are independent: one round trip per 32 chunks
         constexpr int kBatch = 32;
-        for (int c0 = 0; c0 < a.numChunks; c0 += kBatch) {
+        for (int c0 = 0; c0 < a.numChunks && a.numChunks > 1; c0 += kBatch) {
             int v[kBatch];
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 const int c = c0 + u;
-                v[u] = c < a.numChunks ? a.s.chunkHist[static_cast<int64_t>(c) * a.numKeys + key] : 0;
+                v[u] = c < a.numChunks ? __hip_atomic_load(&a.s.chunkHist[static_cast<int64_t>(c) * a.numKeys + key],
+                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
             }
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
@@ -261,9 +276,10 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     int *etot = s_cnt + 2 * kMaxKeys;  // [numExperts]
     if (expHist) {
         for (int e = tid; e < a.numExperts; e += kThreads) {
-            int run = 0;
-            for (int c = 0; c < a.numChunks; ++c) {
-                run += a.s.chunkExpHist[static_cast<int64_t>(c) * a.numExperts + e];
+            int run = a.numChunks == 1 ? s_exp[e] : 0;
+            for (int c = 0; c < a.numChunks && a.numChunks > 1; ++c) {
+                run += __hip_atomic_load(&a.s.chunkExpHist[static_cast<int64_t>(c) * a.numExperts + e], __ATOMIC_RELAXED,
+                    __HIP_MEMORY_SCOPE_AGENT);
             }
             etot[e] = run;
         }
@@ -298,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
             }
         }
     }
-    if (tid == 0) {
+    if (tid == 0 && a.numChunks > 1) {
         *a.s.ticket = 0u;
     }
 }
@@ -393,6 +409,7 @@ CountScratchLayout PlanCountScratch(int64_t routes, int64_t numKeys, int64_t num
     while (p.chunkShift < kMaxChunkShift && ((routes + (1ll << p.chunkShift) - 1) >> p.chunkShift) > kTargetChunks) {
         ++p.chunkShift;
     }
+
     p.chunks = (routes + (1ll << p.chunkShift) - 1) >> p.chunkShift;
     int64_t off = 256;   // word 0 is the ticket
     p.localRankOff = off;
