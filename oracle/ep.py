@@ -27,6 +27,8 @@ class _Case(C.Structure):
         ("token_nums_type", C.c_int32),
         ("mask_type", C.c_int32),
         ("capacity", C.c_int64),
+        ("shared_expert_num", C.c_int64),
+        ("shared_expert_rank_num", C.c_int64),
     ]
 
 
@@ -43,18 +45,24 @@ class Case:
     token_nums_type: int = 1
     mask_type: int = MASK_NONE
     capacity: int = 0
+    shared_expert_num: int = 0
+    shared_expert_rank_num: int = 0
 
     def c(self):
         return _Case(self.rank_size, self.bs, self.h, self.top_k, self.moe_expert_num, self.dtype,
-                     self.quant_mode, self.out_dtype, self.token_nums_type, self.mask_type, self.capacity)
+                     self.quant_mode, self.out_dtype, self.token_nums_type, self.mask_type, self.capacity,
+                     self.shared_expert_num, self.shared_expert_rank_num)
 
     @property
     def local_experts(self):
-        return self.moe_expert_num // self.rank_size
+        return self.moe_expert_num // (self.rank_size - self.shared_expert_rank_num)
+
+    def out_local_experts(self, rank):
+        return 1 if rank < self.shared_expert_rank_num else self.local_experts
 
     @property
     def max_rows(self):
-        return self.rank_size * self.bs * self.top_k
+        return self.rank_size * self.bs * (self.top_k + self.shared_expert_num)
 
     @property
     def out_row_bytes(self):
@@ -223,8 +231,8 @@ def mem_dispatch(case, dst_rank, x, ids, mask=None):
     else:
         scales = np.zeros((rows, max(spr, 1)), np.float32)
     assist = np.zeros((rows, 4), np.int32)
-    send = np.zeros(case.local_experts * case.rank_size, np.int32)
-    nums = np.zeros(case.local_experts, np.int64)
+    send = np.zeros(case.out_local_experts(dst_rank) * case.rank_size, np.int32)
+    nums = np.zeros(case.out_local_experts(dst_rank), np.int64)
     cc = case.c()
     n = lib().orc_mem_dispatch_rank(C.byref(cc), dst_rank, _p(x), _p(ids), _p(mask), _p(expand), _p(scales),
                                     _p(assist), _p(send), _p(nums))

@@ -323,9 +323,24 @@ void orc_quant_row_fp8_block128(const uint16_t *src, int64_t h, int32_t dtype, u
  * Dispatch
  * ---------------------------------------------------------------------------------------------- */
 
+/* src/ep/host/ep_layout.cpp:156,171; tests/ep/demo/tilexr_ep_dispatch_demo.cpp:622-630 */
 static int64_t local_expert_num(const orc_case *c)
 {
-    return c->moe_expert_num / c->rank_size;
+    return c->moe_expert_num / (c->rank_size - c->shared_expert_rank_num);
+}
+
+/* tests/ep/demo/tilexr_ep_dispatch_demo.cpp:632-635: a shared rank presents one local expert */
+static int64_t out_local_expert_num(const orc_case *c, int32_t rank)
+{
+    return rank < c->shared_expert_rank_num ? 1 : local_expert_num(c);
+}
+
+/* Destination rank of a shared route (demo :654-657; src/ep/kernels/tilexr_ep_dispatch_memory_kernel.h:635-643;
+ * MVP route, where SR == S: tilexr_ep_dispatch_helpers.h:85-87). */
+static int64_t shared_dst_rank(const orc_case *c, int32_t src, int64_t s)
+{
+    const int64_t per = c->shared_expert_rank_num / c->shared_expert_num;
+    return src % per + s * per;
 }
 
 static int64_t out_row_bytes(const orc_case *c)
@@ -359,13 +374,30 @@ int64_t orc_mvp_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_
             if (ms && ms[t] == 0) {
                 continue;
             }
-            for (int64_t k = 0; k < c->top_k; ++k) {
-                const int32_t e = is[t * c->top_k + k];
-                if (e < 0 || (int64_t)e >= c->moe_expert_num) {
-                    continue;
-                }
-                if ((int64_t)e / local_e != dst_rank) {
-                    continue;
+            /* one pass over the token's S shared routes, then its top_k routed ones
+             * (src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:536-568) */
+            for (int64_t r = 0; r < c->shared_expert_num + c->top_k; ++r) {
+                const int shared = r < c->shared_expert_num;
+                const int64_t k = shared ? c->top_k + r : r - c->shared_expert_num;
+                int32_t e;
+                int64_t local;
+                if (shared) {
+                    if (shared_dst_rank(c, src, r) != dst_rank) {
+                        continue;
+                    }
+                    e = (int32_t)r;
+                    /* tilexr_ep_dispatch_helpers.h:99-101: a shared row counts at index expertId */
+                    local = r;
+                } else {
+                    const int32_t id = is[t * c->top_k + k];
+                    if (id < 0 || (int64_t)id >= c->moe_expert_num) {
+                        continue;
+                    }
+                    if (c->shared_expert_rank_num + (int64_t)id / local_e != dst_rank) {
+                        continue;
+                    }
+                    e = (int32_t)(c->shared_expert_num + id);
+                    local = (int64_t)id % local_e;
                 }
                 uint8_t *dst = expand_x + out * row_bytes;
                 const uint16_t *row = xs + t * c->h;
@@ -380,7 +412,9 @@ int64_t orc_mvp_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_
                 assist[out * 4 + 1] = (int32_t)t;
                 assist[out * 4 + 2] = (int32_t)k;
                 assist[out * 4 + 3] = e;
-                ++expert_token_nums[(int64_t)e % local_e];
+                if (local < local_e) {          /* tilexr_ep_combine_helpers.h:124-128 */
+                    ++expert_token_nums[local];
+                }
                 ++count;
                 ++out;
             }
@@ -433,28 +467,49 @@ int64_t orc_mem_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_
     const int64_t mask_stride = c->mask_type == ORC_MASK_EXPERT ? routes : c->bs;
     const int64_t mx_scales = orc_mxfp8_scale_count(c->h);
     const int64_t b128 = (c->h + 127) / 128;
+    const int64_t out_local = out_local_expert_num(c, dst_rank);
+    const int is_shared_rank = dst_rank < c->shared_expert_rank_num;
     int64_t out = 0;
-    for (int64_t le = 0; le < local_e; ++le) {
-        const int64_t expert = (int64_t)dst_rank * local_e + le;
+    for (int64_t le = 0; le < out_local; ++le) {
+        /* id (as the caller numbers routed experts) whose rows this segment collects; on a shared rank the
+         * segment collects the shared routes aimed at it instead (tilexr_ep_dispatch_memory_kernel.h:622-663) */
+        const int64_t expert = ((int64_t)dst_rank - c->shared_expert_rank_num) * local_e + le;
         for (int32_t src = 0; src < c->rank_size; ++src) {
             const uint16_t *xs = x + (int64_t)src * c->bs * c->h;
             const int32_t *is = ids + (int64_t)src * routes;
             const uint8_t *ms = (mask && c->mask_type != ORC_MASK_NONE) ? mask + (int64_t)src * mask_stride : NULL;
             const int64_t limit = mem_route_limit(c, ms);
             int64_t kept = 0;
-            for (int64_t i = 0; i < limit; ++i) {
-                if (c->mask_type == ORC_MASK_EXPERT && ms && ms[i] == 0) {
-                    continue;
-                }
-                if ((int64_t)is[i] != expert) {
-                    continue;
-                }
-                if (c->capacity > 0 && kept >= c->capacity) {
-                    continue;
+            /* shared rank: walk (shared expert, token) pairs; otherwise the flat routes */
+            const int64_t walk = is_shared_rank ? c->shared_expert_num * (limit / c->top_k) : limit;
+            for (int64_t i = 0; i < walk; ++i) {
+                int64_t t;
+                int64_t k;
+                int32_t tuple_expert;
+                if (is_shared_rank) {
+                    const int64_t tokens = limit / c->top_k;
+                    const int64_t s = i / tokens;
+                    if (shared_dst_rank(c, src, s) != dst_rank) {
+                        continue;
+                    }
+                    t = i % tokens;
+                    k = c->top_k + s;
+                    tuple_expert = (int32_t)s;      /* :1257 topKId - K on a shared rank */
+                } else {
+                    if (c->mask_type == ORC_MASK_EXPERT && ms && ms[i] == 0) {
+                        continue;
+                    }
+                    if ((int64_t)is[i] != expert) {
+                        continue;
+                    }
+                    if (c->capacity > 0 && kept >= c->capacity) {
+                        continue;
+                    }
+                    t = i / c->top_k;
+                    k = i % c->top_k;
+                    tuple_expert = (int32_t)(c->shared_expert_num + expert);    /* :1241-1244 */
                 }
                 ++kept;
-                const int64_t t = i / c->top_k;
-                const int64_t k = i % c->top_k;
                 uint8_t *dst = expand_x + out * row_bytes;
                 const uint16_t *row = xs + t * c->h;
                 switch (c->quant_mode) {
@@ -474,14 +529,14 @@ int64_t orc_mem_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_
                 assist[out * 4 + 0] = src;
                 assist[out * 4 + 1] = (int32_t)t;
                 assist[out * 4 + 2] = (int32_t)k;
-                assist[out * 4 + 3] = (int32_t)expert;
+                assist[out * 4 + 3] = tuple_expert;
                 ++out;
             }
             send_counts[le * c->rank_size + src] = (int32_t)out;
         }
     }
     int64_t last = 0;
-    for (int64_t le = 0; le < local_e; ++le) {
+    for (int64_t le = 0; le < out_local; ++le) {
         const int64_t cum = send_counts[le * c->rank_size + c->rank_size - 1];
         expert_token_nums[le] = c->token_nums_type == 0 ? cum : cum - last;
         last = cum;
@@ -560,7 +615,8 @@ void orc_mem_combine_rank(const orc_case *c, int32_t rank, int64_t max_rows, con
 {
     const int64_t local_e = local_expert_num(c);
     const int64_t n_counts = local_e * c->rank_size;
-    const int64_t slots = c->bs * c->top_k;
+    const int64_t per_token = c->top_k + c->shared_expert_num;
+    const int64_t slots = c->bs * per_token;
     const int64_t rb = in_row_bytes(c, in_quant);
     const int64_t b128 = (c->h + 127) / 128;
     const int64_t in_scales_per_row = in_quant == ORC_QUANT_FP8_BLOCK128 ? b128 : 1;
@@ -575,17 +631,17 @@ void orc_mem_combine_rank(const orc_case *c, int32_t rank, int64_t max_rows, con
         slot_row[i] = -1;
     }
     for (int32_t er = 0; er < c->rank_size; ++er) {
-        int64_t rows = send_counts[(int64_t)er * n_counts + n_counts - 1];
+        int64_t rows = send_counts[(int64_t)er * n_counts + out_local_expert_num(c, er) * c->rank_size - 1];
         if (rows < 0) {
             rows = 0;
         }
         for (int64_t row = 0; row < rows; ++row) {
             const int32_t *tuple = assist + ((int64_t)er * max_rows + row) * 4;
             if (tuple[0] != rank || tuple[1] < 0 || (int64_t)tuple[1] >= c->bs || tuple[2] < 0 ||
-                (int64_t)tuple[2] >= c->top_k) {
+                (int64_t)tuple[2] >= per_token) {
                 continue;
             }
-            slot_row[(int64_t)tuple[1] * c->top_k + tuple[2]] = (int64_t)er * max_rows + row;
+            slot_row[(int64_t)tuple[1] * per_token + tuple[2]] = (int64_t)er * max_rows + row;
         }
     }
     for (int64_t t = 0; t < c->bs; ++t) {
@@ -597,12 +653,14 @@ void orc_mem_combine_rank(const orc_case *c, int32_t rank, int64_t max_rows, con
         for (int64_t i = 0; i < c->h; ++i) {
             sum[i] = 0.0f;
         }
-        for (int64_t k = 0; k < c->top_k; ++k) {
-            const int64_t row = slot_row[t * c->top_k + k];
+        /* the top_k routed slots with their gate weights, then the shared slots with weight 1
+         * (tilexr_ep_combine_memory_kernel.h:650-657) */
+        for (int64_t k = 0; k < per_token; ++k) {
+            const int64_t row = slot_row[t * per_token + k];
             if (row < 0) {
                 continue;
             }
-            const float w = expert_scales ? expert_scales[t * c->top_k + k] : 1.0f;
+            const float w = (expert_scales && k < c->top_k) ? expert_scales[t * c->top_k + k] : 1.0f;
             const uint8_t *raw = (const uint8_t *)expert_out + row * rb;
             const uint16_t *elems = (const uint16_t *)raw;
             if (in_quant != 0) {

@@ -23,6 +23,8 @@
  *   capacity drop (ext)                           : brute force            (reference: parity unpinned)
  *   MVP combine (per-add rounding)                : numpy float16 sequential sum
  *   memory combine (fp32 acc, RINT)               : numpy float32 sequential sum + torch cast
+ *   shared experts (both routes)                  : the reference demo's golden route model restated as a
+ *                                                   brute-force walk in the tests, closed-form row counts
  */
 #ifndef TILEXR_EP_ORACLE_H
 #define TILEXR_EP_ORACLE_H
@@ -64,6 +66,8 @@ typedef struct {
     int32_t token_nums_type;  /* 0 = inclusive prefix sum, 1 = counts */
     int32_t mask_type;
     int64_t capacity;         /* ext: rows kept per expert per destination (0 = unlimited) */
+    int64_t shared_expert_num;      /* S: every active token also goes to each of S shared experts */
+    int64_t shared_expert_rank_num; /* ranks [0, SR) host the shared experts (SR % S == 0); E % (R - SR) == 0 */
 } orc_case;
 
 /* ---- scalar numerics ---- */
@@ -86,7 +90,11 @@ void orc_quant_row_fp8_block128(const uint16_t *src, int64_t h, int32_t dtype, u
 
 /* ---- dispatch (outputs of ONE destination rank, inputs of ALL source ranks) ----
  * x     [R][bs*h] u16, ids [R][bs*top_k], mask [R][bs] or [R][bs*top_k] (may be NULL)
- * Returns the number of rows written. */
+ * Returns the number of rows written.
+ * With shared experts a token emits its S shared routes (topKId = top_k + s, expertId = s, destination rank
+ * src % (SR/S) + s * (SR/S)) before its top_k routed ones (expertId = S + id, destination SR + id / localE),
+ * localE = E / (R - SR).  expert_token_nums has localE entries (MVP route) or, on the memory route, 1 entry on
+ * a shared rank and localE on the others; send_counts likewise 1*R or localE*R entries. */
 int64_t orc_mvp_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_t *x, const int32_t *ids,
     const uint8_t *mask, const float *static_scale, uint8_t *expand_x, float *dyn_scales, int32_t *assist,
     int32_t *recv_counts, int64_t *expert_token_nums);
@@ -96,7 +104,8 @@ int64_t orc_mem_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_
     int64_t *expert_token_nums);
 
 /* ---- combine (output of ONE source rank, inputs of ALL expert ranks) ----
- * expert_out [R][max_rows*row_bytes], assist [R][max_rows*4], counts [R][R] (MVP) or [R][localE*R] (memory). */
+ * expert_out [R][max_rows*row_bytes], assist [R][max_rows*4], counts [R][R] (MVP) or [R][localE*R] (memory;
+ * a shared rank uses the first R entries of its block). */
 void orc_mvp_combine_rank(const orc_case *c, int32_t rank, int64_t max_rows, const uint16_t *expert_out,
     const int32_t *assist, const int32_t *recv_counts, uint16_t *y);
 

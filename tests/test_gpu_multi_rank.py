@@ -312,3 +312,159 @@ def test_exchange_protocol_errors():
             n = want["rows"]
             assert np.array_equal(outs[r]["expand_x"].cpu().numpy()[:n], want["expand_x"][:n])
             assert np.array_equal(counts[r].cpu().numpy(), want["send_counts"])
+
+
+# ---------------------------------------------------------------------------------------------
+# Shared experts: ranks [0, SR) host S shared experts that every active token is also sent to
+# ---------------------------------------------------------------------------------------------
+def alloc_shared_outputs(R, bs, h, K, S, local_experts, quant, memory, dst, SR):
+    rows = R * bs * (K + S)
+    row_bytes = h * 2 if quant == ep.Q_NONE else h
+    out_local = (1 if dst < SR else local_experts) if memory else local_experts
+    out = dict(
+        expand_x=torch.full((rows, row_bytes), 0x5a, dtype=torch.uint8, device=DEV),
+        assist=torch.full((rows, 4), -77, dtype=torch.int32, device=DEV),
+        token_nums=torch.full((out_local,), -5, dtype=torch.int64, device=DEV),
+        counts=torch.full((out_local * R if memory else R,), -1, dtype=torch.int32, device=DEV),
+        tp_counts=torch.full((R,), -1, dtype=torch.int32, device=DEV),
+        scales=None,
+    )
+    if quant == ep.Q_TOKEN_INT8:
+        out["scales"] = torch.full((rows, 1), -3.0, dtype=torch.float32, device=DEV)
+    elif quant == ep.Q_MXFP8:
+        out["scales"] = torch.full((rows, ((h + 31) // 32 + 1) // 2 * 2), 0xee, dtype=torch.uint8, device=DEV)
+    return out
+
+
+SHARED_SHAPES = [  # R, bs, h, K, E, S, SR
+    (4, 6, 16, 2, 6, 1, 1), (4, 40, 256, 3, 8, 2, 2), (8, 25, 64, 2, 12, 2, 4), (3, 17, 40, 2, 4, 1, 1),
+    (6, 300, 512, 4, 16, 1, 2), (4, 128, 1024, 8, 32, 2, 2)]
+
+
+@pytest.mark.parametrize("shape", [s for s in SHARED_SHAPES if s[5] == s[6]])
+def test_mvp_dispatch_with_shared_experts(shape):
+    R, bs, h, K, E, S, SR = shape
+    rng = np.random.default_rng(sum(shape))
+    ids = rand_ids(rng, R, bs, K, E, invalid=0.1)
+    xt, xb = rand_x(rng, R, bs, h, ep.DT_FP16, scale=3.0)
+    mask = (rng.random((R, bs)) < 0.7).astype(np.uint8)
+    with World(R) as w:
+        for quant, use_mask, nums_type in ((ep.Q_NONE, False, 1), (ep.Q_NONE, True, 0), (ep.Q_TOKEN_INT8, True, 1)):
+            case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16, quant_mode=quant, token_nums_type=nums_type,
+                          shared_expert_num=S, shared_expert_rank_num=SR)
+            outs = [alloc_shared_outputs(R, bs, h, K, S, case.local_experts, quant, False, r, SR) for r in range(R)]
+            dev_ids = [to_dev(ids[r]) for r in range(R)]
+            dev_mask = [to_dev(mask[r]) if use_mask else None for r in range(R)]
+            for r in rng.permutation(R):
+                o = outs[r]
+                st = ep.dispatch_v2(xt[r], dev_ids[r], w.comms[r], bs, h, K, E, o["expand_x"], o["assist"],
+                                    o["token_nums"], o["counts"], ep.DT_FP16 if quant == ep.Q_NONE else ep.DT_INT8,
+                                    w.streams[r], active_mask=dev_mask[r], shared_expert_num=S,
+                                    shared_expert_rank_num=SR, quant_mode=quant, token_nums_type=nums_type,
+                                    dynamic_scales=o["scales"], tp_recv_counts=o["tp_counts"])
+                assert st == 0, f"rank {r}: status {st}"
+            w.sync()
+            for r in range(R):
+                want = O.mvp_dispatch(case, r, xb, ids, mask if use_mask else None)
+                check_rank(outs[r], want, "recv_counts")
+                if quant == ep.Q_TOKEN_INT8:
+                    n = want["rows"]
+                    assert np.array_equal(outs[r]["scales"].cpu().numpy()[:n, 0], want["dyn_scales"][:n])
+            if quant != ep.Q_NONE:
+                continue
+            # the MVP combine drops the shared-expert rows (their topKId is not below topK)
+            ys = [torch.full((bs, h), 7.0, dtype=torch.float16, device=DEV) for _ in range(R)]
+            eo = [(outs[r]["expand_x"].view(torch.float16) * (1.0 + 0.25 * r)).contiguous() for r in range(R)]
+            if E % R != 0:
+                # the MVP combine call carries no shared-expert arguments and checks the plain placement rule
+                # (reference: src/ep/host/ep_dispatch_host.cpp:155-163 -> ep_layout.cpp:152-226 with 0 shared ranks)
+                assert ep.combine_v2(eo[0], outs[0]["assist"], outs[0]["counts"], w.comms[0], bs, h, K, E, ys[0],
+                                     ep.DT_FP16, w.streams[0]) == ep.ERR_PARA_CHECK_FAIL
+                continue
+            for r in range(R):
+                assert ep.combine_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
+                                     ep.DT_FP16, w.streams[r]) == 0
+            w.sync()
+            eo_np = np.stack([bits16(t) for t in eo])
+            assist_np = np.stack([o["assist"].cpu().numpy() for o in outs])
+            counts_np = np.stack([o["counts"].cpu().numpy() for o in outs])
+            plain = O.Case(R, bs, h, K, E, dtype=O.DT_FP16, shared_expert_num=S, shared_expert_rank_num=SR)
+            for r in range(R):
+                assert np.array_equal(bits16(ys[r]), O.mvp_combine(plain, r, eo_np, assist_np, counts_np)), f"rank {r}"
+
+
+@pytest.mark.parametrize("shape", SHARED_SHAPES)
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+def test_memory_dispatch_and_combine_with_shared_experts(shape, dtype):
+    R, bs, h, K, E, S, SR = shape
+    rng = np.random.default_rng(sum(shape) + dtype)
+    ids = rand_ids(rng, R, bs, K, E, invalid=0.1)
+    xt, xb = rand_x(rng, R, bs, h, dtype)
+    tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+    with World(R) as w:
+        for mask_type, nums_type, quant in ((ep.MASK_NONE, 1, ep.Q_NONE), (ep.MASK_TOKEN, 0, ep.Q_NONE),
+                                            (ep.MASK_NONE, 1, ep.Q_MXFP8)):
+            if quant == ep.Q_MXFP8 and h % 32 != 0:
+                continue
+            mask = (rng.random((R, bs)) < 0.7).astype(np.uint8) if mask_type == ep.MASK_TOKEN else None
+            case = O.Case(R, bs, h, K, E, dtype=dtype, mask_type=mask_type, token_nums_type=nums_type, quant_mode=quant,
+                          out_dtype=O.DT_FP8E4M3, shared_expert_num=S, shared_expert_rank_num=SR)
+            outs = [alloc_shared_outputs(R, bs, h, K, S, case.local_experts, quant, True, r, SR) for r in range(R)]
+            dev_ids = [to_dev(ids[r]) for r in range(R)]
+            dev_mask = [None if mask is None else to_dev(mask[r]) for r in range(R)]
+            order = list(rng.permutation(R))
+            for r in order:
+                o = outs[r]
+                st = ep.dispatch_memory_v2(xt[r], dev_ids[r], w.comms[r], bs, h, K, E, o["expand_x"], o["assist"],
+                                           o["token_nums"], o["counts"], dtype, w.streams[r], active_mask=dev_mask[r],
+                                           active_mask_type=mask_type, shared_expert_num=S, shared_expert_rank_num=SR,
+                                           quant_mode=quant, token_nums_type=nums_type, dynamic_scales=o["scales"],
+                                           expand_x_dtype=ep.DT_FP8E4M3 if quant == ep.Q_MXFP8 else ep.DT_RESERVED)
+                assert st == 0, f"rank {r}: status {st}"
+            w.sync()
+            wants = [O.mem_dispatch(case, r, xb, ids, mask) for r in range(R)]
+            for r in range(R):
+                check_rank(outs[r], wants[r], "send_counts")
+                if quant == ep.Q_MXFP8:
+                    n = wants[r]["rows"]
+                    assert np.array_equal(outs[r]["scales"].cpu().numpy()[:n], wants[r]["dyn_scales"][:n])
+            if quant != ep.Q_NONE:
+                continue
+            weights = rng.random((R, bs, K)).astype(np.float32)
+            shared_t, shared_b = rand_x(rng, R, bs, h, dtype)
+            ys = [torch.full((bs, h), 7.0, dtype=tdt, device=DEV) for _ in range(R)]
+            eo = [(outs[r]["expand_x"].view(tdt) * (1.0 + 0.25 * r)).contiguous() for r in range(R)]
+            dev_w = [to_dev(weights[r]) for r in range(R)]
+            for r in reversed(order):
+                st = ep.combine_memory_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
+                                          dtype, w.streams[r], expert_scales=dev_w[r], shared_expert_x=shared_t[r],
+                                          shared_expert_num=S, shared_expert_rank_num=SR)
+                assert st == 0
+            w.sync()
+            mr = case.max_rows
+            eo_np = np.stack([bits16(t) for t in eo])
+            assist_np = np.stack([o["assist"].cpu().numpy() for o in outs])
+            counts_np = np.zeros((R, case.local_experts * R), np.int32)
+            for r in range(R):
+                c = outs[r]["counts"].cpu().numpy()
+                counts_np[r, :c.size] = c
+            assert eo_np.shape[1] == mr
+            plain = O.Case(R, bs, h, K, E, dtype=dtype, shared_expert_num=S, shared_expert_rank_num=SR)
+            for r in range(R):
+                want_y = O.mem_combine(plain, r, eo_np, assist_np, counts_np, expert_scales=weights[r],
+                                       shared_expert_x=shared_b[r])
+                assert np.array_equal(bits16(ys[r]), want_y), f"rank {r}"
+
+
+def test_expert_mask_with_shared_experts_is_reported_as_unsupported():
+    R, bs, h, K, E, S, SR = 4, 8, 16, 2, 6, 1, 1
+    rng = np.random.default_rng(5)
+    ids = rand_ids(rng, R, bs, K, E)
+    xt, _ = rand_x(rng, R, bs, h, ep.DT_BF16)
+    mask = np.ones((bs, K), np.uint8)
+    with World(R) as w:
+        o = alloc_shared_outputs(R, bs, h, K, S, E // (R - SR), ep.Q_NONE, True, 0, SR)
+        st = ep.dispatch_memory_v2(xt[0], to_dev(ids[0]), w.comms[0], bs, h, K, E, o["expand_x"], o["assist"],
+                                   o["token_nums"], o["counts"], ep.DT_BF16, w.streams[0], active_mask=to_dev(mask),
+                                   active_mask_type=ep.MASK_EXPERT, shared_expert_num=S, shared_expert_rank_num=SR)
+        assert st == ep.ERR_NOT_SUPPORT

@@ -463,3 +463,134 @@ def test_oracle_matches_committed_checker_fixtures(orc):
                 digest = np.frombuffer(hashlib.sha256(np.ascontiguousarray(want).tobytes()).digest(), np.uint8)
                 assert np.array_equal(digest, fx[f"case{i}_combine_sha256"][r])
     assert int(fx["case3_dispatch_events"][0]) == 4148 and int(fx["case3_combine_events"][0]) == 6164
+
+
+# ---------------------------------------------------------------------------------------------
+# Shared experts: the reference demo's golden route model, restated as a brute-force walk
+# (tests/ep/demo/tilexr_ep_dispatch_demo.cpp:622-792: LocalExpertNum, DstRankForExpert, LocalExpertForExpert,
+# BuildExpectedRoutes, BuildExpectedMemoryRoutes, BuildExpectedRecvCounts)
+# ---------------------------------------------------------------------------------------------
+def demo_routes(case, dst, ids, token_live):
+    """Source-major routes of destination rank `dst`: [(src, token, topKId, expertId)]."""
+    R, S, SR, K = case.rank_size, case.shared_expert_num, case.shared_expert_rank_num, case.top_k
+    le = case.moe_expert_num // (R - SR)
+    per = SR // S if S else 1
+    out = []
+    for src in range(R):
+        for t in range(case.bs):
+            if not token_live[src][t]:
+                continue
+            for s in range(S):
+                if src % per + s * per == dst:
+                    out.append((src, t, K + s, s))
+            for k in range(K):
+                e = int(ids[src, t, k])
+                if 0 <= e < case.moe_expert_num and SR + e // le == dst:
+                    out.append((src, t, k, S + e))
+    return out
+
+
+def demo_local_expert(case, expert_id):
+    le = case.moe_expert_num // (case.rank_size - case.shared_expert_rank_num)
+    return 0 if expert_id < case.shared_expert_num else (expert_id - case.shared_expert_num) % le
+
+
+SHARED_SHAPES = [  # R, bs, h, K, E, S, SR
+    (4, 6, 8, 2, 6, 1, 1), (4, 9, 8, 3, 8, 2, 2), (8, 5, 8, 2, 12, 2, 4), (3, 7, 8, 2, 4, 1, 1), (6, 4, 8, 4, 16, 1, 2)]
+
+
+@pytest.mark.parametrize("shape", SHARED_SHAPES)
+@pytest.mark.parametrize("masked", [False, True])
+def test_shared_experts_memory_route_matches_demo_golden(orc, shape, masked):
+    R, bs, h, K, E, S, SR = shape
+    rng = np.random.default_rng(sum(shape) + masked)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16, shared_expert_num=S, shared_expert_rank_num=SR,
+                  mask_type=O.MASK_TOKEN if masked else O.MASK_NONE, token_nums_type=1)
+    ids = rand_ids(rng, R, bs, K, E, invalid_frac=0.1)
+    x = rand_x(rng, R, bs, h)
+    mask = (rng.random((R, bs)) < 0.7).astype(np.uint8) if masked else None
+    # the memory route dispatches the first sum(mask) tokens of a source rank (prefix rule)
+    live = [[t < int(mask[s].sum()) for t in range(bs)] for s in range(R)] if masked else [[True] * bs] * R
+    total = 0
+    for dst in range(R):
+        got = orc.mem_dispatch(case, dst, x, ids, mask)
+        source_major = demo_routes(case, dst, ids, live)
+        out_local = 1 if dst < SR else case.local_experts
+        want = [r for loc in range(out_local) for src in range(R) for r in source_major
+                if r[0] == src and demo_local_expert(case, r[3]) == loc]
+        assert got["rows"] == len(want)
+        assert got["assist"][:len(want)].tolist() == [list(r) for r in want]
+        running, counts = 0, []
+        for loc in range(out_local):
+            for src in range(R):
+                running += sum(1 for r in source_major if r[0] == src and demo_local_expert(case, r[3]) == loc)
+                counts.append(running)
+        assert got["send_counts"].tolist() == counts
+        per_expert = [sum(1 for r in want if demo_local_expert(case, r[3]) == loc) for loc in range(out_local)]
+        assert got["expert_token_nums"].tolist() == per_expert
+        for row, (src, t, _, _) in enumerate(want):
+            assert np.array_equal(got["expand_x"][row].view(np.uint16), x[src, t])
+        total += len(want)
+    # closed form: every live token reaches each shared expert once, every valid routed id once
+    live_tokens = sum(sum(l) for l in live)
+    valid = sum(1 for s in range(R) for t in range(bs) for k in range(K) if live[s][t] and 0 <= ids[s, t, k] < E)
+    assert total == live_tokens * S + valid
+
+
+@pytest.mark.parametrize("shape", [s for s in SHARED_SHAPES if s[5] == s[6]])     # the MVP route needs S == SR
+@pytest.mark.parametrize("masked", [False, True])
+def test_shared_experts_mvp_route_matches_demo_golden(orc, shape, masked):
+    R, bs, h, K, E, S, SR = shape
+    rng = np.random.default_rng(sum(shape) * 3 + masked)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16, shared_expert_num=S, shared_expert_rank_num=SR, token_nums_type=1)
+    ids = rand_ids(rng, R, bs, K, E, invalid_frac=0.1)
+    x = rand_x(rng, R, bs, h)
+    mask = (rng.random((R, bs)) < 0.7).astype(np.uint8) if masked else None
+    live = [[bool(mask[s][t]) for t in range(bs)] for s in range(R)] if masked else [[True] * bs] * R
+    le = case.local_experts
+    for dst in range(R):
+        got = orc.mvp_dispatch(case, dst, x, ids, mask)
+        want = demo_routes(case, dst, ids, live)
+        assert got["rows"] == len(want)
+        assert got["assist"][:len(want)].tolist() == [list(r) for r in want]
+        assert got["recv_counts"].tolist() == [sum(1 for r in want if r[0] == src) for src in range(R)]
+        # per-expert counts follow the kernel, which files a shared row under its expert id
+        # (src/ep/kernels/tilexr_ep_dispatch_helpers.h:99-101, tilexr_ep_combine_helpers.h:124-128), not the demo's
+        # "local expert 0"; the two agree for shared expert 0
+        counts = [0] * le
+        for r in want:
+            loc = r[3] if r[3] < S else (r[3] - S) % le
+            if loc < le:
+                counts[loc] += 1
+        assert got["expert_token_nums"].tolist() == counts
+        if dst == 0 and S >= 1:
+            assert counts[0] >= sum(1 for r in want if r[3] == 0)
+
+
+def test_shared_slots_enter_the_memory_combine_after_the_routed_ones(orc):
+    R, bs, h, K, E, S, SR = 4, 5, 16, 2, 6, 2, 2
+    rng = np.random.default_rng(77)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16, shared_expert_num=S, shared_expert_rank_num=SR, token_nums_type=1)
+    ids = rand_ids(rng, R, bs, K, E)
+    x = torch.from_numpy(rng.standard_normal((R, bs, h)).astype(np.float32)).to(torch.bfloat16)
+    xb = x.view(torch.int16).numpy().view(np.uint16)
+    w = rng.random((R, bs, K)).astype(np.float32)
+    outs = [orc.mem_dispatch(case, d, xb, ids) for d in range(R)]
+    mr = case.max_rows
+    eo = np.zeros((R, mr, h), np.uint16)
+    asst = np.zeros((R, mr, 4), np.int32)
+    sc = np.zeros((R, case.local_experts * R), np.int32)
+    for d, o in enumerate(outs):
+        eo[d], asst[d] = o["expand_x"].view(np.uint16), o["assist"]
+        sc[d, :o["send_counts"].size] = o["send_counts"]
+    for r in range(R):
+        y = orc.mem_combine(case, r, eo, asst, sc, expert_scales=w[r])
+        xf = x[r].to(torch.float32).numpy()
+        for t in range(bs):
+            acc = np.zeros(h, np.float32)
+            for k in range(K):
+                acc = acc + xf[t] * np.float32(w[r, t, k])        # identity experts: every slot returns x[t]
+            for _ in range(S):
+                acc = acc + xf[t]
+            want = torch.from_numpy(acc).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+            assert np.array_equal(y[t], want)

@@ -236,8 +236,8 @@ int DispatchMvp(const EpDispatchParams &p)
     if (ret != kOk) {
         return ret;
     }
-    if ((p.tpWorldSize != 0 && p.tpWorldSize != 1) || p.sharedExpertNum != 0) {
-        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // tensor-parallel groups and shared experts: not built yet
+    if (p.tpWorldSize != 0 && p.tpWorldSize != 1) {
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // tensor-parallel groups: not built
     }
     int64_t magic = 0;
     ret = TileXRCommNextMagic(p.comm, &magic);
@@ -288,9 +288,6 @@ int DispatchMemory(const EpDispatchParams &p)
     ret = TileXREpValidateDispatchMemoryConfig(rules, *args, kEpReferenceBlockDim, &config, false);
     if (ret != kOk) {
         return ret;
-    }
-    if (p.sharedExpertNum != 0) {
-        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // shared-expert ranks: not built yet
     }
     int64_t magic = 0;
     ret = TileXRCommNextMagic(p.comm, &magic);
@@ -362,9 +359,6 @@ int CombineMemory(const EpCombineParams &p)
     ret = TileXREpValidateCombineMemoryConfig(p, *args, kEpReferenceBlockDim, &config, false);
     if (ret != kOk) {
         return ret;
-    }
-    if (p.sharedExpertNum != 0) {
-        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // shared-expert slots: not built yet
     }
     int64_t magic = 0;
     ret = TileXRCommNextMagic(p.comm, &magic);

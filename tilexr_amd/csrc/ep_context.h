@@ -42,13 +42,16 @@ struct ExchangeShape {
     int64_t topK = 0;
     int64_t experts = 0;
     int64_t quantMode = 0;
+    int64_t sharedNum = 0;       // shared experts every active token is also sent to
+    int64_t sharedRanks = 0;     // ranks [0, sharedRanks) host them
     int dtype = 0;
     int outDtype = 0;
     bool memoryRoute = false;
     bool operator==(const ExchangeShape &o) const
     {
         return bs == o.bs && h == o.h && topK == o.topK && experts == o.experts && quantMode == o.quantMode &&
-            dtype == o.dtype && outDtype == o.outDtype && memoryRoute == o.memoryRoute;
+            sharedNum == o.sharedNum && sharedRanks == o.sharedRanks && dtype == o.dtype && outDtype == o.outDtype &&
+            memoryRoute == o.memoryRoute;
     }
 };
 

@@ -28,11 +28,32 @@ struct StageLayout {
     int64_t expertTotalOffset;   // in ints
 };
 
+// Builds the per-source route tables of a dispatch with shared experts: for every token its sharedNum shared routes
+// followed by its topK routed ones, as positions in the world's key space (rank * keysPerRank + local index).
+struct AugmentLaunch {
+    const int32_t *ids;      // [bs, topK]
+    int64_t bs;
+    int64_t topK;
+    int64_t moeExpertNum;
+    int rankSize;
+    int srcRank;
+    int sharedNum;
+    int sharedRanks;
+    int localExperts;        // routed experts per non-shared rank
+    int keysPerRank;
+    bool sharedAtExpertId;   // local index of shared route s on its rank: s (MVP route) or 0 (memory route)
+    int32_t *keyIdsOut;      // [bs, sharedNum + topK]; -1 = not routed
+    int32_t *tupleExpertsOut;// [bs, sharedNum + topK]
+    hipStream_t stream;
+};
+
 struct DrainPlanLaunch {
     StageLayout stage;
     int rankSize;
     int dstRank;
-    int localExperts;
+    int localExperts;        // keys per rank in the staging areas' key space
+    int outLocalExperts;     // memory route: segments per source on this rank (1 on a shared-expert rank)
+    int tokenNumsCount;      // entries of expertTokenNumsOut
     bool memoryRoute;        // segments (localExpert, src) with inclusive-sum counts, else (src) with plain counts
     int32_t *planOffsets;    // [numSeg + 1] exclusive offsets (scratch of the destination rank)
     int32_t *countsOut;
@@ -47,6 +68,7 @@ struct DrainCopyLaunch {
     int rankSize;
     int dstRank;
     int localExperts;
+    int outLocalExperts;
     bool memoryRoute;
     const int32_t *planOffsets;
     int64_t maxRows;
@@ -70,7 +92,7 @@ struct ReturnRowsLaunch {
     int rankSize;
     int expertRank;          // the calling rank
     int64_t bs;
-    int64_t topK;
+    int64_t topK;            // slots per token: rows whose topKId is not below it are skipped
     uint64_t epoch;
     char *slots;             // [R] x slotsStride: rows at slot token*topK + k of the source rank
     int64_t slotsStride;
@@ -79,6 +101,7 @@ struct ReturnRowsLaunch {
     hipStream_t stream;
 };
 
+hipError_t LaunchAugment(const AugmentLaunch &l);
 hipError_t LaunchDrainPlan(const DrainPlanLaunch &l);
 hipError_t LaunchDrainCopy(const DrainCopyLaunch &l);
 hipError_t LaunchReturnRows(const ReturnRowsLaunch &l);

@@ -30,11 +30,60 @@ __device__ __forceinline__ void SegmentOf(int idx, int rankSize, int dstRank, in
     }
 }
 
+// Shared experts: route table of one source rank in the world's key space.
+//   shared route s   -> rank srcRank % per + s * per (per = sharedRanks / sharedNum), tuple expert id s
+//   routed id e      -> rank sharedRanks + e / localExperts, local index e % localExperts, tuple expert id sharedNum + e
+// (reference: src/ep/kernels/tilexr_ep_dispatch_helpers.h:78-103, tilexr_ep_dispatch_memory_kernel.h:635-643,686-688,
+//  tests/ep/demo/tilexr_ep_dispatch_demo.cpp:647-673)
+struct AugmentArgs {
+    const int32_t *ids;
+    int n;                   // bs * (sharedNum + topK)
+    int topK;
+    int moeExpertNum;
+    int srcRank;
+    int sharedNum;
+    int sharedRanks;
+    int localExperts;
+    int keysPerRank;
+    int sharedAtExpertId;
+    int32_t *keyIdsOut;
+    int32_t *tupleExpertsOut;
+};
+
+__global__ __launch_bounds__(kThreads) void ep_augment_kernel(AugmentArgs a)
+{
+    const int i = blockIdx.x * kThreads + threadIdx.x;
+    if (i >= a.n) {
+        return;
+    }
+    const int perToken = a.sharedNum + a.topK;
+    const int token = i / perToken;
+    const int pos = i % perToken;
+    int keyId = -1;
+    int tupleExpert = -1;
+    if (pos < a.sharedNum) {
+        const int per = a.sharedRanks / a.sharedNum;
+        const int dst = a.srcRank % per + pos * per;
+        keyId = dst * a.keysPerRank + (a.sharedAtExpertId ? pos : 0);
+        tupleExpert = pos;
+    } else {
+        const int e = a.ids[token * a.topK + (pos - a.sharedNum)];
+        if (e >= 0 && e < a.moeExpertNum) {
+            keyId = (a.sharedRanks + e / a.localExperts) * a.keysPerRank + e % a.localExperts;
+            tupleExpert = a.sharedNum + e;
+        }
+    }
+    a.keyIdsOut[i] = keyId;
+    a.tupleExpertsOut[i] = tupleExpert;
+}
+
 struct DrainPlanArgs {
     StageLayout stage;
     int rankSize;
     int dstRank;
     int localExperts;
+    int outLocalExperts;
+    int tokenNumsCount;
     int memoryRoute;
     int32_t *planOffsets;
     int32_t *countsOut;
@@ -50,7 +99,7 @@ __global__ __launch_bounds__(kThreads) void ep_drain_plan_kernel(DrainPlanArgs a
     __shared__ int s_tok[kMaxKeys];
     __shared__ int s_part[kThreads];
     const int tid = threadIdx.x;
-    const int numSeg = a.memoryRoute ? a.localExperts * a.rankSize : a.rankSize;
+    const int numSeg = a.memoryRoute ? a.outLocalExperts * a.rankSize : a.rankSize;
     for (int idx = tid; idx < numSeg; idx += kThreads) {
         int src, key;
         SegmentOf(idx, a.rankSize, a.dstRank, a.localExperts, a.memoryRoute != 0, &src, &key);
@@ -73,7 +122,7 @@ __global__ __launch_bounds__(kThreads) void ep_drain_plan_kernel(DrainPlanArgs a
         a.planOffsets[numSeg] = total;
     }
     // rows per local expert
-    for (int le = tid; le < a.localExperts; le += kThreads) {
+    for (int le = tid; le < a.tokenNumsCount; le += kThreads) {
         int n = 0;
         if (a.memoryRoute) {
             for (int s = 0; s < a.rankSize; ++s) {
@@ -90,16 +139,16 @@ __global__ __launch_bounds__(kThreads) void ep_drain_plan_kernel(DrainPlanArgs a
     }
     __syncthreads();
     if (a.tokenNumsType == 0) {
-        for (int le = tid; le < a.localExperts; le += kThreads) {
+        for (int le = tid; le < a.tokenNumsCount; le += kThreads) {
             s_cnt[le] = s_tok[le];
         }
         __syncthreads();
-        BlockExclusiveScan(s_cnt, a.localExperts, s_part);
-        for (int le = tid; le < a.localExperts; le += kThreads) {
+        BlockExclusiveScan(s_cnt, a.tokenNumsCount, s_part);
+        for (int le = tid; le < a.tokenNumsCount; le += kThreads) {
             a.expertTokenNumsOut[le] = static_cast<int64_t>(s_cnt[le]) + s_tok[le];
         }
     } else {
-        for (int le = tid; le < a.localExperts; le += kThreads) {
+        for (int le = tid; le < a.tokenNumsCount; le += kThreads) {
             a.expertTokenNumsOut[le] = s_tok[le];
         }
     }
@@ -125,6 +174,7 @@ struct DrainCopyArgs {
     int rankSize;
     int dstRank;
     int localExperts;
+    int outLocalExperts;
     int memoryRoute;
     const int32_t *planOffsets;
     int64_t rowBytes;
@@ -136,7 +186,7 @@ struct DrainCopyArgs {
 
 __global__ __launch_bounds__(kThreads) void ep_drain_copy_kernel(DrainCopyArgs a)
 {
-    const int numSeg = a.memoryRoute ? a.localExperts * a.rankSize : a.rankSize;
+    const int numSeg = a.memoryRoute ? a.outLocalExperts * a.rankSize : a.rankSize;
     const int row = blockIdx.x;
     if (row >= a.planOffsets[numSeg]) {
         return;
@@ -237,6 +287,26 @@ __global__ __launch_bounds__(kThreads) void ep_return_rows_kernel(ReturnRowsArgs
 
 } // namespace
 
+hipError_t LaunchAugment(const AugmentLaunch &l)
+{
+    AugmentArgs a {};
+    a.ids = l.ids;
+    a.n = static_cast<int>(l.bs * (l.sharedNum + l.topK));
+    a.topK = static_cast<int>(l.topK);
+    a.moeExpertNum = static_cast<int>(l.moeExpertNum);
+    a.srcRank = l.srcRank;
+    a.sharedNum = l.sharedNum;
+    a.sharedRanks = l.sharedRanks;
+    a.localExperts = l.localExperts;
+    a.keysPerRank = l.keysPerRank;
+    a.sharedAtExpertId = l.sharedAtExpertId ? 1 : 0;
+    a.keyIdsOut = l.keyIdsOut;
+    a.tupleExpertsOut = l.tupleExpertsOut;
+    const int grid = (a.n + kThreads - 1) / kThreads;
+    hipLaunchKernelGGL(ep_augment_kernel, dim3(grid > 0 ? grid : 1), dim3(kThreads), 0, l.stream, a);
+    return hipGetLastError();
+}
+
 hipError_t LaunchDrainPlan(const DrainPlanLaunch &l)
 {
     DrainPlanArgs a {};
@@ -244,6 +314,8 @@ hipError_t LaunchDrainPlan(const DrainPlanLaunch &l)
     a.rankSize = l.rankSize;
     a.dstRank = l.dstRank;
     a.localExperts = l.localExperts;
+    a.outLocalExperts = l.outLocalExperts;
+    a.tokenNumsCount = l.tokenNumsCount;
     a.memoryRoute = l.memoryRoute ? 1 : 0;
     a.planOffsets = l.planOffsets;
     a.countsOut = l.countsOut;
@@ -261,6 +333,7 @@ hipError_t LaunchDrainCopy(const DrainCopyLaunch &l)
     a.rankSize = l.rankSize;
     a.dstRank = l.dstRank;
     a.localExperts = l.localExperts;
+    a.outLocalExperts = l.outLocalExperts;
     a.memoryRoute = l.memoryRoute ? 1 : 0;
     a.planOffsets = l.planOffsets;
     a.rowBytes = l.rowBytes;

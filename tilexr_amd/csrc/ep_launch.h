@@ -74,6 +74,12 @@ struct RoutePlaceLaunch {
     CountScratch scratch;
     int32_t srcRank;
     int32_t expertIdBias;        // added to the id stored in the assist tuple (shared experts shift ids)
+    // Shared experts (logical multi-rank worlds): a token's routes are its `sharedNum` shared routes followed by
+    // its routed ones, `topK` counts both, `ids` holds positions in the world's key space and `tupleExperts`
+    // the expert id each route reports in its assist tuple.  The tuple's topKId is topK - sharedNum + s for
+    // shared route s and the routed index otherwise.
+    int32_t sharedNum;
+    const int32_t *tupleExperts; // [n] or nullptr (the tuple then reports ids[i] + expertIdBias)
     int32_t *rowOf;              // [n] out
     int32_t *assist;             // [rows, 4] out
     hipStream_t stream;
@@ -144,6 +150,9 @@ struct ReduceLaunch {
     int64_t bs;
     int64_t h;
     int64_t topK;
+    int64_t sharedSlots;             // slots per token beyond topK (shared experts): summed after the routed ones
+                                     // with weight 1; the row map / inverse then has topK + sharedSlots entries
+                                     // per token while expertScales keeps topK
     void *y;
     const uint64_t *tileFlags;       // optional: a tile is ready once the upper half of its word equals flagEpoch
     int64_t tileRows;

@@ -27,6 +27,8 @@ struct PlaceArgs {
     int capacity;
     int32_t srcRank;
     int32_t expertIdBias;
+    int32_t sharedNum;           // leading shared routes per token (see RoutePlaceLaunch)
+    const int32_t *tupleExperts; // optional [n]: expert id reported by the tuple
     int32_t *rowOf;              // optional out [n]
     int32_t *assist;             // out [rows, 4]
 };
@@ -46,6 +48,8 @@ inline PlaceArgs MakePlaceArgs(const RoutePlaceLaunch &l)
     a.capacity = static_cast<int>(l.capacity);
     a.srcRank = l.srcRank;
     a.expertIdBias = l.expertIdBias;
+    a.sharedNum = l.sharedNum;
+    a.tupleExperts = l.tupleExperts;
     a.rowOf = l.rowOf;
     a.assist = l.assist;
     return a;
@@ -63,10 +67,13 @@ __device__ __forceinline__ int PlaceRoute(const PlaceArgs &a, int i)
         if (a.capacity <= 0 || within < a.capacity) {
             row = a.keyOffset[key] + within;
             int32_t *tuple = a.assist + static_cast<int64_t>(row) * 4;
+            const int pos = i % a.topK;
             tuple[0] = a.srcRank;
             tuple[1] = i / a.topK;
-            tuple[2] = i % a.topK;
-            tuple[3] = e + a.expertIdBias;
+            // shared routes come first in a token's row and report the slots after the routed ones
+            // (reference: src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:536-568)
+            tuple[2] = pos < a.sharedNum ? a.topK - a.sharedNum + pos : pos - a.sharedNum;
+            tuple[3] = a.tupleExperts != nullptr ? a.tupleExperts[i] : e + a.expertIdBias;
         }
     }
     if (a.rowOf != nullptr) {

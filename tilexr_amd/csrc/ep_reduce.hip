@@ -17,6 +17,8 @@
 //                 type first (no reference counterpart)
 #include <hip/hip_runtime.h>
 
+#include <cstdlib>
+
 #include "ep_kernel_common.cuh"
 #include "ep_launch.h"
 #include "ep_numerics.cuh"
@@ -39,6 +41,7 @@ struct ReduceArgs {
     int bs;
     int h;
     int topK;
+    int slots;                       // rows summed per token: topK routed ones, then the shared-expert slots
     void *y;
     int colSlices;                   // slices a row is cut into (vec kernel, wide rows), else 1
     const uint64_t *tileFlags;
@@ -148,8 +151,8 @@ template <bool FENCE>
 __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
     float *weights)
 {
-    for (int k = lane; k < a.topK; k += lanes) {
-        const int64_t slot = static_cast<int64_t>(tokOk ? token : 0) * a.topK + k;
+    for (int k = lane; k < a.slots; k += lanes) {
+        const int64_t slot = static_cast<int64_t>(tokOk ? token : 0) * a.slots + k;
         int row = tokOk ? LookupRow(a, slot) : -1;
         if (row >= 0 && a.tileFlags != nullptr && !WaitTile(a, row)) {
             if (a.deviceStatus != nullptr) {
@@ -158,9 +161,12 @@ __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool 
             row = -1;
         }
         rows[k] = row;
-        weights[k] = (tokOk && a.expertScales != nullptr) ? a.expertScales[slot] : 1.0f;
+        // shared-expert slots follow the routed ones and carry no gate weight
+        // (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:650-657)
+        weights[k] = (tokOk && a.expertScales != nullptr && k < a.topK) ?
+            a.expertScales[static_cast<int64_t>(token) * a.topK + k] : 1.0f;
     }
-    if (FENCE && a.tileFlags != nullptr && lane < a.topK) {
+    if (FENCE && a.tileFlags != nullptr && lane < a.slots) {
         // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
         // workgroup after the barrier that follows) are at least as new as the flag values seen above
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -196,7 +202,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
         __syncthreads();
         if (KIND == kReducePerAdd) {
             if (lane == 0) {
-                SortRows(s_row[tg], a.topK, a.orderKeys);
+                SortRows(s_row[tg], a.slots, a.orderKeys);
             }
             __syncthreads();
         }
@@ -211,14 +217,14 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             }
         }
         // control flow below is uniform across the lanes that share a token (the MXFP8 round trip shuffles)
-        for (int k0 = 0; k0 < a.topK; k0 += KB) {
+        for (int k0 = 0; k0 < a.slots; k0 += KB) {
             u32x4 v16[KB][V];
             int rowOfK[KB];
 #pragma unroll
             for (int u = 0; u < KB; ++u) {
                 const int k = k0 + u;
                 // the lanes of a wave share one token, so the row is wave-uniform
-                const int row = __builtin_amdgcn_readfirstlane((k < a.topK && active) ? s_row[tg][k] : -1);
+                const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
                 rowOfK[u] = row;
                 const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
                 const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
@@ -340,14 +346,14 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
                 acc[j][e] = 0.0f;
             }
         }
-        for (int k0 = 0; k0 < a.topK; k0 += KB) {
+        for (int k0 = 0; k0 < a.slots; k0 += KB) {
             u32x4 q[KB][V];
             float sc[KB][V];
             int rowOfK[KB];
 #pragma unroll
             for (int u = 0; u < KB; ++u) {
                 const int k = k0 + u;
-                const int row = __builtin_amdgcn_readfirstlane((k < a.topK && active) ? s_row[tg][k] : -1);
+                const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
                 rowOfK[u] = row;
                 const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
                 const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
@@ -458,7 +464,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
         __syncthreads();
         if (kind == kReducePerAdd) {
             if (tid == 0) {
-                SortRows(s_row, a.topK, a.orderKeys);
+                SortRows(s_row, a.slots, a.orderKeys);
             }
             __syncthreads();
         }
@@ -473,7 +479,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
                 acc[i] = 0.0f;
             }
             if (active) {
-                for (int k = 0; k < a.topK; ++k) {
+                for (int k = 0; k < a.slots; ++k) {
                     const int row = s_row[k];
                     if (row < 0) {
                         continue;
@@ -549,10 +555,11 @@ void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
     if (gridLimit > 0 && grid > gridLimit * (kThreads / threads)) {
         grid = gridLimit * (kThreads / threads);
     }
+    static const int extraLds = getenv("TILEXR_EP_REDUCE_LDS") ? atoi(getenv("TILEXR_EP_REDUCE_LDS")) : 0;
     if (a.tileFlags != nullptr) {
         hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, true>), dim3(grid), dim3(threads), 0, stream, a);
     } else {
-        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, false>), dim3(grid), dim3(threads), 0, stream, a);
+        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, false>), dim3(grid), dim3(threads), extraLds, stream, a);
     }
 }
 
@@ -633,6 +640,7 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     a.bs = static_cast<int>(l.bs);
     a.h = static_cast<int>(l.h);
     a.topK = static_cast<int>(l.topK);
+    a.slots = static_cast<int>(l.topK + l.sharedSlots);
     a.y = l.y;
     a.tileFlags = l.tileFlags;
     a.tileRows = static_cast<int>(l.tileRows);

@@ -7,6 +7,8 @@
 // the world has called, the DRAIN half of every rank is enqueued on that rank's own stream behind events of all
 // send halves.  A rank's outputs are therefore complete once every rank has made the call and the rank's stream
 // has been synchronised -- the same moment the reference's kernels would pass their barriers.
+#include <algorithm>
+
 #include "ep_context.h"
 #include "ep_exchange.h"
 #include "ep_host.h"
@@ -39,12 +41,22 @@ bool EnsureEvents(RankEvents *e)
     return true;
 }
 
+// Key space of a world: position = rank * keysPerRank + local index on that rank.  Without shared experts this is
+// the expert id itself (keysPerRank = experts per rank).  With shared experts (reference: expert placement in
+// src/ep/kernels/tilexr_ep_dispatch_helpers.h:63-103) ranks [0, sharedRanks) host them, the routed experts are spread
+// over the other ranks, and a shared route takes local index 0 on its rank (memory route: a shared rank presents one
+// local expert, tilexr_ep_dispatch_memory_kernel.h:1153) or its own expert id (MVP route: the drain files a shared row
+// under index expertId, tilexr_ep_combine_helpers.h:124-128), hence keysPerRank = max(localExperts, sharedNum) there.
 struct StagePlan {
     StageLayout layout {};
     int64_t rowBytes = 0;
     int64_t scaleBytesPerRow = 0;
     int64_t numKeys = 0;
     int64_t keyDiv = 1;
+    int64_t localExperts = 0;    // routed experts per non-shared rank
+    int64_t keysPerRank = 0;
+    int64_t keySpace = 0;        // rankSize * keysPerRank
+    int64_t perToken = 0;        // routes per token: shared + topK
     bool expertHist = false;
 };
 
@@ -52,20 +64,23 @@ struct StagePlan {
 bool PlanStage(EpWorld *world, const ExchangeShape &shape, bool reserve, StagePlan *plan)
 {
     const int64_t R = world->rankSize;
-    const int64_t n = shape.bs * shape.topK;
-    const int64_t localExperts = shape.experts / R;
+    plan->perToken = shape.topK + shape.sharedNum;
+    const int64_t n = shape.bs * plan->perToken;
+    plan->localExperts = shape.experts / (R - shape.sharedRanks);
+    plan->keysPerRank = shape.memoryRoute ? plan->localExperts : std::max(plan->localExperts, shape.sharedNum);
+    plan->keySpace = R * plan->keysPerRank;
     plan->rowBytes = shape.quantMode == TILEXR_EP_QUANT_NONE ? shape.h * 2 : shape.h;
     plan->scaleBytesPerRow = shape.quantMode == TILEXR_EP_QUANT_TOKEN_INT8 ? 4 :
         (shape.quantMode == TILEXR_EP_QUANT_MXFP8 ? MxScaleBytes(shape.h) : 0);
-    plan->numKeys = shape.memoryRoute ? shape.experts : R;
-    plan->keyDiv = shape.memoryRoute ? 1 : localExperts;
+    plan->numKeys = shape.memoryRoute ? plan->keySpace : R;
+    plan->keyDiv = shape.memoryRoute ? 1 : plan->keysPerRank;
     plan->expertHist = !shape.memoryRoute;
     StageLayout &l = plan->layout;
     l.rowsStride = Align256(n * plan->rowBytes);
     l.scalesOffset = Align256(n * 16);
     l.auxStride = l.scalesOffset + Align256(n * plan->scaleBytesPerRow);
     l.expertTotalOffset = plan->numKeys + 1;
-    l.countsStride = (plan->numKeys + 1 + shape.experts + 63) / 64 * 64;
+    l.countsStride = (plan->numKeys + 1 + plan->keySpace + 63) / 64 * 64;
     if (reserve) {
         if (!world->stageRows.Reserve(static_cast<size_t>(R * l.rowsStride), false) ||
             !world->stageAux.Reserve(static_cast<size_t>(R * l.auxStride), false) ||
@@ -85,8 +100,11 @@ int DrainRank(EpWorld *world, int q, const ExchangeShape &shape, const StagePlan
     const EpDispatchParams &p = world->pendingDispatch[static_cast<size_t>(q)].params;
     hipStream_t stream = static_cast<hipStream_t>(p.stream);
     const int R = world->rankSize;
-    const int localExperts = static_cast<int>(shape.experts / R);
-    const int64_t numSeg = shape.memoryRoute ? static_cast<int64_t>(localExperts) * R : R;
+    const int localExperts = static_cast<int>(plan.keysPerRank);
+    // a shared-expert rank presents one local expert on the memory route
+    // (reference: src/ep/kernels/tilexr_ep_dispatch_memory_kernel.h:1153, tests/ep/demo/tilexr_ep_dispatch_demo.cpp:632-635)
+    const int outLocalExperts = q < shape.sharedRanks ? 1 : static_cast<int>(plan.localExperts);
+    const int64_t numSeg = shape.memoryRoute ? static_cast<int64_t>(outLocalExperts) * R : R;
     for (int s = 0; s < R; ++s) {
         if (hipStreamWaitEvent(stream, world->dispatchEvents[static_cast<size_t>(s)].sent, 0) != hipSuccess) {
             return TileXR::TILEXR_ERROR_INTERNAL;
@@ -100,6 +118,8 @@ int DrainRank(EpWorld *world, int q, const ExchangeShape &shape, const StagePlan
     dp.rankSize = R;
     dp.dstRank = q;
     dp.localExperts = localExperts;
+    dp.outLocalExperts = outLocalExperts;
+    dp.tokenNumsCount = shape.memoryRoute ? outLocalExperts : static_cast<int>(plan.localExperts);
     dp.memoryRoute = shape.memoryRoute;
     dp.planOffsets = static_cast<int32_t *>(comm->drainScratch.ptr);
     dp.countsOut = p.epRecvCountsOut;
@@ -116,9 +136,10 @@ int DrainRank(EpWorld *world, int q, const ExchangeShape &shape, const StagePlan
     dc.rankSize = R;
     dc.dstRank = q;
     dc.localExperts = localExperts;
+    dc.outLocalExperts = outLocalExperts;
     dc.memoryRoute = shape.memoryRoute;
     dc.planOffsets = dp.planOffsets;
-    dc.maxRows = static_cast<int64_t>(R) * shape.bs * shape.topK;
+    dc.maxRows = static_cast<int64_t>(R) * shape.bs * plan.perToken;
     dc.rowBytes = plan.rowBytes;
     dc.scaleBytesPerRow = plan.scaleBytesPerRow;
     dc.expandXOut = p.expandXOut;
@@ -144,7 +165,14 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     EpWorld *world = comm->world;
     const int R = world->rankSize;
     const int r = comm->rank;
-    if (!WithinKernelLimits(p.bs, p.h, p.topK, p.moeExpertNum, R) || p.extended) {
+    const int64_t shared = p.sharedExpertNum;
+    const int64_t keySpaceBound = static_cast<int64_t>(R) * std::max(p.moeExpertNum / (R - p.sharedExpertRankNum), shared);
+    if (!WithinKernelLimits(p.bs, p.h, p.topK + shared, std::max(p.moeExpertNum, keySpaceBound), R) || p.extended) {
+        return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+    }
+    if (shared > 0 && p.xActiveMask != nullptr && memoryRoute && p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT) {
+        // the reference compacts the tokens that keep at least one route before it walks the shared routes
+        // (tilexr_ep_dispatch_memory_kernel.h:1483-1500, 645-647); that combination is not built
         return TileXR::TILEXR_ERROR_NOT_SUPPORT;
     }
     hipStream_t stream = static_cast<hipStream_t>(p.stream);
@@ -154,6 +182,8 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     shape.topK = p.topK;
     shape.experts = p.moeExpertNum;
     shape.quantMode = p.quantMode;
+    shape.sharedNum = shared;
+    shape.sharedRanks = p.sharedExpertRankNum;
     shape.dtype = static_cast<int>(p.dtype);
     shape.outDtype = static_cast<int>(p.expandXOutDtype);
     shape.memoryRoute = memoryRoute;
@@ -193,12 +223,41 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     }
 
     // ---- send half: group this rank's rows by destination in its staging area ----
-    const int64_t n = p.bs * p.topK;
-    const CountScratchLayout cs = PlanCountScratch(n, plan.numKeys, p.moeExpertNum, plan.expertHist);
-    if (!comm->dispatchScratch.Reserve(static_cast<size_t>(cs.totalBytes), true)) {
+    const int64_t n = p.bs * plan.perToken;
+    const CountScratchLayout cs = PlanCountScratch(n, plan.numKeys, plan.keySpace, plan.expertHist);
+    const int64_t tableBytes = shared > 0 ? Align256(n * 4) : 0;      // key ids, then tuple expert ids
+    if (!comm->dispatchScratch.Reserve(static_cast<size_t>(cs.totalBytes + 2 * tableBytes), true)) {
         return TileXR::TILEXR_ERROR_INTERNAL;
     }
     CountScratch scratch = CarveCountScratch(comm->dispatchScratch.ptr, cs, plan.expertHist);
+    const int32_t *routeIds = p.expertIds;
+    const int32_t *tupleExperts = nullptr;
+    if (shared > 0) {
+        int32_t *keyIds = reinterpret_cast<int32_t *>(static_cast<char *>(comm->dispatchScratch.ptr) + cs.totalBytes);
+        int32_t *tuples = reinterpret_cast<int32_t *>(static_cast<char *>(comm->dispatchScratch.ptr) + cs.totalBytes +
+            tableBytes);
+        AugmentLaunch aug {};
+        aug.ids = p.expertIds;
+        aug.bs = p.bs;
+        aug.topK = p.topK;
+        aug.moeExpertNum = p.moeExpertNum;
+        aug.rankSize = R;
+        aug.srcRank = r;
+        aug.sharedNum = static_cast<int>(shared);
+        aug.sharedRanks = static_cast<int>(p.sharedExpertRankNum);
+        aug.localExperts = static_cast<int>(plan.localExperts);
+        aug.keysPerRank = static_cast<int>(plan.keysPerRank);
+        aug.sharedAtExpertId = !memoryRoute;
+        aug.keyIdsOut = keyIds;
+        aug.tupleExpertsOut = tuples;
+        aug.stream = stream;
+        const int ar = LaunchStatus(LaunchAugment(aug), "route tables");
+        if (ar != kOk) {
+            return ar;
+        }
+        routeIds = keyIds;
+        tupleExperts = tuples;
+    }
     int32_t *myCounts = plan.layout.counts + static_cast<int64_t>(r) * plan.layout.countsStride;
     scratch.keyOffset = myCounts;
     scratch.expertTotal = myCounts + plan.layout.expertTotalOffset;
@@ -207,7 +266,7 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     char *myAux = plan.layout.aux + static_cast<int64_t>(r) * plan.layout.auxStride;
 
     RouteCountLaunch count {};
-    count.ids = p.expertIds;
+    count.ids = routeIds;
     count.mask = reinterpret_cast<const uint8_t *>(p.xActiveMask);
     if (p.xActiveMask == nullptr) {
         count.maskMode = kMaskNone;
@@ -217,8 +276,8 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
         count.maskMode = p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT ? kMaskPerRoute : kMaskTokenPrefix;
     }
     count.bs = p.bs;
-    count.topK = p.topK;
-    count.numExperts = p.moeExpertNum;
+    count.topK = plan.perToken;
+    count.numExperts = plan.keySpace;
     count.keyDiv = plan.keyDiv;
     count.numKeys = plan.numKeys;
     count.capacity = 0;
@@ -230,14 +289,16 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
         return ret;
     }
     RoutePlaceLaunch place {};
-    place.ids = p.expertIds;
+    place.ids = routeIds;
     place.bs = p.bs;
-    place.topK = p.topK;
+    place.topK = plan.perToken;
     place.keyDiv = plan.keyDiv;
     place.numKeys = plan.numKeys;
     place.scratch = scratch;
     place.srcRank = r;
     place.expertIdBias = 0;
+    place.sharedNum = static_cast<int32_t>(shared);
+    place.tupleExperts = tupleExperts;
     place.rowOf = rowOf;
     place.assist = reinterpret_cast<int32_t *>(myAux);
     place.stream = stream;
@@ -250,7 +311,7 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     scatter.rowOf = rowOf;
     scatter.bs = p.bs;
     scatter.h = p.h;
-    scatter.topK = p.topK;
+    scatter.topK = plan.perToken;
     scatter.quantMode = static_cast<int>(p.quantMode);
     scatter.inputBf16 = memoryRoute && p.dtype == TileXR::TILEXR_DATA_TYPE_BFP16;
     scatter.fp8E5m2 = p.expandXOutDtype == TileXR::TILEXR_DATA_TYPE_FP8E5M2;
@@ -298,7 +359,11 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
     EpWorld *world = comm->world;
     const int R = world->rankSize;
     const int er = comm->rank;
-    if (!WithinKernelLimits(p.bs, p.h, p.topK, p.moeExpertNum, R) || p.extended) {
+    // shared-expert rows come back to the slots after the routed ones on the memory route; the MVP route's combine
+    // drops them (reference: src/ep/kernels/tilexr_ep_combine_kernel.cpp:94-97)
+    const int64_t shared = memoryRoute ? p.sharedExpertNum : 0;
+    const int64_t perToken = p.topK + shared;
+    if (!WithinKernelLimits(p.bs, p.h, perToken, p.moeExpertNum, R) || p.extended) {
         return TileXR::TILEXR_ERROR_NOT_SUPPORT;
     }
     hipStream_t stream = static_cast<hipStream_t>(p.stream);
@@ -308,6 +373,8 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
     shape.topK = p.topK;
     shape.experts = p.moeExpertNum;
     shape.quantMode = p.quantMode;
+    shape.sharedNum = shared;
+    shape.sharedRanks = memoryRoute ? p.sharedExpertRankNum : 0;
     shape.dtype = static_cast<int>(p.dtype);
     shape.memoryRoute = memoryRoute;
 
@@ -324,7 +391,7 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
     for (const PendingCombine &pc : world->pendingCombine) {
         first = first && !pc.present;
     }
-    const int64_t n = p.bs * p.topK;
+    const int64_t n = p.bs * perToken;
     const int64_t rowBytes = p.h * 2;
     const int64_t slotsStride = Align256(n * rowBytes);
     const int64_t metaStride = (2 * n + 31) / 32 * 32;
@@ -355,7 +422,10 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
     back.expertOut = p.expertOut;
     back.assist = p.assistInfoForCombine;
     back.counts = p.epRecvCounts;
-    back.numCounts = memoryRoute ? p.moeExpertNum : R;      // localExperts * R == experts
+    // memory route: the rows of this expert rank = last entry of its sendCounts, which has one block of R entries per
+    // local expert (a single block on a shared-expert rank)
+    const int64_t localExperts = p.moeExpertNum / (R - shape.sharedRanks);
+    back.numCounts = memoryRoute ? (er < shape.sharedRanks ? 1 : localExperts) * R : R;
     back.memoryRoute = memoryRoute;
     back.maxCountPerEntry = n;
     back.maxRows = static_cast<int64_t>(R) * n;
@@ -363,7 +433,7 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
     back.rankSize = R;
     back.expertRank = er;
     back.bs = p.bs;
-    back.topK = p.topK;
+    back.topK = perToken;
     back.epoch = epoch;
     back.slots = static_cast<char *>(world->combineSlots.ptr);
     back.slotsStride = slotsStride;
@@ -417,6 +487,7 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
         red.bs = rp.bs;
         red.h = rp.h;
         red.topK = rp.topK;
+        red.sharedSlots = shared;
         red.y = rp.yOut;
         red.numComputeUnits = world->numComputeUnits;
         red.stream = rs;
