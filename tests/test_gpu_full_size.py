@@ -157,3 +157,29 @@ def test_c1_checker_configuration_round_trip():
         for r in range(R):
             # two bf16 additions of the same value: 0 + x = x, x + x = 2x, both exact
             assert torch.equal(ys[r].float(), xt[r].float() * K)
+
+
+def test_rows_beyond_four_gib_keep_their_addresses():
+    """40960 tokens x 7168 x top-8: 327 680 rows of 14 336 bytes = 4.7 GB, so row offsets do not fit 32 bits.
+    Checked through properties on the device (the oracle would take minutes here): the payload rows are their source
+    rows, and combine with all weights 1/8 returns every token unchanged up to one rounding."""
+    w = workloads.Workload("wide", 1, 40960, 7168, 8, 256, routing="zipf", zipf_s=1.0, seed=77)
+    bs, h, K, E = w.bs, w.h, w.top_k, w.experts
+    x = workloads.make_x(w)
+    ids, _ = workloads.make_routing(w)
+    weights = torch.full((bs, K), 0.125, dtype=torch.float32)
+    with Session() as s:
+        t = run_layer(s, w, x, ids, weights)
+        rows = bs * K
+        assert int(t["send_counts"][-1].item()) == rows
+        a = t["assist"].long()
+        flat = a[:, 1] * K + a[:, 2]
+        assert torch.equal(t["ids"].view(-1).long()[flat], a[:, 3])
+        assert torch.equal(t["row_map"].view(-1).long()[flat], torch.arange(rows, device=DEV))
+        got = t["expand_x"].view(torch.int16).view(rows, h)
+        src = t["x"].view(torch.int16)
+        for begin in range(0, rows, 65536):                                  # in pieces: the gather is 4.7 GB
+            end = min(begin + 65536, rows)
+            assert torch.equal(got[begin:end], src[a[begin:end, 1]]), f"rows {begin}..{end}"
+        # 8 x (x / 8) summed in fp32 is x exactly (power-of-two weights), so y == x bit for bit
+        assert torch.equal(t["y"].view(torch.int16), src)

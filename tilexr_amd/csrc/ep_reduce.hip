@@ -17,8 +17,6 @@
 //                 type first (no reference counterpart)
 #include <hip/hip_runtime.h>
 
-#include <cstdlib>
-
 #include "ep_kernel_common.cuh"
 #include "ep_launch.h"
 #include "ep_numerics.cuh"
@@ -555,11 +553,10 @@ void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
     if (gridLimit > 0 && grid > gridLimit * (kThreads / threads)) {
         grid = gridLimit * (kThreads / threads);
     }
-    static const int extraLds = getenv("TILEXR_EP_REDUCE_LDS") ? atoi(getenv("TILEXR_EP_REDUCE_LDS")) : 0;
     if (a.tileFlags != nullptr) {
         hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, true>), dim3(grid), dim3(threads), 0, stream, a);
     } else {
-        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, false>), dim3(grid), dim3(threads), extraLds, stream, a);
+        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, false>), dim3(grid), dim3(threads), 0, stream, a);
     }
 }
 
