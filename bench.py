@@ -167,6 +167,7 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    torch.cuda.synchronize()        # torch's fills ran on its default stream, the library runs on `stream`
     for _ in range(args.warmup):
         step()
     torch.cuda.synchronize()

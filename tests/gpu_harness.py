@@ -1,5 +1,9 @@
 """Drives libtilexr-ep through its C ABI with torch tensors as device memory, and fetches results as numpy arrays
-shaped like the oracle's outputs (tests/ and the smoke check use it)."""
+shaped like the oracle's outputs (tests/ and the smoke check use it).
+
+Stream discipline of the tests: torch's own work (fills, host copies, comparisons) stays on torch's default stream
+and is waited for (`torch.cuda.synchronize()`) before a library call is issued on a session's own stream; library
+results are read after that stream has been synchronised."""
 import numpy as np
 import torch
 
@@ -68,6 +72,8 @@ def alloc_dispatch_outputs(bs, h, top_k, experts, ranks=1, quant=ep.Q_NONE, fill
         out["scales"] = torch.full((rows, 1), -3.0, dtype=torch.float32, device=DEV)
     else:
         out["scales"] = None
+    # the fills run on torch's default stream, the library on the caller's own (non-blocking) stream
+    torch.cuda.synchronize()
     return out
 
 

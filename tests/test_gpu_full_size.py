@@ -34,6 +34,9 @@ def run_layer(s, w, x, ids, weights):
         t["scales"] = torch.full((n, 1), -3.0, dtype=torch.float32, device=DEV)
     elif quant == ep.Q_FP8_BLOCK128:
         t["scales"] = torch.full((n, (h + 127) // 128), -3.0, dtype=torch.float32, device=DEV)
+    # the fills above run on torch's default stream, the library on the session's own (non-blocking) stream: without
+    # this wait a 4.7 GB fill can still be writing when the first rows land
+    torch.cuda.synchronize()
     st, _ = ep.dispatch_memory_ex(t["x"], t["ids"], s.comm, bs, h, K, E, t["expand_x"], t["assist"], t["token_nums"],
                                   t["send_counts"], ep.DT_BF16, s.stream, quant_mode=quant,
                                   expert_capacity=w.capacity, dynamic_scales=t["scales"], row_index_map=t["row_map"])

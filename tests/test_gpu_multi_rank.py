@@ -68,6 +68,7 @@ def run_dispatch(world, memory, xt, ids, bs, h, K, E, dtype, order=None, quant=e
     dev_mask = [None if mask is None else to_dev(mask[r]) for r in range(R)]
     dev_static = to_dev(static)
     keep = (dev_ids, dev_mask, dev_static)
+    torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
     for r in (order or range(R)):
         o = outs[r]
         if memory:
@@ -132,6 +133,7 @@ def test_mvp_dispatch_and_combine_across_ranks(shape):
                 for r in range(R):
                     t = outs[r]["expand_x"].view(torch.float16) * (1.0 + 0.25 * r)
                     eo.append(t.contiguous())
+                torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
                 for r in reversed(order):
                     st = ep.combine_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
                                        ep.DT_FP16, w.streams[r])
@@ -176,6 +178,7 @@ def test_memory_dispatch_and_combine_across_ranks(shape, dtype):
             eo = [(outs[r]["expand_x"].view(tdt) * (1.0 + 0.25 * r)).contiguous() for r in range(R)]
             dev_w = [to_dev(weights[r]) for r in range(R)]
             dev_m = [None if tmask is None else to_dev(tmask[r]) for r in range(R)]
+            torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
             for r in reversed(order):
                 st = ep.combine_memory_v2(
                     eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r], dtype, w.streams[r],
@@ -251,6 +254,7 @@ def test_reference_checker_blobs():
                     keep = (outs[r]["assist"][:, 2] == k).view(-1, 1)
                     rows = outs[r]["expand_x"].view(torch.int16)
                     eo.append(torch.where(keep, rows, torch.zeros_like(rows)).contiguous())
+                torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
                 for r in range(R):
                     assert ep.combine_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
                                          dtype, w.streams[r]) == 0
@@ -355,6 +359,7 @@ def test_mvp_dispatch_with_shared_experts(shape):
             outs = [alloc_shared_outputs(R, bs, h, K, S, case.local_experts, quant, False, r, SR) for r in range(R)]
             dev_ids = [to_dev(ids[r]) for r in range(R)]
             dev_mask = [to_dev(mask[r]) if use_mask else None for r in range(R)]
+            torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
             for r in rng.permutation(R):
                 o = outs[r]
                 st = ep.dispatch_v2(xt[r], dev_ids[r], w.comms[r], bs, h, K, E, o["expand_x"], o["assist"],
@@ -381,6 +386,7 @@ def test_mvp_dispatch_with_shared_experts(shape):
                 assert ep.combine_v2(eo[0], outs[0]["assist"], outs[0]["counts"], w.comms[0], bs, h, K, E, ys[0],
                                      ep.DT_FP16, w.streams[0]) == ep.ERR_PARA_CHECK_FAIL
                 continue
+            torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
             for r in range(R):
                 assert ep.combine_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
                                      ep.DT_FP16, w.streams[r]) == 0
@@ -413,6 +419,7 @@ def test_memory_dispatch_and_combine_with_shared_experts(shape, dtype):
             dev_ids = [to_dev(ids[r]) for r in range(R)]
             dev_mask = [None if mask is None else to_dev(mask[r]) for r in range(R)]
             order = list(rng.permutation(R))
+            torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
             for r in order:
                 o = outs[r]
                 st = ep.dispatch_memory_v2(xt[r], dev_ids[r], w.comms[r], bs, h, K, E, o["expand_x"], o["assist"],
@@ -435,6 +442,7 @@ def test_memory_dispatch_and_combine_with_shared_experts(shape, dtype):
             ys = [torch.full((bs, h), 7.0, dtype=tdt, device=DEV) for _ in range(R)]
             eo = [(outs[r]["expand_x"].view(tdt) * (1.0 + 0.25 * r)).contiguous() for r in range(R)]
             dev_w = [to_dev(weights[r]) for r in range(R)]
+            torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
             for r in reversed(order):
                 st = ep.combine_memory_v2(eo[r], outs[r]["assist"], outs[r]["counts"], w.comms[r], bs, h, K, E, ys[r],
                                           dtype, w.streams[r], expert_scales=dev_w[r], shared_expert_x=shared_t[r],

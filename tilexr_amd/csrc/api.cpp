@@ -39,6 +39,31 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     const bool expertHist = !memoryRoute;
 
     std::lock_guard<std::mutex> lock(comm->mu);
+    if (memoryRoute && p.quantMode == TILEXR_EP_QUANT_NONE && p.xActiveMask == nullptr && p.tileFlagsOut == nullptr &&
+        p.metaReadyEvent == nullptr) {
+        // decode-sized calls: one launch instead of count + scatter
+        SmallDispatchLaunch small {};
+        small.x = p.x;
+        small.ids = p.expertIds;
+        small.bs = p.bs;
+        small.h = p.h;
+        small.topK = p.topK;
+        small.numExperts = experts;
+        small.capacity = p.expertCapacity;
+        small.srcRank = comm->rank;
+        small.expertIdBias = static_cast<int32_t>(p.sharedExpertNum);
+        small.out = p.expandXOut;
+        small.assist = p.assistInfoForCombineOut;
+        small.rowOf = p.rowIndexMapOut;
+        small.sendCountsOut = p.epRecvCountsOut;
+        small.expertTokenNumsOut = p.expertTokenNumsOut;
+        small.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
+        small.stream = stream;
+        if (SmallDispatchFits(small)) {
+            comm->lastKernel[kKernelScatter] = "ep_dispatch_small_kernel";
+            return Timed(comm, kKernelScatter, stream, "small dispatch", [&] { return LaunchSmallDispatch(small); });
+        }
+    }
     const CountScratchLayout plan = PlanCountScratch(n, numKeys, experts, expertHist);
     if (!comm->dispatchScratch.Reserve(static_cast<size_t>(plan.totalBytes), true)) {
         return TileXR::TILEXR_ERROR_INTERNAL;

@@ -164,6 +164,30 @@ struct ReduceLaunch {
     hipStream_t stream;
 };
 
+// Memory-route dispatch of a small batch (plain copies, one rank, no mask, no readiness flags) in a single launch:
+// every workgroup counts the whole id table itself instead of waiting for a counting kernel.
+constexpr int kSmallRoutes = 2048;
+struct SmallDispatchLaunch {
+    const void *x;
+    const int32_t *ids;
+    int64_t bs;
+    int64_t h;
+    int64_t topK;
+    int64_t numExperts;
+    int64_t capacity;
+    int32_t srcRank;
+    int32_t expertIdBias;
+    void *out;
+    int32_t *assist;
+    int32_t *rowOf;                  // optional
+    int32_t *sendCountsOut;
+    int64_t *expertTokenNumsOut;
+    int tokenNumsType;
+    hipStream_t stream;
+};
+bool SmallDispatchFits(const SmallDispatchLaunch &l);
+hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l);
+
 hipError_t LaunchRouteCount(const RouteCountLaunch &l);
 hipError_t LaunchRoutePlace(const RoutePlaceLaunch &l);
 hipError_t LaunchScatter(const ScatterLaunch &l);
