@@ -1,9 +1,10 @@
 """Drives libtilexr-ep through its C ABI with torch tensors as device memory, and fetches results as numpy arrays
 shaped like the oracle's outputs (tests/ and the smoke check use it).
 
-Stream discipline of the tests: torch's own work (fills, host copies, comparisons) stays on torch's default stream
-and is waited for (`torch.cuda.synchronize()`) before a library call is issued on a session's own stream; library
-results are read after that stream has been synchronised."""
+Stream discipline of the tests: inside a Session torch's own work (fills, host copies, comparisons) runs on the
+session's stream, the one the library calls use.  Multi-rank worlds and side streams use torch's default stream for
+that work and wait for it (`torch.cuda.synchronize()`) before a library call is issued on another stream.  Library
+results are read after the stream of the call has been synchronised."""
 import numpy as np
 import torch
 
@@ -40,8 +41,15 @@ class Session:
         torch.cuda.set_device(0)
         self.comm = ep.Comm(rank_size, rank)
         self.stream = torch.cuda.Stream()
+        # torch's own work (fills, host copies, comparisons) goes on the same stream as the library calls, as a
+        # caller that keeps a whole layer on one stream would have it
+        self._previous = torch.cuda.current_stream()
+        torch.cuda.synchronize()
+        torch.cuda.set_stream(self.stream)
 
     def close(self):
+        torch.cuda.synchronize()
+        torch.cuda.set_stream(self._previous)
         release_device_copies()
         self.comm.destroy()
 

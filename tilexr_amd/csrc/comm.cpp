@@ -84,7 +84,9 @@ bool DeviceBuffer::Reserve(size_t want, bool zero)
         (void)hipGetLastError();
         return false;
     }
-    if (zero && hipMemset(p, 0, rounded) != hipSuccess) {
+    // The fill runs on the null stream, which a caller's non-blocking stream does not wait for: the kernels that
+    // are about to use the buffer on that stream must not be able to overtake it.
+    if (zero && (hipMemset(p, 0, rounded) != hipSuccess || hipStreamSynchronize(nullptr) != hipSuccess)) {
         (void)hipFree(p);
         return false;
     }
