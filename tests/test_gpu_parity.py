@@ -341,3 +341,59 @@ def test_unsupported_requests_are_reported():
             ep.ERR_NOT_SUPPORT
         # nothing above consumed a magic or launched anything
         assert s.comm.next_magic() == 1
+
+
+# ---------------------------------------------------------------------------------------------
+# Degenerate and extreme routing tables (both dispatch paths: one launch for small batches, count + scatter above)
+# ---------------------------------------------------------------------------------------------
+def _edge_ids(kind, rng, bs, K, E):
+    if kind == "all_invalid":
+        return rng.choice([-1, -5, E, E + 9], size=(bs, K)).astype(np.int32)
+    if kind == "one_expert":
+        return np.full((bs, K), E - 1, np.int32)                       # every route, duplicates within a token too
+    if kind == "duplicates":
+        ids = rng.integers(0, E, size=(bs, K)).astype(np.int32)
+        ids[:, 1:] = ids[:, :1]                                         # a token names the same expert K times
+        return ids
+    if kind == "last_token_only":
+        ids = np.full((bs, K), -1, np.int32)
+        ids[-1] = rng.permutation(E)[:K]
+        return ids
+    raise ValueError(kind)
+
+
+@pytest.mark.parametrize("kind", ["all_invalid", "one_expert", "duplicates", "last_token_only"])
+@pytest.mark.parametrize("shape", [(1, 8, 1, 1), (3, 64, 64, 64), (200, 40, 8, 2048), (300, 1024, 8, 2048), (1500, 256, 2, 7)])
+def test_degenerate_routing_tables(kind, shape):
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape))
+    ids = _edge_ids(kind, rng, bs, K, E)
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+    w = rng.random((bs, K)).astype(np.float32)
+    with Session() as s:
+        for capacity in (0, 3):
+            out = alloc_dispatch_outputs(bs, h, K, E)
+            counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
+            st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                          out["token_nums"], counts, ep.DT_BF16, s.stream, expert_capacity=capacity,
+                                          row_index_map=out["row_map"])
+            assert st == 0
+            y = torch.full((bs, h), 9.0, dtype=torch.bfloat16, device=DEV)
+            assert ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16,
+                                        s.stream, expert_scales=to_dev(w), row_index_map=out["row_map"]) == 0
+            s.sync()
+            case = O.Case(1, bs, h, K, E, dtype=O.DT_BF16, capacity=capacity, token_nums_type=1)
+            want = O.mem_dispatch(case, 0, xb[None], ids[None])
+            got = fetch(out, "send_counts", counts)
+            check_dispatch(got, want)
+            assert np.array_equal(got["send_counts"], want["send_counts"])
+            # the row map is the inverse of the tuples, -1 where a route has no row
+            rm = np.full(bs * K, -1, np.int32)
+            n = want["rows"]
+            rm[want["assist"][:n, 1] * K + want["assist"][:n, 2]] = np.arange(n, dtype=np.int32)
+            assert np.array_equal(got["row_map"].reshape(-1), rm)
+            wy = O.mem_combine(O.Case(1, bs, h, K, E, dtype=O.DT_BF16), 0, want["expand_x"].view(np.uint16)[None],
+                               want["assist"][None], want["send_counts"][None], expert_scales=w)
+            assert np.array_equal(bits16(y), wy)
+            if kind == "all_invalid":
+                assert n == 0 and not bits16(y).any()

@@ -55,7 +55,8 @@ EpWorld *CreateWorld(int rankSize)
         world->device = device;
         void *area = nullptr;
         const size_t bytes = static_cast<size_t>(rankSize) * kFlagAreaBytesPerRank;
-        if (hipMalloc(&area, bytes) == hipSuccess && hipMemset(area, 0, bytes) == hipSuccess) {
+        if (hipMalloc(&area, bytes) == hipSuccess && hipMemset(area, 0, bytes) == hipSuccess &&
+            hipStreamSynchronize(nullptr) == hipSuccess) {
             world->flagArea = static_cast<uint8_t *>(area);
             world->deviceReady = true;
             int cus = 0;
