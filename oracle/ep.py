@@ -29,6 +29,7 @@ class _Case(C.Structure):
         ("capacity", C.c_int64),
         ("shared_expert_num", C.c_int64),
         ("shared_expert_rank_num", C.c_int64),
+        ("tp_world_size", C.c_int64),
     ]
 
 
@@ -47,22 +48,23 @@ class Case:
     capacity: int = 0
     shared_expert_num: int = 0
     shared_expert_rank_num: int = 0
+    tp_world_size: int = 0
 
     def c(self):
         return _Case(self.rank_size, self.bs, self.h, self.top_k, self.moe_expert_num, self.dtype,
                      self.quant_mode, self.out_dtype, self.token_nums_type, self.mask_type, self.capacity,
-                     self.shared_expert_num, self.shared_expert_rank_num)
+                     self.shared_expert_num, self.shared_expert_rank_num, self.tp_world_size)
 
     @property
     def local_experts(self):
-        return self.moe_expert_num // (self.rank_size - self.shared_expert_rank_num)
+        return self.moe_expert_num // (self.rank_size // max(self.tp_world_size, 1) - self.shared_expert_rank_num)
 
     def out_local_experts(self, rank):
         return 1 if rank < self.shared_expert_rank_num else self.local_experts
 
     @property
     def max_rows(self):
-        return self.rank_size * self.bs * (self.top_k + self.shared_expert_num)
+        return self.rank_size * self.bs * (self.top_k + self.shared_expert_num)     # tp lanes included
 
     @property
     def out_row_bytes(self):
@@ -115,7 +117,7 @@ def lib():
         _lib.orc_quant_row_fp8_block128.restype = None
         _lib.orc_quant_row_fp8_block128.argtypes = [C.c_void_p, C.c_int64, C.c_int32, C.c_void_p, C.c_void_p]
         _lib.orc_mvp_dispatch_rank.restype = C.c_int64
-        _lib.orc_mvp_dispatch_rank.argtypes = [C.POINTER(_Case), C.c_int32] + [C.c_void_p] * 9
+        _lib.orc_mvp_dispatch_rank.argtypes = [C.POINTER(_Case), C.c_int32] + [C.c_void_p] * 10
         _lib.orc_mem_dispatch_rank.restype = C.c_int64
         _lib.orc_mem_dispatch_rank.argtypes = [C.POINTER(_Case), C.c_int32] + [C.c_void_p] * 8
         _lib.orc_mvp_combine_rank.restype = None
@@ -200,8 +202,9 @@ def quant_row_fp8_block128(row_u16, dtype):
 
 
 # ---- dispatch ----
-def mvp_dispatch(case, dst_rank, x, ids, mask=None, static_scale=None):
-    """x [R, bs, h] u16, ids [R, bs, K] i32, mask [R, bs] u8 -> dict of this destination rank's outputs."""
+def mvp_dispatch(case, dst_rank, x, ids, mask=None, static_scale=None, count_fill=0):
+    """x [R, bs, h] u16, ids [R, bs, K] i32, mask [R, bs] u8 -> dict of this destination rank's outputs.
+    `count_fill` is what the count arrays hold before the call (entries the path does not write keep it)."""
     x = _c(x, np.uint16)
     ids = _c(ids, np.int32)
     mask = _c(mask, np.uint8)
@@ -210,13 +213,14 @@ def mvp_dispatch(case, dst_rank, x, ids, mask=None, static_scale=None):
     expand = np.zeros((rows, case.out_row_bytes), np.uint8)
     scales = np.zeros(rows, np.float32)
     assist = np.zeros((rows, 4), np.int32)
-    recv = np.zeros(case.rank_size, np.int32)
+    recv = np.full(case.rank_size, count_fill, np.int32)
+    tp_recv = np.full(case.rank_size, count_fill, np.int32)
     nums = np.zeros(case.local_experts, np.int64)
     cc = case.c()
     n = lib().orc_mvp_dispatch_rank(C.byref(cc), dst_rank, _p(x), _p(ids), _p(mask), _p(static_scale),
-                                    _p(expand), _p(scales), _p(assist), _p(recv), _p(nums))
+                                    _p(expand), _p(scales), _p(assist), _p(recv), _p(tp_recv), _p(nums))
     return dict(rows=int(n), expand_x=expand, dyn_scales=scales, assist=assist, recv_counts=recv,
-                expert_token_nums=nums)
+                tp_recv_counts=tp_recv, expert_token_nums=nums)
 
 
 def mem_dispatch(case, dst_rank, x, ids, mask=None):

@@ -323,10 +323,15 @@ void orc_quant_row_fp8_block128(const uint16_t *src, int64_t h, int32_t dtype, u
  * Dispatch
  * ---------------------------------------------------------------------------------------------- */
 
+static int64_t tp_size(const orc_case *c)
+{
+    return c->tp_world_size > 1 ? c->tp_world_size : 1;
+}
+
 /* src/ep/host/ep_layout.cpp:156,171; tests/ep/demo/tilexr_ep_dispatch_demo.cpp:622-630 */
 static int64_t local_expert_num(const orc_case *c)
 {
-    return c->moe_expert_num / (c->rank_size - c->shared_expert_rank_num);
+    return c->moe_expert_num / (c->rank_size / tp_size(c) - c->shared_expert_rank_num);
 }
 
 /* tests/ep/demo/tilexr_ep_dispatch_demo.cpp:632-635: a shared rank presents one local expert */
@@ -355,71 +360,114 @@ static int64_t out_row_bytes(const orc_case *c)
  *                  expertTokenNums incremented per drained row; optional prefix-sum finalize :67-80)
  *   checker model  tools/checker/src/oracle.cpp:447-484 (same order, unmasked)
  * Quantised payloads always decode the input as fp16 (tilexr_ep_dispatch_helpers.h:121,167). */
-int64_t orc_mvp_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_t *x, const int32_t *ids,
+/* Appends the rows source rank `src` sends to expert rank `er` (token-major, shared routes then routed ones) and
+ * returns how many there were. */
+static int32_t mvp_rows_from_source(const orc_case *c, int32_t src, int64_t er, const uint16_t *x, const int32_t *ids,
     const uint8_t *mask, const float *static_scale, uint8_t *expand_x, float *dyn_scales, int32_t *assist,
-    int32_t *recv_counts, int64_t *expert_token_nums)
+    int64_t *expert_token_nums, int64_t *out_io)
 {
     const int64_t local_e = local_expert_num(c);
     const int64_t row_bytes = out_row_bytes(c);
+    const uint16_t *xs = x + (int64_t)src * c->bs * c->h;
+    const int32_t *is = ids + (int64_t)src * c->bs * c->top_k;
+    const uint8_t *ms = mask ? mask + (int64_t)src * c->bs : NULL;
+    /* with tensor-parallel groups the placement rules run over expert ranks and the source is known by its
+     * expert rank there (tilexr_ep_dispatch_kernel.cpp:724, 774-776) */
+    const int32_t src_expert_rank = src / (int32_t)tp_size(c);
+    int64_t out = *out_io;
+    int32_t count = 0;
+    for (int64_t t = 0; t < c->bs; ++t) {
+        if (ms && ms[t] == 0) {
+            continue;
+        }
+        /* one pass over the token's S shared routes, then its top_k routed ones
+         * (src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:536-568) */
+        for (int64_t r = 0; r < c->shared_expert_num + c->top_k; ++r) {
+            const int shared = r < c->shared_expert_num;
+            const int64_t k = shared ? c->top_k + r : r - c->shared_expert_num;
+            int32_t e;
+            int64_t local;
+            if (shared) {
+                if (shared_dst_rank(c, src_expert_rank, r) != er) {
+                    continue;
+                }
+                e = (int32_t)r;
+                /* tilexr_ep_dispatch_helpers.h:99-101: a shared row counts at index expertId */
+                local = r;
+            } else {
+                const int32_t id = is[t * c->top_k + k];
+                if (id < 0 || (int64_t)id >= c->moe_expert_num) {
+                    continue;
+                }
+                if (c->shared_expert_rank_num + (int64_t)id / local_e != er) {
+                    continue;
+                }
+                e = (int32_t)(c->shared_expert_num + id);
+                local = (int64_t)id % local_e;
+            }
+            uint8_t *dst = expand_x + out * row_bytes;
+            const uint16_t *row = xs + t * c->h;
+            if (c->quant_mode == ORC_QUANT_STATIC_INT8) {
+                orc_quant_row_static_int8(row, c->h, static_scale[0], (int8_t *)dst);
+            } else if (c->quant_mode == ORC_QUANT_TOKEN_INT8) {
+                dyn_scales[out] = orc_quant_row_token_int8(row, c->h, ORC_DT_FP16, (int8_t *)dst);
+            } else {
+                memcpy(dst, row, (size_t)row_bytes);
+            }
+            assist[out * 4 + 0] = src;
+            assist[out * 4 + 1] = (int32_t)t;
+            assist[out * 4 + 2] = (int32_t)k;
+            assist[out * 4 + 3] = e;
+            if (local < local_e) {          /* tilexr_ep_combine_helpers.h:124-128 */
+                ++expert_token_nums[local];
+            }
+            ++count;
+            ++out;
+        }
+    }
+    *out_io = out;
+    return count;
+}
+
+int64_t orc_mvp_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_t *x, const int32_t *ids,
+    const uint8_t *mask, const float *static_scale, uint8_t *expand_x, float *dyn_scales, int32_t *assist,
+    int32_t *recv_counts, int32_t *tp_recv_counts, int64_t *expert_token_nums)
+{
+    const int64_t local_e = local_expert_num(c);
+    const int64_t tp = tp_size(c);
+    const int64_t expert_ranks = c->rank_size / tp;
+    const int64_t er = dst_rank / tp;
+    const int64_t lane = dst_rank % tp;
     int64_t out = 0;
     for (int64_t e = 0; e < local_e; ++e) {
         expert_token_nums[e] = 0;
     }
-    for (int32_t src = 0; src < c->rank_size; ++src) {
-        const uint16_t *xs = x + (int64_t)src * c->bs * c->h;
-        const int32_t *is = ids + (int64_t)src * c->bs * c->top_k;
-        const uint8_t *ms = mask ? mask + (int64_t)src * c->bs : NULL;
-        int32_t count = 0;
-        for (int64_t t = 0; t < c->bs; ++t) {
-            if (ms && ms[t] == 0) {
+    /* own lane: the sources of this rank's lane in expert-rank order (tilexr_ep_dispatch_kernel.cpp:809-817);
+     * both count arrays are indexed by the source's global rank here (tilexr_ep_combine_helpers.h:92-95) */
+    for (int64_t es = 0; es < expert_ranks; ++es) {
+        const int32_t src = (int32_t)(es * tp + lane);
+        const int32_t count = mvp_rows_from_source(c, src, er, x, ids, mask, static_scale, expand_x, dyn_scales,
+            assist, expert_token_nums, &out);
+        recv_counts[src] = count;
+        if (tp_recv_counts) {
+            tp_recv_counts[src] = count;
+        }
+    }
+    /* tensor-parallel publish: the rows the other lanes of the group received follow in lane order, and the
+     * first tp entries of tpRecvCounts become rows per lane (:818-827, 662-697) */
+    if (tp > 1 && tp_recv_counts) {
+        tp_recv_counts[lane] = (int32_t)out;
+        for (int64_t l = 0; l < tp; ++l) {
+            if (l == lane) {
                 continue;
             }
-            /* one pass over the token's S shared routes, then its top_k routed ones
-             * (src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:536-568) */
-            for (int64_t r = 0; r < c->shared_expert_num + c->top_k; ++r) {
-                const int shared = r < c->shared_expert_num;
-                const int64_t k = shared ? c->top_k + r : r - c->shared_expert_num;
-                int32_t e;
-                int64_t local;
-                if (shared) {
-                    if (shared_dst_rank(c, src, r) != dst_rank) {
-                        continue;
-                    }
-                    e = (int32_t)r;
-                    /* tilexr_ep_dispatch_helpers.h:99-101: a shared row counts at index expertId */
-                    local = r;
-                } else {
-                    const int32_t id = is[t * c->top_k + k];
-                    if (id < 0 || (int64_t)id >= c->moe_expert_num) {
-                        continue;
-                    }
-                    if (c->shared_expert_rank_num + (int64_t)id / local_e != dst_rank) {
-                        continue;
-                    }
-                    e = (int32_t)(c->shared_expert_num + id);
-                    local = (int64_t)id % local_e;
-                }
-                uint8_t *dst = expand_x + out * row_bytes;
-                const uint16_t *row = xs + t * c->h;
-                if (c->quant_mode == ORC_QUANT_STATIC_INT8) {
-                    orc_quant_row_static_int8(row, c->h, static_scale[0], (int8_t *)dst);
-                } else if (c->quant_mode == ORC_QUANT_TOKEN_INT8) {
-                    dyn_scales[out] = orc_quant_row_token_int8(row, c->h, ORC_DT_FP16, (int8_t *)dst);
-                } else {
-                    memcpy(dst, row, (size_t)row_bytes);
-                }
-                assist[out * 4 + 0] = src;
-                assist[out * 4 + 1] = (int32_t)t;
-                assist[out * 4 + 2] = (int32_t)k;
-                assist[out * 4 + 3] = e;
-                if (local < local_e) {          /* tilexr_ep_combine_helpers.h:124-128 */
-                    ++expert_token_nums[local];
-                }
-                ++count;
-                ++out;
+            int32_t lane_rows = 0;
+            for (int64_t es = 0; es < expert_ranks; ++es) {
+                lane_rows += mvp_rows_from_source(c, (int32_t)(es * tp + l), er, x, ids, mask, static_scale, expand_x,
+                    dyn_scales, assist, expert_token_nums, &out);
             }
+            tp_recv_counts[l] = lane_rows;
         }
-        recv_counts[src] = count;
     }
     if (c->token_nums_type == 0) {
         int64_t running = 0;

@@ -25,6 +25,7 @@
  *   memory combine (fp32 acc, RINT)               : numpy float32 sequential sum + torch cast
  *   shared experts (both routes)                  : the reference demo's golden route model restated as a
  *                                                   brute-force walk in the tests, closed-form row counts
+ *   tensor-parallel groups (MVP route)            : the demo's BuildExpectedTpRoutes restated in the tests
  */
 #ifndef TILEXR_EP_ORACLE_H
 #define TILEXR_EP_ORACLE_H
@@ -68,6 +69,8 @@ typedef struct {
     int64_t capacity;         /* ext: rows kept per expert per destination (0 = unlimited) */
     int64_t shared_expert_num;      /* S: every active token also goes to each of S shared experts */
     int64_t shared_expert_rank_num; /* ranks [0, SR) host the shared experts (SR % S == 0); E % (R - SR) == 0 */
+    int64_t tp_world_size;          /* MVP route: ranks form groups of this many lanes (0 or 1 = none); the
+                                       placement rules then run over the R / tp expert ranks */
 } orc_case;
 
 /* ---- scalar numerics ---- */
@@ -95,9 +98,13 @@ void orc_quant_row_fp8_block128(const uint16_t *src, int64_t h, int32_t dtype, u
  * src % (SR/S) + s * (SR/S)) before its top_k routed ones (expertId = S + id, destination SR + id / localE),
  * localE = E / (R - SR).  expert_token_nums has localE entries (MVP route) or, on the memory route, 1 entry on
  * a shared rank and localE on the others; send_counts likewise 1*R or localE*R entries. */
+/* With tensor-parallel groups (tp lanes per expert rank) a rank receives from the sources of its own lane, then
+ * appends what the other lanes of its group received, in lane order.  recv_counts[src] is written for own-lane
+ * sources only (other entries are left as they are); tp_recv_counts (may be NULL when tp <= 1) gets the same
+ * per-source entries and then rows per lane in its first tp entries. */
 int64_t orc_mvp_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_t *x, const int32_t *ids,
     const uint8_t *mask, const float *static_scale, uint8_t *expand_x, float *dyn_scales, int32_t *assist,
-    int32_t *recv_counts, int64_t *expert_token_nums);
+    int32_t *recv_counts, int32_t *tp_recv_counts, int64_t *expert_token_nums);
 
 int64_t orc_mem_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_t *x, const int32_t *ids,
     const uint8_t *mask, uint8_t *expand_x, uint8_t *dyn_scales, int32_t *assist, int32_t *send_counts,

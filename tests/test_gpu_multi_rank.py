@@ -476,3 +476,68 @@ def test_expert_mask_with_shared_experts_is_reported_as_unsupported():
                                    o["token_nums"], o["counts"], ep.DT_BF16, w.streams[0], active_mask=to_dev(mask),
                                    active_mask_type=ep.MASK_EXPERT, shared_expert_num=S, shared_expert_rank_num=SR)
         assert st == ep.ERR_NOT_SUPPORT
+
+
+# ---------------------------------------------------------------------------------------------
+# Tensor-parallel groups (MVP route): a rank receives from its own lane, then appends its group's other lanes
+# ---------------------------------------------------------------------------------------------
+TP_SHAPES = [  # R, bs, h, K, E, S, SR, tp
+    (4, 6, 16, 2, 4, 0, 0, 2), (8, 40, 256, 3, 8, 0, 0, 2), (8, 25, 64, 2, 6, 1, 1, 2), (8, 64, 1024, 4, 8, 0, 0, 4),
+    (6, 300, 512, 2, 6, 0, 0, 3)]
+
+
+@pytest.mark.parametrize("shape", TP_SHAPES)
+def test_mvp_dispatch_with_tensor_parallel_groups(shape):
+    R, bs, h, K, E, S, SR, tp = shape
+    rng = np.random.default_rng(sum(shape))
+    ids = rand_ids(rng, R, bs, K, E, invalid=0.1)
+    xt, xb = rand_x(rng, R, bs, h, ep.DT_FP16, scale=3.0)
+    mask = (rng.random((R, bs)) < 0.7).astype(np.uint8)
+    with World(R) as w:
+        for quant, use_mask, nums_type in ((ep.Q_NONE, False, 1), (ep.Q_TOKEN_INT8, True, 0)):
+            case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16, quant_mode=quant, token_nums_type=nums_type,
+                          shared_expert_num=S, shared_expert_rank_num=SR, tp_world_size=tp)
+            outs = [alloc_shared_outputs(R, bs, h, K, S, case.local_experts, quant, False, r, SR) for r in range(R)]
+            dev_ids = [to_dev(ids[r]) for r in range(R)]
+            dev_mask = [to_dev(mask[r]) if use_mask else None for r in range(R)]
+            torch.cuda.synchronize()      # fills ran on the default stream, the calls use the ranks' streams
+            for r in rng.permutation(R):
+                o = outs[r]
+                st = ep.dispatch_v2(xt[r], dev_ids[r], w.comms[r], bs, h, K, E, o["expand_x"], o["assist"],
+                                    o["token_nums"], o["counts"], ep.DT_FP16 if quant == ep.Q_NONE else ep.DT_INT8,
+                                    w.streams[r], active_mask=dev_mask[r], tp_world_size=tp, tp_rank_id=int(r % tp),
+                                    shared_expert_num=S, shared_expert_rank_num=SR, quant_mode=quant,
+                                    token_nums_type=nums_type, dynamic_scales=o["scales"],
+                                    tp_recv_counts=o["tp_counts"])
+                assert st == 0, f"rank {r}: status {st}"
+            w.sync()
+            for r in range(R):
+                want = O.mvp_dispatch(case, r, xb, ids, mask if use_mask else None, count_fill=-1)
+                check_rank(outs[r], want, "recv_counts")
+                assert np.array_equal(outs[r]["tp_counts"].cpu().numpy(), want["tp_recv_counts"])
+                if quant == ep.Q_TOKEN_INT8:
+                    n = want["rows"]
+                    assert np.array_equal(outs[r]["scales"].cpu().numpy()[:n, 0], want["dyn_scales"][:n])
+            if quant != ep.Q_NONE or E % R != 0:
+                continue
+            # combine returns each row once: from the rank whose own lane received it (the count entries of the
+            # other lanes are zero, as a caller that clears its outputs has them)
+            ys = [torch.full((bs, h), 7.0, dtype=torch.float16, device=DEV) for _ in range(R)]
+            eo = [(outs[r]["expand_x"].view(torch.float16) * (1.0 + 0.25 * r)).contiguous() for r in range(R)]
+            counts = [torch.clamp(outs[r]["counts"], min=0) for r in range(R)]
+            torch.cuda.synchronize()
+            for r in range(R):
+                assert ep.combine_v2(eo[r], outs[r]["assist"], counts[r], w.comms[r], bs, h, K, E, ys[r], ep.DT_FP16,
+                                     w.streams[r]) == 0
+            w.sync()
+            eo_np = np.stack([bits16(t) for t in eo])
+            assist_np = np.stack([o["assist"].cpu().numpy() for o in outs])
+            counts_np = np.stack([c.cpu().numpy() for c in counts])
+            plain = O.Case(R, bs, h, K, E, dtype=O.DT_FP16)
+            for r in range(R):
+                assert np.array_equal(bits16(ys[r]), O.mvp_combine(plain, r, eo_np, assist_np, counts_np)), f"rank {r}"
+            # and nothing is lost: every valid route of every active token comes back exactly once
+            for r in range(R):
+                valid = ((ids[r] >= 0) & (ids[r] < E)).sum(1)
+                got = bits16(ys[r]).view(np.float16).astype(np.float32)
+                assert np.all((np.abs(got).sum(1) > 0) == (valid > 0))

@@ -594,3 +594,84 @@ def test_shared_slots_enter_the_memory_combine_after_the_routed_ones(orc):
                 acc = acc + xf[t]
             want = torch.from_numpy(acc).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
             assert np.array_equal(y[t], want)
+
+
+# ---------------------------------------------------------------------------------------------
+# Tensor-parallel groups on the MVP route: the demo's BuildExpectedRoutes / BuildExpectedTpRoutes restated
+# (tests/ep/demo/tilexr_ep_dispatch_demo.cpp:687-743), counts per the kernel
+# (src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:809-827, tilexr_ep_combine_helpers.h:92-95)
+# ---------------------------------------------------------------------------------------------
+def demo_tp_own_routes(case, rank, ids, token_live):
+    R, S, SR, K, tp = case.rank_size, case.shared_expert_num, case.shared_expert_rank_num, case.top_k, case.tp_world_size
+    er_size = R // tp
+    le = case.moe_expert_num // (er_size - SR)
+    per = SR // S if S else 1
+    out = []
+    for src in range(R):
+        if src % tp != rank % tp:
+            continue
+        for t in range(case.bs):
+            if not token_live[src][t]:
+                continue
+            for s in range(S):
+                if (src // tp) % per + s * per == rank // tp:
+                    out.append((src, t, K + s, s))
+            for k in range(K):
+                e = int(ids[src, t, k])
+                if 0 <= e < case.moe_expert_num and SR + e // le == rank // tp:
+                    out.append((src, t, k, S + e))
+    return out
+
+
+TP_SHAPES = [  # R, bs, h, K, E, S, SR, tp
+    (4, 6, 8, 2, 4, 0, 0, 2), (8, 9, 8, 3, 8, 0, 0, 2), (8, 5, 8, 2, 6, 1, 1, 2), (8, 7, 8, 2, 8, 0, 0, 4),
+    (6, 4, 8, 2, 6, 0, 0, 3)]
+
+
+@pytest.mark.parametrize("shape", TP_SHAPES)
+@pytest.mark.parametrize("masked", [False, True])
+def test_tensor_parallel_groups_match_demo_golden(orc, shape, masked):
+    R, bs, h, K, E, S, SR, tp = shape
+    rng = np.random.default_rng(sum(shape) * 5 + masked)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16, shared_expert_num=S, shared_expert_rank_num=SR, tp_world_size=tp,
+                  token_nums_type=1)
+    ids = rand_ids(rng, R, bs, K, E, invalid_frac=0.1)
+    x = rand_x(rng, R, bs, h)
+    mask = (rng.random((R, bs)) < 0.7).astype(np.uint8) if masked else None
+    live = [[bool(mask[s][t]) for t in range(bs)] for s in range(R)] if masked else [[True] * bs] * R
+    le = case.local_experts
+    for rank in range(R):
+        got = orc.mvp_dispatch(case, rank, x, ids, mask, count_fill=-1)
+        own = demo_tp_own_routes(case, rank, ids, live)
+        group = (rank // tp) * tp
+        want = list(own)
+        for lane in range(tp):
+            if group + lane != rank:
+                want += demo_tp_own_routes(case, group + lane, ids, live)
+        assert got["rows"] == len(want)
+        assert got["assist"][:len(want)].tolist() == [list(r) for r in want]
+        for row, (src, t, _, _) in enumerate(want):
+            assert np.array_equal(got["expand_x"][row].view(np.uint16), x[src, t])
+        # recvCounts: own-lane sources only, the rest is left alone
+        recv = [-1] * R
+        for src in range(rank % tp, R, tp):
+            recv[src] = sum(1 for r in own if r[0] == src)
+        assert got["recv_counts"].tolist() == recv
+        # tpRecvCounts: the same per-source entries, then rows per lane in the first tp entries
+        tp_recv = list(recv)
+        for lane in range(tp):
+            tp_recv[lane] = len(own) if group + lane == rank else len(demo_tp_own_routes(case, group + lane, ids, live))
+        assert got["tp_recv_counts"].tolist() == tp_recv
+        counts = [0] * le
+        for r in want:
+            loc = r[3] if r[3] < S else (r[3] - S) % le
+            if loc < le:
+                counts[loc] += 1
+        assert got["expert_token_nums"].tolist() == counts
+    # every rank of a group ends up with the same multiset of rows
+    for g in range(0, R, tp):
+        sets = []
+        for lane in range(tp):
+            o = orc.mvp_dispatch(case, g + lane, x, ids, mask)
+            sets.append(sorted(map(tuple, o["assist"][:o["rows"]].tolist())))
+        assert all(s == sets[0] for s in sets)

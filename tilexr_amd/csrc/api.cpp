@@ -261,9 +261,6 @@ int DispatchMvp(const EpDispatchParams &p)
     if (ret != kOk) {
         return ret;
     }
-    if (p.tpWorldSize != 0 && p.tpWorldSize != 1) {
-        return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // tensor-parallel groups: not built
-    }
     int64_t magic = 0;
     ret = TileXRCommNextMagic(p.comm, &magic);
     if (ret != kOk) {

@@ -44,13 +44,14 @@ struct ExchangeShape {
     int64_t quantMode = 0;
     int64_t sharedNum = 0;       // shared experts every active token is also sent to
     int64_t sharedRanks = 0;     // ranks [0, sharedRanks) host them
+    int64_t tp = 1;              // MVP route: lanes per tensor-parallel group
     int dtype = 0;
     int outDtype = 0;
     bool memoryRoute = false;
     bool operator==(const ExchangeShape &o) const
     {
         return bs == o.bs && h == o.h && topK == o.topK && experts == o.experts && quantMode == o.quantMode &&
-            sharedNum == o.sharedNum && sharedRanks == o.sharedRanks && dtype == o.dtype && outDtype == o.outDtype &&
+            sharedNum == o.sharedNum && sharedRanks == o.sharedRanks && tp == o.tp && dtype == o.dtype && outDtype == o.outDtype &&
             memoryRoute == o.memoryRoute;
     }
 };

@@ -54,6 +54,7 @@ struct DrainPlanLaunch {
     int localExperts;        // keys per rank in the staging areas' key space
     int outLocalExperts;     // memory route: segments per source on this rank (1 on a shared-expert rank)
     int tokenNumsCount;      // entries of expertTokenNumsOut
+    int tp;                  // MVP route: lanes per tensor-parallel group (<= 1: none)
     bool memoryRoute;        // segments (localExpert, src) with inclusive-sum counts, else (src) with plain counts
     int32_t *planOffsets;    // [numSeg + 1] exclusive offsets (scratch of the destination rank)
     int32_t *countsOut;
@@ -69,6 +70,7 @@ struct DrainCopyLaunch {
     int dstRank;
     int localExperts;
     int outLocalExperts;
+    int tp;
     bool memoryRoute;
     const int32_t *planOffsets;
     int64_t maxRows;

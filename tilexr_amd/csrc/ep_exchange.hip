@@ -18,15 +18,28 @@
 namespace TileXREp {
 namespace {
 
-__device__ __forceinline__ void SegmentOf(int idx, int rankSize, int dstRank, int localExperts, bool memoryRoute, int *src,
-    int *key)
+// Segment idx of destination rank dstRank: which source's staging area it comes from and under which key.
+//   memory route             local expert major, source minor
+//   MVP route                one segment per source
+//   MVP route, tp lanes      the sources of the rank's own lane first (in expert-rank order), then those of the other
+//                            lanes of its group in lane order; the key is the expert rank
+//                            (reference: src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:809-827, 662-697)
+__device__ __forceinline__ void SegmentOf(int idx, int rankSize, int dstRank, int localExperts, bool memoryRoute, int tp,
+    int *src, int *key)
 {
     if (memoryRoute) {
         *src = idx % rankSize;
         *key = dstRank * localExperts + idx / rankSize;
-    } else {
+    } else if (tp <= 1) {
         *src = idx;
         *key = dstRank;
+    } else {
+        const int expertRanks = rankSize / tp;
+        const int myLane = dstRank % tp;
+        const int block = idx / expertRanks;
+        const int lane = block == 0 ? myLane : (block - 1 < myLane ? block - 1 : block);
+        *src = (idx % expertRanks) * tp + lane;
+        *key = dstRank / tp;
     }
 }
 
@@ -84,6 +97,7 @@ struct DrainPlanArgs {
     int localExperts;
     int outLocalExperts;
     int tokenNumsCount;
+    int tp;
     int memoryRoute;
     int32_t *planOffsets;
     int32_t *countsOut;
@@ -102,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void ep_drain_plan_kernel(DrainPlanArgs a
     const int numSeg = a.memoryRoute ? a.outLocalExperts * a.rankSize : a.rankSize;
     for (int idx = tid; idx < numSeg; idx += kThreads) {
         int src, key;
-        SegmentOf(idx, a.rankSize, a.dstRank, a.localExperts, a.memoryRoute != 0, &src, &key);
+        SegmentOf(idx, a.rankSize, a.dstRank, a.localExperts, a.memoryRoute != 0, a.tp, &src, &key);
         const int32_t *ko = a.stage.counts + static_cast<int64_t>(src) * a.stage.countsStride;
         const int c = ko[key + 1] - ko[key];
         s_cnt[idx] = c;
@@ -110,16 +124,37 @@ __global__ __launch_bounds__(kThreads) void ep_drain_plan_kernel(DrainPlanArgs a
     }
     __syncthreads();
     const int total = BlockExclusiveScan(s_off, numSeg, s_part);
+    const int expertRanks = a.tp > 1 ? a.rankSize / a.tp : a.rankSize;
     for (int idx = tid; idx < numSeg; idx += kThreads) {
         a.planOffsets[idx] = s_off[idx];
-        const int out = a.memoryRoute ? s_off[idx] + s_cnt[idx] : s_cnt[idx];
-        a.countsOut[idx] = out;
-        if (a.tpCountsOut != nullptr) {
-            a.tpCountsOut[idx] = out;
+        if (a.memoryRoute) {
+            a.countsOut[idx] = s_off[idx] + s_cnt[idx];
+        } else if (idx < expertRanks) {
+            // plain per-source counts, indexed by the source's rank; with tp lanes only the rank's own lane is
+            // counted here and the other entries are left alone (reference: tilexr_ep_combine_helpers.h:92-95)
+            int src, key;
+            SegmentOf(idx, a.rankSize, a.dstRank, a.localExperts, false, a.tp, &src, &key);
+            a.countsOut[src] = s_cnt[idx];
+            if (a.tpCountsOut != nullptr) {
+                a.tpCountsOut[src] = s_cnt[idx];
+            }
         }
     }
     if (tid == 0) {
         a.planOffsets[numSeg] = total;
+    }
+    if (a.tp > 1 && a.tpCountsOut != nullptr) {
+        // afterwards the first tp entries become rows per lane (reference: tilexr_ep_dispatch_kernel.cpp:818-827)
+        __syncthreads();
+        if (tid < a.tp) {
+            int rows = 0;
+            for (int es = 0; es < expertRanks; ++es) {
+                rows += s_cnt[tid * expertRanks + es];
+            }
+            const int myLane = a.dstRank % a.tp;
+            const int lane = tid == 0 ? myLane : (tid - 1 < myLane ? tid - 1 : tid);
+            a.tpCountsOut[lane] = rows;
+        }
     }
     // rows per local expert
     for (int le = tid; le < a.tokenNumsCount; le += kThreads) {
@@ -132,7 +167,7 @@ __global__ __launch_bounds__(kThreads) void ep_drain_plan_kernel(DrainPlanArgs a
             for (int s = 0; s < a.rankSize; ++s) {
                 const int32_t *et = a.stage.counts + static_cast<int64_t>(s) * a.stage.countsStride +
                     a.stage.expertTotalOffset;
-                n += et[a.dstRank * a.localExperts + le];
+                n += et[(a.tp > 1 ? a.dstRank / a.tp : a.dstRank) * a.localExperts + le];
             }
         }
         s_tok[le] = n;
@@ -175,6 +210,7 @@ struct DrainCopyArgs {
     int dstRank;
     int localExperts;
     int outLocalExperts;
+    int tp;
     int memoryRoute;
     const int32_t *planOffsets;
     int64_t rowBytes;
@@ -203,7 +239,7 @@ __global__ __launch_bounds__(kThreads) void ep_drain_copy_kernel(DrainCopyArgs a
         }
     }
     int src, key;
-    SegmentOf(lo, a.rankSize, a.dstRank, a.localExperts, a.memoryRoute != 0, &src, &key);
+    SegmentOf(lo, a.rankSize, a.dstRank, a.localExperts, a.memoryRoute != 0, a.tp, &src, &key);
     const int32_t *ko = a.stage.counts + static_cast<int64_t>(src) * a.stage.countsStride;
     const int64_t srcRow = ko[key] + (row - a.planOffsets[lo]);
     const char *rows = a.stage.rows + static_cast<int64_t>(src) * a.stage.rowsStride;
@@ -316,6 +352,7 @@ hipError_t LaunchDrainPlan(const DrainPlanLaunch &l)
     a.localExperts = l.localExperts;
     a.outLocalExperts = l.outLocalExperts;
     a.tokenNumsCount = l.tokenNumsCount;
+    a.tp = l.tp;
     a.memoryRoute = l.memoryRoute ? 1 : 0;
     a.planOffsets = l.planOffsets;
     a.countsOut = l.countsOut;
@@ -334,6 +371,7 @@ hipError_t LaunchDrainCopy(const DrainCopyLaunch &l)
     a.dstRank = l.dstRank;
     a.localExperts = l.localExperts;
     a.outLocalExperts = l.outLocalExperts;
+    a.tp = l.tp;
     a.memoryRoute = l.memoryRoute ? 1 : 0;
     a.planOffsets = l.planOffsets;
     a.rowBytes = l.rowBytes;

@@ -66,13 +66,16 @@ bool PlanStage(EpWorld *world, const ExchangeShape &shape, bool reserve, StagePl
     const int64_t R = world->rankSize;
     plan->perToken = shape.topK + shape.sharedNum;
     const int64_t n = shape.bs * plan->perToken;
-    plan->localExperts = shape.experts / (R - shape.sharedRanks);
+    // with tensor-parallel groups (MVP route) experts are placed on the R / tp expert ranks and a key names an
+    // expert rank; the lane a row travels on is the source's own (reference: tilexr_ep_dispatch_kernel.cpp:382-392)
+    const int64_t expertRanks = R / shape.tp;
+    plan->localExperts = shape.experts / (expertRanks - shape.sharedRanks);
     plan->keysPerRank = shape.memoryRoute ? plan->localExperts : std::max(plan->localExperts, shape.sharedNum);
-    plan->keySpace = R * plan->keysPerRank;
+    plan->keySpace = expertRanks * plan->keysPerRank;
     plan->rowBytes = shape.quantMode == TILEXR_EP_QUANT_NONE ? shape.h * 2 : shape.h;
     plan->scaleBytesPerRow = shape.quantMode == TILEXR_EP_QUANT_TOKEN_INT8 ? 4 :
         (shape.quantMode == TILEXR_EP_QUANT_MXFP8 ? MxScaleBytes(shape.h) : 0);
-    plan->numKeys = shape.memoryRoute ? plan->keySpace : R;
+    plan->numKeys = shape.memoryRoute ? plan->keySpace : expertRanks;
     plan->keyDiv = shape.memoryRoute ? 1 : plan->keysPerRank;
     plan->expertHist = !shape.memoryRoute;
     StageLayout &l = plan->layout;
@@ -120,6 +123,7 @@ int DrainRank(EpWorld *world, int q, const ExchangeShape &shape, const StagePlan
     dp.localExperts = localExperts;
     dp.outLocalExperts = outLocalExperts;
     dp.tokenNumsCount = shape.memoryRoute ? outLocalExperts : static_cast<int>(plan.localExperts);
+    dp.tp = static_cast<int>(shape.tp);
     dp.memoryRoute = shape.memoryRoute;
     dp.planOffsets = static_cast<int32_t *>(comm->drainScratch.ptr);
     dp.countsOut = p.epRecvCountsOut;
@@ -137,6 +141,7 @@ int DrainRank(EpWorld *world, int q, const ExchangeShape &shape, const StagePlan
     dc.dstRank = q;
     dc.localExperts = localExperts;
     dc.outLocalExperts = outLocalExperts;
+    dc.tp = static_cast<int>(shape.tp);
     dc.memoryRoute = shape.memoryRoute;
     dc.planOffsets = dp.planOffsets;
     dc.maxRows = static_cast<int64_t>(R) * shape.bs * plan.perToken;
@@ -166,7 +171,9 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     const int R = world->rankSize;
     const int r = comm->rank;
     const int64_t shared = p.sharedExpertNum;
-    const int64_t keySpaceBound = static_cast<int64_t>(R) * std::max(p.moeExpertNum / (R - p.sharedExpertRankNum), shared);
+    const int64_t tp = (!memoryRoute && p.tpWorldSize > 1) ? p.tpWorldSize : 1;
+    const int64_t keySpaceBound = static_cast<int64_t>(R / tp) *
+        std::max(p.moeExpertNum / (R / tp - p.sharedExpertRankNum), shared);
     if (!WithinKernelLimits(p.bs, p.h, p.topK + shared, std::max(p.moeExpertNum, keySpaceBound), R) || p.extended) {
         return TileXR::TILEXR_ERROR_NOT_SUPPORT;
     }
@@ -184,6 +191,7 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     shape.quantMode = p.quantMode;
     shape.sharedNum = shared;
     shape.sharedRanks = p.sharedExpertRankNum;
+    shape.tp = tp;
     shape.dtype = static_cast<int>(p.dtype);
     shape.outDtype = static_cast<int>(p.expandXOutDtype);
     shape.memoryRoute = memoryRoute;
@@ -242,7 +250,7 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
         aug.topK = p.topK;
         aug.moeExpertNum = p.moeExpertNum;
         aug.rankSize = R;
-        aug.srcRank = r;
+        aug.srcRank = static_cast<int>(r / tp);      // the placement rules see the source's expert rank
         aug.sharedNum = static_cast<int>(shared);
         aug.sharedRanks = static_cast<int>(p.sharedExpertRankNum);
         aug.localExperts = static_cast<int>(plan.localExperts);
