@@ -155,8 +155,7 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     scatter.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
     scatter.totalRowsPtr = scratch.keyOffset + numKeys;
     if (p.tileFlagsOut != nullptr) {
-        const int64_t tiles = (n + p.tileRows - 1) / p.tileRows;
-        if (!comm->tileCounters.Reserve(static_cast<size_t>(tiles) * sizeof(uint32_t), true)) {
+        if (!comm->tileCounters.Reserve(static_cast<size_t>(TileCounterWords(n, p.tileRows)) * sizeof(uint32_t), true)) {
             return TileXR::TILEXR_ERROR_INTERNAL;
         }
         scatter.tileCounters = static_cast<uint32_t *>(comm->tileCounters.ptr);

@@ -104,7 +104,7 @@ struct ScatterLaunch {
     // word that atomics are hitting holds those atomics up (measured: 20 000 polls slow the scatter from 95 to
     // 215 us), a poll of a word that is stored once costs the producer nothing.
     uint64_t *tileFlags;
-    uint32_t *tileCounters;      // [ceil(rows / tileRows)]
+    uint32_t *tileCounters;      // TileCounterWords(bs * topK, tileRows) words
     int64_t tileRows;
     uint64_t epoch;
     const int32_t *totalRowsPtr; // device word: rows kept by this dispatch (size of the last tile)
@@ -186,6 +186,15 @@ struct SmallDispatchLaunch {
     hipStream_t stream;
 };
 bool SmallDispatchFits(const SmallDispatchLaunch &l);
+
+// Readiness tiles wider than this many rows are counted in two levels (see PublishRow in ep_scatter.hip).
+constexpr int kTileSubRows = 16;
+inline int64_t TileCounterWords(int64_t maxRows, int64_t tileRows)
+{
+    const int64_t tiles = (maxRows + tileRows - 1) / tileRows;
+    const int64_t groupsPerTile = tileRows > kTileSubRows ? (tileRows + kTileSubRows - 1) / kTileSubRows : 0;
+    return tiles * (1 + groupsPerTile);
+}
 hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l);
 
 hipError_t LaunchRouteCount(const RouteCountLaunch &l);

@@ -35,6 +35,7 @@ struct ScatterArgs {
     void *scalesOut;
     uint64_t *tileFlags;
     uint32_t *tileCounters;
+    int maxTiles;                // tiles of the largest possible row count: the group counters start there
     int tileRows;
     uint64_t epoch;
     const int32_t *totalRowsPtr;
@@ -101,19 +102,43 @@ __device__ __forceinline__ void ScalarStore(T *p, T v)
 // at zero for the next dispatch).  The caller has made the row complete in memory first, so has every earlier counter
 // of the tile, and the atomics on one counter are totally ordered: when the last one returns, all rows of the tile are
 // in memory.  The words consumers poll are only ever stored to, never hit by atomics.
-// `parts` callers publish each row (the slices a row is cut into).
+// `parts` callers publish each row (the slices a row is cut into).  Atomics on one address complete at about three per
+// microsecond on this part, so a tile wider than kTileSubRows rows is counted in two levels: groups of kTileSubRows
+// rows first (their counters follow the per-tile ones in `tileCounters`), completed groups second.
+__device__ __forceinline__ bool CountLanded(uint32_t *counter, int target)
+{
+    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (static_cast<int>(before) + 1 != target) {
+        return false;
+    }
+    __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return true;
+}
+
 __device__ __forceinline__ void PublishRow(const ScatterArgs &a, int row, int parts)
 {
     const int tile = row / a.tileRows;
     int rowsInTile = 1;
     if (a.tileRows > 1 || parts > 1) {
-        const int left = *a.totalRowsPtr - tile * a.tileRows;
+        const int total = *a.totalRowsPtr;
+        const int left = total - tile * a.tileRows;
         rowsInTile = left < a.tileRows ? left : a.tileRows;
-        const uint32_t before = __hip_atomic_fetch_add(&a.tileCounters[tile], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (static_cast<int>(before) + 1 != rowsInTile * parts) {
-            return;
+        if (a.tileRows <= kTileSubRows) {
+            if (!CountLanded(&a.tileCounters[tile], rowsInTile * parts)) {
+                return;
+            }
+        } else {
+            const int groupsPerTile = (a.tileRows + kTileSubRows - 1) / kTileSubRows;
+            const int group = (row - tile * a.tileRows) / kTileSubRows;
+            const int leftInTile = rowsInTile - group * kTileSubRows;
+            const int rowsInGroup = leftInTile < kTileSubRows ? leftInTile : kTileSubRows;
+            if (!CountLanded(&a.tileCounters[a.maxTiles + tile * groupsPerTile + group], rowsInGroup * parts)) {
+                return;
+            }
+            if (!CountLanded(&a.tileCounters[tile], (rowsInTile + kTileSubRows - 1) / kTileSubRows)) {
+                return;
+            }
         }
-        __hip_atomic_store(&a.tileCounters[tile], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __hip_atomic_store(&a.tileFlags[tile], (a.epoch << 32) | static_cast<uint32_t>(rowsInTile), __ATOMIC_RELAXED,
         __HIP_MEMORY_SCOPE_AGENT);
@@ -535,6 +560,7 @@ hipError_t LaunchScatter(const ScatterLaunch &l)
     a.tileFlags = l.tileFlags;
     a.tileCounters = l.tileCounters;
     a.tileRows = static_cast<int>(l.tileRows);
+    a.maxTiles = l.tileRows > 0 ? static_cast<int>((l.bs * l.topK + l.tileRows - 1) / l.tileRows) : 0;
     a.epoch = l.epoch;
     a.totalRowsPtr = l.totalRowsPtr;
     a.colSlices = static_cast<int>((l.h / 8 + kRouteVecs * kThreads - 1) / (kRouteVecs * kThreads));
