@@ -356,3 +356,27 @@ def test_comm_shim_rules():
     assert lib.TileXRGetCommArgsHost(C.c_void_p(0x1234), C.byref(host)) == ep.ERR_NOT_INITIALIZED
     for comm in (a, b, c):
         comm.destroy()
+
+
+# ---------------------------------------------------------------------------------------------
+# a C++ caller built against include/ only, as the reference's demo is built against its installed headers
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.skipif(torch.cuda.is_available(), reason="fabricated pointers must never reach a real device")
+def test_cxx_caller_links_against_the_headers_and_the_library(tmp_path):
+    import os
+    import shutil
+    import subprocess
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    gxx = shutil.which("g++")
+    if gxx is None:
+        pytest.skip("no host C++ compiler")
+    exe = str(tmp_path / "caller")
+    lib_dir = os.path.join(root, "tilexr_amd", "lib")
+    # C++14 like the reference's host code; no HIP or torch header is on the include path
+    subprocess.run([gxx, "-std=c++14", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(root, "include"),
+                    os.path.join(root, "tests", "cxx", "caller.cpp"), "-o", exe, "-L", lib_dir, "-ltilexr-ep",
+                    f"-Wl,-rpath,{lib_dir}", "-Wl,-rpath-link,/opt/rocm/lib"], check=True)
+    run = subprocess.run([exe], capture_output=True, text=True)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "caller ok" in run.stdout
