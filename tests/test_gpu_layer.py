@@ -1,0 +1,95 @@
+"""The torch-facing layer (tilexr_amd/layer.py) against a plain PyTorch fp32 reference of the same two ops, on torch's
+default stream like ordinary torch code.
+
+Reference dispatch: stable sort of the valid routes by expert; reference combine: fp32 sum over k of w * row.
+Layout, indices and counts must be identical; the combined rows are bit-identical to the k-ordered fp32 loop and
+within 1e-2 relative of torch's own reduction order (the tolerance the workload definition states for the combine).
+"""
+import numpy as np
+import pytest
+import torch
+
+from tilexr_amd import layer, workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def torch_dispatch(x, ids, experts):
+    bs, K = ids.shape
+    flat = torch.arange(bs * K, device=x.device)
+    e = ids.reshape(-1).long()
+    valid = (e >= 0) & (e < experts)
+    key = torch.where(valid, e * (bs * K) + flat, torch.full_like(flat, experts * bs * K))
+    order = torch.argsort(key, stable=True)[: int(valid.sum().item())]
+    rows = x[order // K]
+    assist = torch.stack([torch.zeros_like(order), order // K, order % K, e[order]], 1).int()
+    counts = torch.bincount(e[valid], minlength=experts)
+    row_map = torch.full((bs * K,), -1, dtype=torch.int32, device=x.device)
+    row_map[order] = torch.arange(order.numel(), device=x.device, dtype=torch.int32)
+    return rows, assist, counts, row_map.view(bs, K)
+
+
+def torch_combine_k_ordered(expert_out, row_map, weights):
+    bs, K = row_map.shape
+    acc = torch.zeros((bs, expert_out.shape[1]), dtype=torch.float32, device=expert_out.device)
+    for k in range(K):
+        r = row_map[:, k].long()
+        row = expert_out[r.clamp(min=0)].float() * weights[:, k:k + 1]
+        acc = acc + torch.where((r >= 0)[:, None], row, torch.zeros_like(row))
+    return acc
+
+
+@pytest.mark.parametrize("name,bs", [("C2", 128), ("C3", 1536), ("C3", 4096)])
+def test_layer_matches_torch_reference(name, bs):
+    w = workloads.scaled(workloads.CONFIGS[name], bs)
+    x = workloads.make_x(w).to(DEV)
+    ids, weights = workloads.make_routing(w)
+    ids[::7, 0] = -1                                      # some invalid routes
+    ids, weights = ids.to(DEV), weights.to(DEV)
+    with layer.MoeEpLayer(w.experts, w.top_k, w.h) as moe:
+        d = moe.dispatch(x, ids)
+        want_rows, want_assist, want_counts, want_map = torch_dispatch(x, ids, w.experts)
+        n = d.rows()
+        assert n == want_rows.shape[0]
+        assert torch.equal(d.expand_x[:n].view(torch.int16), want_rows.view(torch.int16))
+        assert torch.equal(d.assist[:n], want_assist)
+        assert torch.equal(d.token_nums, want_counts)
+        assert torch.equal(d.send_counts.long(), torch.cumsum(want_counts, 0))
+        assert torch.equal(d.row_map, want_map)
+        # an "expert stage" written in torch on the current stream, then combine
+        expert_out = (d.expand_x.float() * 0.5 + 1.0).to(torch.bfloat16)
+        y = moe.combine(expert_out, d, weights)
+        ref = torch_combine_k_ordered(expert_out, d.row_map, weights)
+        assert torch.equal(y.view(torch.int16), ref.to(torch.bfloat16).view(torch.int16))
+        # torch's own reduction order: within 1e-2 relative
+        gathered = expert_out[d.row_map.long().clamp(min=0)].float() * (d.row_map >= 0)[..., None]
+        other = (gathered * weights[..., None]).sum(1)
+        err = (y.float() - other).abs()
+        assert torch.all(err <= 1e-2 * other.abs() + 1e-2 * other.abs().mean())
+
+
+@pytest.mark.parametrize("quant", ["int8", "fp8_block128"])
+def test_layer_quantised_round_trip(quant):
+    w = workloads.scaled(workloads.CONFIGS["C4" if quant == "int8" else "C5"], 512)
+    x = workloads.make_x(w).to(DEV)
+    ids, weights = workloads.make_routing(w)
+    ids, weights = ids.to(DEV), weights.to(DEV)
+    with layer.MoeEpLayer(w.experts, w.top_k, w.h) as moe:
+        d = moe.dispatch(x, ids, quant=quant, capacity=w.capacity)
+        n = d.rows()
+        if quant == "int8":
+            deq = d.expand_x[:n].view(torch.int8).float() * d.scales[:n]
+        else:
+            deq = (d.expand_x[:n].view(torch.float8_e4m3fn).float().view(n, w.h // 128, 128) *
+                   d.scales[:n, :, None]).view(n, w.h)
+        src = x.float()[d.assist[:n, 1].long()]
+        bound = d.scales[:n] * 0.5001 if quant == "int8" else torch.maximum(
+            src.abs() * 2.0 ** -4, d.scales[:n].repeat_interleave(128, dim=1) * 2.0 ** -10) * 1.0001
+        assert torch.all((deq - src).abs() <= bound)
+        # identity expert on the quantised payload: combine dequantises, rounds to bf16 and reduces
+        y = moe.combine(d.expand_x, d, weights, expert_out_scales=d.scales, expert_out_quant=quant)
+        padded = torch.zeros((w.bs * w.top_k, w.h), dtype=torch.bfloat16, device=DEV)
+        padded[:n] = deq.to(torch.bfloat16)
+        ref = torch_combine_k_ordered(padded, d.row_map, weights)
+        assert torch.equal(y.view(torch.int16), ref.to(torch.bfloat16).view(torch.int16))
