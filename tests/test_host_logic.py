@@ -380,3 +380,30 @@ def test_cxx_caller_links_against_the_headers_and_the_library(tmp_path):
     run = subprocess.run([exe], capture_output=True, text=True)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "caller ok" in run.stdout
+
+
+# ---------------------------------------------------------------------------------------------
+# readiness-tile bookkeeping: the scatter kernels' counting code, run on CPU threads with random landing orders
+# ---------------------------------------------------------------------------------------------
+def _publish_stress(*args):
+    fn = ep.lib().TileXREpHookTilePublishStress
+    fn.argtypes = [C.c_int] * 6 + [C.c_uint32, C.c_int]
+    return fn(*args)
+
+
+@pytest.mark.parametrize("rows,max_rows,tile_rows,parts", [
+    (1000, 1024, 1, 1), (1000, 1024, 1, 2), (1000, 1024, 7, 1), (1000, 1024, 16, 2), (1000, 1024, 17, 2),
+    (1000, 1024, 100, 2), (4096, 4096, 256, 2), (4095, 5000, 1024, 3), (0, 64, 8, 1), (5, 64, 64, 2), (33, 33, 32, 1)])
+def test_tile_publication_holds_under_random_landing_orders(rows, max_rows, tile_rows, parts):
+    # invariants checked inside the hook: a readiness word is stored once per dispatch and only after every part of
+    # every row of its tile has landed; afterwards every word is (epoch << 32) | rows in the tile and every counter is
+    # zero again, over several dispatches on the same scratch
+    for seed in (1, 2, 3):
+        assert _publish_stress(rows, max_rows, tile_rows, parts, 8, 6, seed, 0) == 0
+
+
+def test_tile_publication_checks_catch_planted_mistakes():
+    # a part reported before it has landed: some tile is published too early (one-row tiles make every report a store)
+    assert _publish_stress(4096, 4096, 1, 1, 8, 4, 7, 1) == -1
+    # a part reported twice: the tile's counter overshoots, so the tile is published early, twice or never
+    assert _publish_stress(4096, 4096, 64, 2, 8, 4, 7, 2) in (-1, -2, -3, -4)

@@ -19,6 +19,8 @@
 
 #include <hip/hip_runtime_api.h>
 
+#include "ep_tile_publish.h"
+
 namespace TileXREp {
 
 constexpr int kMinChunkShift = 10;      // a counting workgroup handles 2^shift routes: 1024 ...
@@ -186,15 +188,6 @@ struct SmallDispatchLaunch {
     hipStream_t stream;
 };
 bool SmallDispatchFits(const SmallDispatchLaunch &l);
-
-// Readiness tiles wider than this many rows are counted in two levels (see PublishRow in ep_scatter.hip).
-constexpr int kTileSubRows = 16;
-inline int64_t TileCounterWords(int64_t maxRows, int64_t tileRows)
-{
-    const int64_t tiles = (maxRows + tileRows - 1) / tileRows;
-    const int64_t groupsPerTile = tileRows > kTileSubRows ? (tileRows + kTileSubRows - 1) / kTileSubRows : 0;
-    return tiles * (1 + groupsPerTile);
-}
 hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l);
 
 hipError_t LaunchRouteCount(const RouteCountLaunch &l);

@@ -18,6 +18,7 @@
 #include "ep_launch.h"
 #include "ep_numerics.cuh"
 #include "ep_place.cuh"
+#include "ep_tile_publish.h"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -98,50 +99,35 @@ __device__ __forceinline__ void ScalarStore(T *p, T v)
     }
 }
 
-// Counts one landed row; whoever lands the last row of a tile stores the tile's readiness word (and leaves the counter
-// at zero for the next dispatch).  The caller has made the row complete in memory first, so has every earlier counter
-// of the tile, and the atomics on one counter are totally ordered: when the last one returns, all rows of the tile are
-// in memory.  The words consumers poll are only ever stored to, never hit by atomics.
-// `parts` callers publish each row (the slices a row is cut into).  Atomics on one address complete at about three per
-// microsecond on this part, so a tile wider than kTileSubRows rows is counted in two levels: groups of kTileSubRows
-// rows first (their counters follow the per-tile ones in `tileCounters`), completed groups second.
-__device__ __forceinline__ bool CountLanded(uint32_t *counter, int target)
-{
-    const uint32_t before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (static_cast<int>(before) + 1 != target) {
-        return false;
+// Device side of ep_tile_publish.h: relaxed agent-scope atomics.  The caller has made the row complete in memory
+// first, so has every earlier counter of the tile, and the atomics on one counter are totally ordered: when the last
+// one returns, all rows of the tile are in memory.
+struct DeviceTileOps {
+    __device__ __forceinline__ uint32_t FetchAdd(uint32_t *p)
+    {
+        return __hip_atomic_fetch_add(p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    return true;
-}
+    __device__ __forceinline__ void Store(uint32_t *p, uint32_t v)
+    {
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ void Store(uint64_t *p, uint64_t v)
+    {
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
 
 __device__ __forceinline__ void PublishRow(const ScatterArgs &a, int row, int parts)
 {
-    const int tile = row / a.tileRows;
-    int rowsInTile = 1;
-    if (a.tileRows > 1 || parts > 1) {
-        const int total = *a.totalRowsPtr;
-        const int left = total - tile * a.tileRows;
-        rowsInTile = left < a.tileRows ? left : a.tileRows;
-        if (a.tileRows <= kTileSubRows) {
-            if (!CountLanded(&a.tileCounters[tile], rowsInTile * parts)) {
-                return;
-            }
-        } else {
-            const int groupsPerTile = (a.tileRows + kTileSubRows - 1) / kTileSubRows;
-            const int group = (row - tile * a.tileRows) / kTileSubRows;
-            const int leftInTile = rowsInTile - group * kTileSubRows;
-            const int rowsInGroup = leftInTile < kTileSubRows ? leftInTile : kTileSubRows;
-            if (!CountLanded(&a.tileCounters[a.maxTiles + tile * groupsPerTile + group], rowsInGroup * parts)) {
-                return;
-            }
-            if (!CountLanded(&a.tileCounters[tile], (rowsInTile + kTileSubRows - 1) / kTileSubRows)) {
-                return;
-            }
-        }
-    }
-    __hip_atomic_store(&a.tileFlags[tile], (a.epoch << 32) | static_cast<uint32_t>(rowsInTile), __ATOMIC_RELAXED,
-        __HIP_MEMORY_SCOPE_AGENT);
+    TilePublishArgs t;
+    t.flags = a.tileFlags;
+    t.counters = a.tileCounters;
+    t.tileRows = a.tileRows;
+    t.maxTiles = a.maxTiles;
+    t.totalRows = (a.tileRows > 1 || parts > 1) ? *a.totalRowsPtr : 0;
+    t.epoch = a.epoch;
+    DeviceTileOps ops;
+    PublishLanded(ops, t, row, parts);
 }
 
 // Publishes the rows of one token.  Each wave waits for its own stores and the barrier collects the waves.

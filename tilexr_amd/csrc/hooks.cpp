@@ -5,6 +5,14 @@
 #include "ep_host.h"
 #include "hooks.h"
 
+#include <algorithm>
+#include <atomic>
+#include <random>
+#include <thread>
+#include <vector>
+
+#include "ep_tile_publish.h"
+
 using namespace TileXREp;
 
 namespace {
@@ -246,6 +254,110 @@ int64_t TileXREpHookUdmaOperationBytes(int64_t totalBytes, int64_t rankSize, int
 int64_t TileXREpHookUdmaWorkspaceBytes(int64_t totalBytes, int64_t rankSize, int64_t slotBytes)
 {
     return TileXREpUdmaRequiredWorkspaceBytes(totalBytes, rankSize, slotBytes);
+}
+
+int TileXREpHookTilePublishStress(int totalRows, int maxRows, int tileRows, int parts, int threads, int rounds,
+    uint32_t seed, int fault)
+{
+    if (totalRows < 0 || maxRows < totalRows || tileRows <= 0 || parts <= 0 || threads <= 0 || rounds <= 0) {
+        return -100;
+    }
+    const int maxTiles = (maxRows + tileRows - 1) / tileRows;
+    const int tiles = (totalRows + tileRows - 1) / tileRows;
+    std::vector<uint32_t> counters(static_cast<size_t>(TileXREp::TileCounterWords(maxRows, tileRows)), 0u);
+    std::vector<uint64_t> flags(static_cast<size_t>(maxTiles > 0 ? maxTiles : 1), 0ull);
+    std::vector<std::atomic<int>> landed(static_cast<size_t>(totalRows > 0 ? totalRows : 1));
+    std::vector<std::atomic<int>> stores(static_cast<size_t>(maxTiles > 0 ? maxTiles : 1));
+    std::atomic<int> violation {0};
+
+    // host flavour of the three memory operations; a store of a readiness word checks the protocol's promise
+    struct HostOps {
+        TileXREp::TilePublishArgs *args;
+        std::vector<uint64_t> *flags;
+        std::vector<std::atomic<int>> *landed;
+        std::vector<std::atomic<int>> *stores;
+        std::atomic<int> *violation;
+        int parts;
+        uint32_t FetchAdd(uint32_t *p) { return __atomic_fetch_add(p, 1u, __ATOMIC_ACQ_REL); }
+        void Store(uint32_t *p, uint32_t v) { __atomic_store_n(p, v, __ATOMIC_RELEASE); }
+        void Store(uint64_t *p, uint64_t v)
+        {
+            const int tile = static_cast<int>(p - flags->data());
+            const int begin = tile * args->tileRows;
+            const int end = begin + args->tileRows < args->totalRows ? begin + args->tileRows : args->totalRows;
+            for (int r = begin; r < end; ++r) {
+                if ((*landed)[static_cast<size_t>(r)].load(std::memory_order_acquire) != parts) {
+                    violation->store(-1);      // published before every part of every row had landed
+                }
+            }
+            if ((*stores)[static_cast<size_t>(tile)].fetch_add(1) != 0) {
+                violation->store(-2);          // published twice in one dispatch
+            }
+            __atomic_store_n(p, v, __ATOMIC_RELEASE);
+        }
+    };
+
+    std::mt19937 rng(seed);
+    for (int round = 0; round < rounds; ++round) {
+        TileXREp::TilePublishArgs args {};
+        args.flags = flags.data();
+        args.counters = counters.data();
+        args.tileRows = tileRows;
+        args.maxTiles = maxTiles;
+        args.totalRows = totalRows;
+        args.epoch = static_cast<uint64_t>(round + 1);
+        for (auto &l : landed) {
+            l.store(0);
+        }
+        for (auto &st : stores) {
+            st.store(0);
+        }
+        // every (row, part) event once, shuffled, dealt to the threads round-robin
+        std::vector<int> events(static_cast<size_t>(totalRows) * parts);
+        for (size_t i = 0; i < events.size(); ++i) {
+            events[i] = static_cast<int>(i);
+        }
+        std::shuffle(events.begin(), events.end(), rng);
+        std::vector<std::thread> pool;
+        for (int t = 0; t < threads; ++t) {
+            pool.emplace_back([&, t] {
+                HostOps ops {&args, &flags, &landed, &stores, &violation, parts};
+                for (size_t i = static_cast<size_t>(t); i < events.size(); i += static_cast<size_t>(threads)) {
+                    const int row = events[i] / parts;
+                    if (fault == 1) {
+                        TileXREp::PublishLanded(ops, args, row, parts);
+                        std::this_thread::yield();
+                        landed[static_cast<size_t>(row)].fetch_add(1, std::memory_order_release);
+                        continue;
+                    }
+                    landed[static_cast<size_t>(row)].fetch_add(1, std::memory_order_release);   // "the part is in memory"
+                    TileXREp::PublishLanded(ops, args, row, parts);
+                    if (fault == 2 && i == static_cast<size_t>(t)) {
+                        TileXREp::PublishLanded(ops, args, row, parts);
+                    }
+                }
+            });
+        }
+        for (auto &th : pool) {
+            th.join();
+        }
+        if (violation.load() != 0) {
+            return violation.load();
+        }
+        for (int tile = 0; tile < tiles; ++tile) {
+            const int left = totalRows - tile * tileRows;
+            const uint64_t want = (args.epoch << 32) | static_cast<uint32_t>(left < tileRows ? left : tileRows);
+            if (flags[static_cast<size_t>(tile)] != want) {
+                return -3;                     // a tile was never published, or with the wrong word
+            }
+        }
+        for (uint32_t c : counters) {
+            if (c != 0u) {
+                return -4;                     // a counter did not return to zero
+            }
+        }
+    }
+    return 0;
 }
 
 }

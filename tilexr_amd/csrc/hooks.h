@@ -80,6 +80,16 @@ int64_t TileXREpHookAlignUp(int64_t value, int64_t alignment);
 int64_t TileXREpHookUdmaOperationBytes(int64_t totalBytes, int64_t rankSize, int64_t slotBytes);
 int64_t TileXREpHookUdmaWorkspaceBytes(int64_t totalBytes, int64_t rankSize, int64_t slotBytes);
 
+/* Runs the readiness-tile bookkeeping of the scatter kernels (ep_tile_publish.h) on `threads` CPU threads that land
+ * the parts of `totalRows` rows in a seeded random order, `rounds` dispatches in a row on the same counters and
+ * flags.  Checks on the way: a readiness word is stored only when every part of every row of its tile has landed,
+ * and exactly once per dispatch.  Checks at the end of each dispatch: every word is (epoch << 32) | rows in the
+ * tile, every counter is back to zero.  Returns 0, or a negative code naming the first violated check.
+ * `fault` plants a caller-side mistake so that a test can see the checks fire: 1 = a part is reported before it has
+ * landed, 2 = one part is reported twice. */
+int TileXREpHookTilePublishStress(int totalRows, int maxRows, int tileRows, int parts, int threads, int rounds,
+    uint32_t seed, int fault);
+
 #ifdef __cplusplus
 }
 #endif
