@@ -160,3 +160,52 @@ def test_flag_wait_expires_instead_of_hanging():
         st = ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream,
                                   tile_flags=flags, tile_rows=0)
         assert st == ep.ERR_PARA_CHECK_FAIL
+
+
+def test_combine_follows_an_expert_stage_that_publishes_tiles_in_random_order():
+    """The producer here is not the dispatch but an "expert stage" written with torch ops on a second stream: it
+    rewrites the rows tile by tile in a random order and stores a tile's readiness word after the tile's rows (a
+    kernel boundary on one stream is a release at device scope).  The combine is enqueued first, so it really waits;
+    it must return the weighted sum of the rewritten rows, never of the rows the buffer held before."""
+    bs, h, K, E, tile_rows = 2048, 1024, 4, 32, 128
+    rng = np.random.default_rng(31)
+    n = bs * K
+    tiles = (n + tile_rows - 1) // tile_rows
+    with Session() as s:
+        producer = torch.cuda.Stream()
+        ids, w = routing(rng, bs, K, E)
+        x = torch.from_numpy(rng.standard_normal((bs, h)).astype(np.float32)).to(torch.bfloat16)
+        d_x, d_ids, d_w = x.to(DEV), to_dev(ids), to_dev(w)
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        st, _ = ep.dispatch_memory_ex(d_x, d_ids, s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, ep.DT_BF16, s.stream, row_index_map=out["row_map"])
+        assert st == 0
+        s.sync()
+        rows = out["expand_x"].view(torch.bfloat16).view(n, h)
+        expert_out = torch.full((n, h), 99.0, dtype=torch.bfloat16, device=DEV)      # what a stale read would return
+        flags = torch.zeros((tiles,), dtype=torch.int64, device=DEV)
+        status = torch.zeros((1,), dtype=torch.int32, device=DEV)
+        y = torch.full((bs, h), 3.0, dtype=torch.bfloat16, device=DEV)
+        for epoch in (5, 6, 7):
+            scale = float(epoch)
+            torch.cuda.synchronize()
+            st = ep.combine_memory_ex(expert_out, out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream,
+                                      expert_scales=d_w, row_index_map=out["row_map"], tile_flags=flags,
+                                      tile_rows=tile_rows, flag_epoch=epoch, wait_timeout_us=10_000_000,
+                                      device_status=status)
+            assert st == 0
+            with torch.cuda.stream(producer):
+                for tile in rng.permutation(tiles):
+                    lo, hi = int(tile) * tile_rows, min(int(tile + 1) * tile_rows, n)
+                    expert_out[lo:hi] = (rows[lo:hi].float() * scale).to(torch.bfloat16)
+                    flags[int(tile)] = (epoch << 32) | (hi - lo)
+            producer.synchronize()
+            s.sync()
+            assert status.item() == 0
+            xb = bits16((x.float() * scale).to(torch.bfloat16))
+            case = O.Case(1, bs, h, K, E, token_nums_type=1)
+            want = O.mem_dispatch(case, 0, xb[None], ids[None])
+            wy = O.mem_combine(case, 0, want["expand_x"].view(np.uint16)[None], want["assist"][None],
+                               want["send_counts"][None], expert_scales=w)
+            assert np.array_equal(bits16(y), wy), f"epoch {epoch}"
