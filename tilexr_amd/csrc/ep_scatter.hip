@@ -1,11 +1,16 @@
 // scatter: each token row is read once and written to the rows its routes were placed at (gfx950, wave64).
 //
-// HBM-bound byte movement, no MFMA.  G lanes cooperate on one token (a wave for narrow rows, the whole workgroup for
-// wide ones); a lane keeps V 16-byte vectors of the row in registers, so every load of the row is in flight before
-// the first store, then writes them to each of the topK destination rows with non-temporal 128-bit stores (the rows
-// are not read again by this kernel; the input row is loaded with the default policy so that a producer's output
-// still sitting in L2 / Infinity Cache is used).  Measured on MI355X this shape moves 4096 x 7168 bf16 x top-8
-// (529 MB) at about 5.6 TB/s; destination order (sorted or random rows) makes no difference.
+// HBM-bound byte movement, no MFMA.  Three kernels share the work:
+//   ep_scatter_route_kernel    plain copies of wide rows in batches of 1024 tokens and more: one workgroup per
+//                              (token, k, slice of 512 vectors), two 16-byte loads and two 16-byte stores per lane
+//   ep_scatter_vec_kernel      everything else that is 16-byte aligned (quantised payloads, narrow rows, small
+//                              batches): G lanes cooperate on one token (a wave for narrow rows, the whole workgroup
+//                              for wide ones); a lane keeps V 16-byte vectors of the row in registers, so every load of
+//                              the row is in flight before the first store, then writes them to each destination row
+//   ep_scatter_generic_kernel  any width and alignment, element by element
+// Rows are written with non-temporal stores (they are not read again by this kernel; the input row is loaded with the
+// default policy so that the sibling workgroups of a token find it in L2), or with agent-scope write-through stores
+// when readiness flags are published.  Destination order (sorted or random rows) makes no difference.
 //
 //   QMODE 0  byte copy             (reference: src/ep/kernels/tilexr_ep_dispatch_helpers.h:104-112)
 //   QMODE 1  static int8           (reference: tilexr_ep_dispatch_helpers.h:114-136)
