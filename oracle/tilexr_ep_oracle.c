@@ -541,6 +541,17 @@ int64_t orc_mem_dispatch_rank(const orc_case *c, int32_t dst_rank, const uint16_
                         continue;
                     }
                     t = i % tokens;
+                    if (c->mask_type == ORC_MASK_EXPERT && ms) {
+                        /* the shared routes go out for the tokens that keep at least one routed expert
+                         * (tilexr_ep_dispatch_memory_kernel.h:1412-1441, 641-647; demo :613-620) */
+                        int any = 0;
+                        for (int64_t kk = 0; kk < c->top_k; ++kk) {
+                            any |= ms[t * c->top_k + kk] != 0;
+                        }
+                        if (!any) {
+                            continue;
+                        }
+                    }
                     k = c->top_k + s;
                     tuple_expert = (int32_t)s;      /* :1257 topKId - K on a shared rank */
                 } else {

@@ -409,10 +409,14 @@ def test_memory_dispatch_and_combine_with_shared_experts(shape, dtype):
     tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
     with World(R) as w:
         for mask_type, nums_type, quant in ((ep.MASK_NONE, 1, ep.Q_NONE), (ep.MASK_TOKEN, 0, ep.Q_NONE),
-                                            (ep.MASK_NONE, 1, ep.Q_MXFP8)):
+                                            (ep.MASK_EXPERT, 1, ep.Q_NONE), (ep.MASK_NONE, 1, ep.Q_MXFP8)):
             if quant == ep.Q_MXFP8 and h % 32 != 0:
                 continue
-            mask = (rng.random((R, bs)) < 0.7).astype(np.uint8) if mask_type == ep.MASK_TOKEN else None
+            mask = None
+            if mask_type == ep.MASK_TOKEN:
+                mask = (rng.random((R, bs)) < 0.7).astype(np.uint8)
+            elif mask_type == ep.MASK_EXPERT:
+                mask = (rng.random((R, bs, K)) < 0.5).astype(np.uint8)
             case = O.Case(R, bs, h, K, E, dtype=dtype, mask_type=mask_type, token_nums_type=nums_type, quant_mode=quant,
                           out_dtype=O.DT_FP8E4M3, shared_expert_num=S, shared_expert_rank_num=SR)
             outs = [alloc_shared_outputs(R, bs, h, K, S, case.local_experts, quant, True, r, SR) for r in range(R)]
@@ -462,20 +466,6 @@ def test_memory_dispatch_and_combine_with_shared_experts(shape, dtype):
                 want_y = O.mem_combine(plain, r, eo_np, assist_np, counts_np, expert_scales=weights[r],
                                        shared_expert_x=shared_b[r])
                 assert np.array_equal(bits16(ys[r]), want_y), f"rank {r}"
-
-
-def test_expert_mask_with_shared_experts_is_reported_as_unsupported():
-    R, bs, h, K, E, S, SR = 4, 8, 16, 2, 6, 1, 1
-    rng = np.random.default_rng(5)
-    ids = rand_ids(rng, R, bs, K, E)
-    xt, _ = rand_x(rng, R, bs, h, ep.DT_BF16)
-    mask = np.ones((bs, K), np.uint8)
-    with World(R) as w:
-        o = alloc_shared_outputs(R, bs, h, K, S, E // (R - SR), ep.Q_NONE, True, 0, SR)
-        st = ep.dispatch_memory_v2(xt[0], to_dev(ids[0]), w.comms[0], bs, h, K, E, o["expand_x"], o["assist"],
-                                   o["token_nums"], o["counts"], ep.DT_BF16, w.streams[0], active_mask=to_dev(mask),
-                                   active_mask_type=ep.MASK_EXPERT, shared_expert_num=S, shared_expert_rank_num=SR)
-        assert st == ep.ERR_NOT_SUPPORT
 
 
 # ---------------------------------------------------------------------------------------------

@@ -500,17 +500,27 @@ SHARED_SHAPES = [  # R, bs, h, K, E, S, SR
 
 
 @pytest.mark.parametrize("shape", SHARED_SHAPES)
-@pytest.mark.parametrize("masked", [False, True])
+@pytest.mark.parametrize("masked", [False, True, "expert"])
 def test_shared_experts_memory_route_matches_demo_golden(orc, shape, masked):
     R, bs, h, K, E, S, SR = shape
-    rng = np.random.default_rng(sum(shape) + masked)
+    rng = np.random.default_rng(sum(shape) + bool(masked) + 2 * (masked == "expert"))
+    mask_type = {False: O.MASK_NONE, True: O.MASK_TOKEN, "expert": O.MASK_EXPERT}[masked]
     case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16, shared_expert_num=S, shared_expert_rank_num=SR,
-                  mask_type=O.MASK_TOKEN if masked else O.MASK_NONE, token_nums_type=1)
+                  mask_type=mask_type, token_nums_type=1)
     ids = rand_ids(rng, R, bs, K, E, invalid_frac=0.1)
     x = rand_x(rng, R, bs, h)
-    mask = (rng.random((R, bs)) < 0.7).astype(np.uint8) if masked else None
-    # the memory route dispatches the first sum(mask) tokens of a source rank (prefix rule)
-    live = [[t < int(mask[s].sum()) for t in range(bs)] for s in range(R)] if masked else [[True] * bs] * R
+    mask = None
+    if masked == "expert":
+        # demo :599-620: a route is live when its mask byte is set, a token when one of its routes is
+        mask = (rng.random((R, bs, K)) < 0.5).astype(np.uint8)
+        live = [[bool(mask[s, t].any()) for t in range(bs)] for s in range(R)]
+        ids = np.where(mask != 0, ids, -1).astype(np.int32)          # what the golden walk sees of a masked route
+    elif masked:
+        mask = (rng.random((R, bs)) < 0.7).astype(np.uint8)
+        # the memory route dispatches the first sum(mask) tokens of a source rank (prefix rule)
+        live = [[t < int(mask[s].sum()) for t in range(bs)] for s in range(R)]
+    else:
+        live = [[True] * bs] * R
     total = 0
     for dst in range(R):
         got = orc.mem_dispatch(case, dst, x, ids, mask)

@@ -44,6 +44,9 @@ struct AugmentLaunch {
     bool sharedAtExpertId;   // local index of shared route s on its rank: s (MVP route) or 0 (memory route)
     int32_t *keyIdsOut;      // [bs, sharedNum + topK]; -1 = not routed
     int32_t *tupleExpertsOut;// [bs, sharedNum + topK]
+    const uint8_t *routeMask;    // optional [bs, topK] expert mask ...
+    uint8_t *routeMaskOut;       // ... widened to [bs, sharedNum + topK]: a token's shared routes are live when the
+                                 // token keeps at least one routed expert
     hipStream_t stream;
 };
 

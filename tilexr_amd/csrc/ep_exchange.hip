@@ -61,6 +61,8 @@ struct AugmentArgs {
     int sharedAtExpertId;
     int32_t *keyIdsOut;
     int32_t *tupleExpertsOut;
+    const uint8_t *routeMask;
+    uint8_t *routeMaskOut;
 };
 
 __global__ __launch_bounds__(kThreads) void ep_augment_kernel(AugmentArgs a)
@@ -88,6 +90,19 @@ __global__ __launch_bounds__(kThreads) void ep_augment_kernel(AugmentArgs a)
     }
     a.keyIdsOut[i] = keyId;
     a.tupleExpertsOut[i] = tupleExpert;
+    if (a.routeMaskOut != nullptr) {
+        // (reference: src/ep/kernels/tilexr_ep_dispatch_memory_kernel.h:1412-1441 keeps the tokens whose mask row
+        // has a set byte and walks the shared routes over those, :641-647)
+        uint8_t live = 0;
+        if (pos < a.sharedNum) {
+            for (int k = 0; k < a.topK; ++k) {
+                live |= a.routeMask[token * a.topK + k];
+            }
+        } else {
+            live = a.routeMask[token * a.topK + (pos - a.sharedNum)];
+        }
+        a.routeMaskOut[i] = live != 0 ? 1 : 0;
+    }
 }
 
 struct DrainPlanArgs {
@@ -338,6 +353,8 @@ hipError_t LaunchAugment(const AugmentLaunch &l)
     a.sharedAtExpertId = l.sharedAtExpertId ? 1 : 0;
     a.keyIdsOut = l.keyIdsOut;
     a.tupleExpertsOut = l.tupleExpertsOut;
+    a.routeMask = l.routeMask;
+    a.routeMaskOut = l.routeMaskOut;
     const int grid = (a.n + kThreads - 1) / kThreads;
     hipLaunchKernelGGL(ep_augment_kernel, dim3(grid > 0 ? grid : 1), dim3(kThreads), 0, l.stream, a);
     return hipGetLastError();

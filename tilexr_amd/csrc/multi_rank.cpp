@@ -177,11 +177,6 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     if (!WithinKernelLimits(p.bs, p.h, p.topK + shared, std::max(p.moeExpertNum, keySpaceBound), R) || p.extended) {
         return TileXR::TILEXR_ERROR_NOT_SUPPORT;
     }
-    if (shared > 0 && p.xActiveMask != nullptr && memoryRoute && p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT) {
-        // the reference compacts the tokens that keep at least one route before it walks the shared routes
-        // (tilexr_ep_dispatch_memory_kernel.h:1483-1500, 645-647); that combination is not built
-        return TileXR::TILEXR_ERROR_NOT_SUPPORT;
-    }
     hipStream_t stream = static_cast<hipStream_t>(p.stream);
     ExchangeShape shape {};
     shape.bs = p.bs;
@@ -233,10 +228,11 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     // ---- send half: group this rank's rows by destination in its staging area ----
     const int64_t n = p.bs * plan.perToken;
     const CountScratchLayout cs = PlanCountScratch(n, plan.numKeys, plan.keySpace, plan.expertHist);
-    const int64_t tableBytes = shared > 0 ? Align256(n * 4) : 0;      // key ids, then tuple expert ids
-    if (!comm->dispatchScratch.Reserve(static_cast<size_t>(cs.totalBytes + 2 * tableBytes), true)) {
+    const int64_t tableBytes = shared > 0 ? Align256(n * 4) : 0;      // key ids, tuple expert ids, widened mask
+    if (!comm->dispatchScratch.Reserve(static_cast<size_t>(cs.totalBytes + 3 * tableBytes), true)) {
         return TileXR::TILEXR_ERROR_INTERNAL;
     }
+    const uint8_t *routeMask = reinterpret_cast<const uint8_t *>(p.xActiveMask);
     CountScratch scratch = CarveCountScratch(comm->dispatchScratch.ptr, cs, plan.expertHist);
     const int32_t *routeIds = p.expertIds;
     const int32_t *tupleExperts = nullptr;
@@ -258,6 +254,13 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
         aug.sharedAtExpertId = !memoryRoute;
         aug.keyIdsOut = keyIds;
         aug.tupleExpertsOut = tuples;
+        if (memoryRoute && p.xActiveMask != nullptr && p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT) {
+            uint8_t *wide = reinterpret_cast<uint8_t *>(static_cast<char *>(comm->dispatchScratch.ptr) + cs.totalBytes +
+                2 * tableBytes);
+            aug.routeMask = routeMask;
+            aug.routeMaskOut = wide;
+            routeMask = wide;
+        }
         aug.stream = stream;
         const int ar = LaunchStatus(LaunchAugment(aug), "route tables");
         if (ar != kOk) {
@@ -275,7 +278,7 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
 
     RouteCountLaunch count {};
     count.ids = routeIds;
-    count.mask = reinterpret_cast<const uint8_t *>(p.xActiveMask);
+    count.mask = routeMask;
     if (p.xActiveMask == nullptr) {
         count.maskMode = kMaskNone;
     } else if (!memoryRoute) {
