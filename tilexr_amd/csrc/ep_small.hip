@@ -143,6 +143,105 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_kernel(SmallArgs a
     }
 }
 
+// Block-wide count of the lanes' set predicates over the kIdsPerLane id slots: ballots per wave, one LDS add per wave.
+__device__ __forceinline__ void AddBallots(const bool (&pred)[kIdsPerLane], int *sum, int lane)
+{
+    int n = 0;
+#pragma unroll
+    for (int j = 0; j < kIdsPerLane; ++j) {
+        n += __popcll(__ballot(pred[j]));
+    }
+    if (lane == 0 && n != 0) {
+        atomicAdd(sum, n);
+    }
+}
+
+// Without a capacity limit a route's row needs no histogram at all:
+//   row = (valid routes with a smaller expert id) + (earlier routes with the same expert id)
+// so one workgroup per route counts those two sets over the id table and writes its one row.  Workgroup b < E also
+// counts expert b's routes for the count outputs.  Eight times as many workgroups as tokens spread a decode batch
+// over the whole chip.
+template <int V>
+__global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(SmallArgs a)
+{
+    __shared__ int s_sum[4];     // smaller ids, earlier equal ids, ids equal to blockIdx, ids not above blockIdx
+
+    const int tid = threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int route = blockIdx.x;
+    const int token = route / a.topK;
+    const int n = a.bs * a.topK;
+    const int vecs = a.h / 8;
+
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.x) + static_cast<int64_t>(token) * a.h * 2);
+    u32x4 v[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int idx = j * kThreads + tid;
+        v[j] = idx < vecs ? src[idx] : u32x4{0u, 0u, 0u, 0u};
+    }
+    int e[kIdsPerLane];
+#pragma unroll
+    for (int j = 0; j < kIdsPerLane; ++j) {
+        const int i = j * kThreads + tid;
+        const int id = i < n ? a.ids[i] : -1;
+        e[j] = (id >= 0 && id < a.numExperts) ? id : -1;
+    }
+    const int mine = a.ids[route];
+    const int key = (mine >= 0 && mine < a.numExperts) ? mine : -1;
+    if (tid < 4) {
+        s_sum[tid] = 0;
+    }
+    __syncthreads();
+    const int expert = blockIdx.x;       // the expert this workgroup counts for the outputs (if there is one)
+    bool less[kIdsPerLane], before[kIdsPerLane], same[kIdsPerLane], upTo[kIdsPerLane];
+#pragma unroll
+    for (int j = 0; j < kIdsPerLane; ++j) {
+        const int i = j * kThreads + tid;
+        less[j] = e[j] >= 0 && e[j] < key;
+        before[j] = e[j] >= 0 && e[j] == key && i < route;
+        same[j] = e[j] == expert;
+        upTo[j] = e[j] >= 0 && e[j] <= expert;
+    }
+    AddBallots(less, &s_sum[0], lane);
+    AddBallots(before, &s_sum[1], lane);
+    if (expert < a.numExperts) {
+        AddBallots(same, &s_sum[2], lane);
+        AddBallots(upTo, &s_sum[3], lane);
+    }
+    __syncthreads();
+    const int row = key >= 0 ? s_sum[0] + s_sum[1] : -1;
+    if (tid == 0) {
+        if (row >= 0) {
+            int32_t *tuple = a.assist + static_cast<int64_t>(row) * 4;
+            tuple[0] = a.srcRank;
+            tuple[1] = token;
+            tuple[2] = route % a.topK;
+            tuple[3] = key + a.expertIdBias;
+        }
+        if (a.rowOf != nullptr) {
+            a.rowOf[route] = row;
+        }
+        if (expert < a.numExperts) {
+            a.sendCountsOut[expert] = s_sum[3];
+            if (a.expertTokenNumsOut != nullptr) {
+                a.expertTokenNumsOut[expert] = a.tokenNumsType == 0 ? s_sum[3] : s_sum[2];
+            }
+        }
+    }
+    if (row < 0) {
+        return;
+    }
+    u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+        const int idx = j * kThreads + tid;
+        if (idx < vecs) {
+            __builtin_nontemporal_store(v[j], dst + idx);
+        }
+    }
+}
+
 } // namespace
 
 bool SmallDispatchFits(const SmallDispatchLaunch &l)
@@ -169,8 +268,20 @@ hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l)
     a.sendCountsOut = l.sendCountsOut;
     a.expertTokenNumsOut = l.expertTokenNumsOut;
     a.tokenNumsType = l.tokenNumsType;
-    const dim3 grid(static_cast<unsigned>(l.bs));
     const int64_t vecs = l.h / 8;
+    if (l.capacity <= 0 && l.bs * l.topK >= l.numExperts) {
+        // one workgroup per route (there are enough of them to cover the experts' count outputs)
+        const dim3 routes(static_cast<unsigned>(l.bs * l.topK));
+        if (vecs <= 2 * kThreads) {
+            hipLaunchKernelGGL(ep_dispatch_small_route_kernel<2>, routes, dim3(kThreads), 0, l.stream, a);
+        } else if (vecs <= 4 * kThreads) {
+            hipLaunchKernelGGL(ep_dispatch_small_route_kernel<4>, routes, dim3(kThreads), 0, l.stream, a);
+        } else {
+            hipLaunchKernelGGL(ep_dispatch_small_route_kernel<8>, routes, dim3(kThreads), 0, l.stream, a);
+        }
+        return hipGetLastError();
+    }
+    const dim3 grid(static_cast<unsigned>(l.bs));
     if (vecs <= 2 * kThreads) {
         hipLaunchKernelGGL(ep_dispatch_small_kernel<2>, grid, dim3(kThreads), 0, l.stream, a);
     } else if (vecs <= 4 * kThreads) {
