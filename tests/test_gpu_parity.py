@@ -397,3 +397,78 @@ def test_degenerate_routing_tables(kind, shape):
             assert np.array_equal(bits16(y), wy)
             if kind == "all_invalid":
                 assert n == 0 and not bits16(y).any()
+
+
+# ---------------------------------------------------------------------------------------------
+# Every finite 16-bit input pattern through the device quantisers and the device reduce
+# ---------------------------------------------------------------------------------------------
+def _all_finite_patterns(dtype, seed):
+    """[128, 512] uint16 holding every finite bf16 / fp16 bit pattern once (non-finite ones replaced by zero), shuffled
+    so that every pattern meets different row and block maxima under different seeds."""
+    bits = np.arange(65536, dtype=np.uint32).astype(np.uint16)
+    exp_all_ones = (bits & 0x7f80) == 0x7f80 if dtype == ep.DT_BF16 else (bits & 0x7c00) == 0x7c00
+    bits[exp_all_ones] = 0
+    np.random.default_rng(seed).shuffle(bits)
+    return bits.reshape(128, 512)
+
+
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+@pytest.mark.parametrize("quant,fp8", [(ep.Q_TOKEN_INT8, None), (ep.Q_MXFP8, ep.DT_FP8E4M3), (ep.Q_MXFP8, ep.DT_FP8E5M2),
+                                       (ep.Q_FP8_BLOCK128, None)])
+def test_device_quantisers_on_every_finite_input_pattern(dtype, quant, fp8):
+    bs, h, K, E = 128, 512, 1, 4
+    for seed in (1, 2, 3):
+        xb = _all_finite_patterns(dtype, seed)
+        if seed == 3:
+            # moderate magnitudes only: the first two seeds put a huge element into nearly every block, which sends
+            # almost everything else to zero; here the small values get quantised for real
+            big = (xb & 0x7fff) > (0x4300 if dtype == ep.DT_BF16 else 0x5800)
+            xb = np.where(big, xb & 0x80ff, xb).astype(np.uint16)
+        xt = torch.from_numpy(xb.view(np.int16)).view(torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16).to(DEV)
+        ids = (np.arange(bs, dtype=np.int32) % E).reshape(bs, K)
+        with Session() as s:
+            out = alloc_dispatch_outputs(bs, h, K, E, quant=quant)
+            counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+            st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                          out["token_nums"], counts, dtype, s.stream, quant_mode=quant,
+                                          dynamic_scales=out["scales"], expand_x_dtype=fp8)
+            assert st == 0
+            s.sync()
+            got = fetch(out, "send_counts", counts)
+            case = O.Case(1, bs, h, K, E, dtype=dtype, quant_mode=quant, out_dtype=fp8 or O.DT_FP8E4M3)
+            want = O.mem_dispatch(case, 0, xb[None], ids[None])
+            assert want["rows"] == bs
+            assert np.array_equal(got["expand_x"], want["expand_x"]), f"seed {seed}"
+            assert np.array_equal(got["scales"].reshape(bs, -1), want["dyn_scales"].reshape(bs, -1)), f"seed {seed}"
+
+
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+@pytest.mark.parametrize("comm_quant", [0, 3, 4])
+def test_device_reduce_on_every_finite_input_pattern(dtype, comm_quant):
+    """Rows holding every finite pattern, weights that are not powers of two, three rows per token: the fp32 multiply,
+    the adds in k order, the MXFP8 exchange round trip and the final rounding all see every input once."""
+    bs, h, K, E = 128, 512, 3, 8
+    rng = np.random.default_rng(17 + dtype + comm_quant)
+    rows = np.concatenate([_all_finite_patterns(dtype, seed) for seed in (5, 6, 7)])          # [384, 512]
+    if dtype == ep.DT_FP16:
+        rows = np.where((rows & 0x7fff) > 0x7000, rows & 0x8fff, rows).astype(np.uint16)     # keep sums finite
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(bs)]).astype(np.int32)
+    w = (rng.random((bs, K)) * 1.7 + 0.05).astype(np.float32)
+    # a layout to combine over: dispatch a dummy x, then put the pattern rows in place of the expert outputs
+    tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+    with Session() as s:
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        xt = torch.zeros((bs, h), dtype=tdt, device=DEV)
+        st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, dtype, s.stream, row_index_map=out["row_map"])
+        assert st == 0
+        expert_out = torch.from_numpy(rows.view(np.int16)).view(tdt).to(DEV)
+        y = torch.zeros((bs, h), dtype=tdt, device=DEV)
+        assert ep.combine_memory_v2(expert_out, out["assist"], counts, s.comm, bs, h, K, E, y, dtype, s.stream,
+                                    expert_scales=to_dev(w), quant_mode=comm_quant) == 0
+        s.sync()
+        case = O.Case(1, bs, h, K, E, dtype=dtype)
+        wy = O.mem_combine(case, 0, rows[None], out["assist"].cpu().numpy()[None], counts.cpu().numpy()[None],
+                           expert_scales=w, comm_quant=comm_quant)
+        assert np.array_equal(bits16(y), wy)
