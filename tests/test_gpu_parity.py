@@ -472,3 +472,41 @@ def test_device_reduce_on_every_finite_input_pattern(dtype, comm_quant):
         wy = O.mem_combine(case, 0, rows[None], out["assist"].cpu().numpy()[None], counts.cpu().numpy()[None],
                            expert_scales=w, comm_quant=comm_quant)
         assert np.array_equal(bits16(y), wy)
+
+
+@pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
+@pytest.mark.parametrize("quant", [ep.Q_TOKEN_INT8, ep.Q_FP8_BLOCK128])
+def test_quantised_combine_input_on_every_code(dtype, quant):
+    """Every int8 value / every e4m3 code that is a number, under scales spread over the fp32 range that keep the
+    dequantised values finite in the output type: dequantise, round to the element type, weight, sum."""
+    bs, h, K, E = 64, 512, 2, 4
+    rng = np.random.default_rng(23 + dtype + quant)
+    n = bs * K
+    ids = np.stack([rng.permutation(E)[:K] for _ in range(bs)]).astype(np.int32)
+    codes = np.arange(256, dtype=np.uint8)
+    if quant == ep.Q_FP8_BLOCK128:
+        codes = codes[(codes & 0x7f) != 0x7f]                       # 0x7f / 0xff are NaN codes
+    payload = rng.choice(codes, size=(n, h)).astype(np.uint8)
+    payload[:, :codes.size] = codes                                 # every code in every row
+    top = 200.0 if dtype == ep.DT_FP16 else 1e30                    # code 448 * scale stays finite in fp16
+    if quant == ep.Q_TOKEN_INT8:
+        scales = np.exp(rng.uniform(np.log(1e-30), np.log(top), size=(n, 1))).astype(np.float32)
+    else:
+        scales = np.exp(rng.uniform(np.log(1e-30), np.log(top / 4), size=(n, h // 128))).astype(np.float32)
+    w = (0.3 + rng.random((bs, K))).astype(np.float32)
+    tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+    with Session() as s:
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        xt = torch.zeros((bs, h), dtype=tdt, device=DEV)
+        st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, dtype, s.stream, row_index_map=out["row_map"])
+        assert st == 0
+        y = torch.zeros((bs, h), dtype=tdt, device=DEV)
+        assert ep.combine_memory_ex(to_dev(payload), out["assist"], counts, s.comm, bs, h, K, E, y, dtype, s.stream,
+                                    expert_out_quant_mode=quant, expert_out_scales=to_dev(scales),
+                                    expert_scales=to_dev(w)) == 0
+        s.sync()
+        want = O.mem_combine(O.Case(1, bs, h, K, E, dtype=dtype), 0, payload[None], out["assist"].cpu().numpy()[None],
+                             counts.cpu().numpy()[None], expert_scales=w, in_quant=quant, in_scales=scales)
+        assert np.array_equal(bits16(y), want)
