@@ -9,6 +9,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include "ep_context.h"
+#include "moonep_host.h"
 #include "tilexr_api.h"
 #include "tilexr_types.h"
 
@@ -38,6 +39,7 @@ void ReleaseWorld(EpWorld *world)
             }
         }
     }
+    TileXRMoon::ReleaseWorldState(world->moon);
     delete world;
 }
 

@@ -22,6 +22,10 @@
 #include "comm_args.h"
 #include "ep_host.h"
 
+namespace TileXRMoon {
+struct WorldState;     // per-world state of the plan-driven stages (moonep_host.h)
+}
+
 namespace TileXREp {
 
 constexpr int64_t kFlagAreaBytesPerRank = 64 * 1024;
@@ -97,6 +101,7 @@ struct EpWorld {
     DeviceBuffer stageCounts;     // [R] keyOffset + expertTotal
     DeviceBuffer combineSlots;    // [R] [bs, topK] rows returned by the expert ranks
     DeviceBuffer combineMeta;     // [R] tagged slot table + order keys
+    TileXRMoon::WorldState *moon = nullptr;   // created by the first plan-driven call of the world
 };
 
 struct EpComm {

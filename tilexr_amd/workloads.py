@@ -132,3 +132,74 @@ def algorithmic_bytes(w: Workload, kept_rows: int, inverse_index: bool = False):
     dispatch = T * H * 2 + T * K * 4 + kept_rows * row + kept_rows * 16 + E * 12
     combine = kept_rows * row + (T * K * 4 if inverse_index else kept_rows * 16) + T * K * 4 + T * H * 2
     return dispatch, combine
+
+
+# ---- plan-driven (MoonEP) stages ---------------------------------------------------------------------------------
+# M1  8 logical ranks x (4096 x 7168 bf16 N(0,1)); 32 experts (4 per rank); top-8 distinct uniform; fp32 route weights.
+#     The shape the reference publishes its MoonEP stage timings for (S=4096, K=8, H=7168, E=32, EP8).
+MOONEP_CONFIGS = {
+    "M1": Workload("M1", 8, 4096, 7168, 8, 32, routing="uniform"),
+}
+
+
+def moonep_home_plan(topk_experts, experts, token_padding=1, prefetch_slots=1, slack_rows=0):
+    """Plan of a world in which every expert is served by its home rank (no expert is replicated).
+
+    topk_experts: int32 tensor [R, S, K].  Returns a dict with
+      dst         int32 [R, S*K]  signed route words: rank * nvS + row, negated (-raw - 1) when an earlier route of the
+                                  same token already goes to that rank
+      cu_seqlens  int32 [R, E+B]  cumulative padded group ends of every rank's receive tensor (groups = the E experts,
+                                  then the B prefetch slots, all empty here)
+      nvs         rows of every rank's receive tensor
+    It follows the reference planner's layout and route numbering for the case without expert moves
+    (src/moonep/planner_v2/reference/ep_plan_reference.cpp:436-459 segments, :461-538 layouts, :540-595 route words):
+    on its home rank an expert's rows are ordered by source rank, then by the order its routes appear in the source's
+    [S, K] table; groups are padded to `token_padding` rows.  The reference sizes nvS for a balanced world
+    (S*K + (padding-1) * 2 * E/R, moonep_stage_reference.cpp:86-107); here it is the larger of that and what the busiest
+    rank receives, plus `slack_rows`, because nothing rebalances this plan."""
+    R, S, K = topk_experts.shape
+    E, B = experts, prefetch_slots
+    per_rank = E // R
+    ids = topk_experts.to(torch.int64).reshape(R, S * K)
+    home = ids // per_rank                                              # [R, N]
+    counts = torch.zeros(R, E, dtype=torch.int64)
+    counts.scatter_add_(1, ids, torch.ones_like(ids))                   # [src, expert]
+    seg_begin = torch.cumsum(counts, dim=0) - counts                     # rows of earlier sources within the expert
+    total = counts.sum(0)                                                # [E] rows of each expert on its home rank
+    padded = torch.where(total > 0, (total + token_padding - 1) // token_padding * token_padding, total)
+    cu = torch.zeros(R, E + B, dtype=torch.int64)
+    base = torch.zeros(E, dtype=torch.int64)
+    for d in range(R):
+        sizes = torch.zeros(E + B, dtype=torch.int64)
+        sizes[d * per_rank:(d + 1) * per_rank] = padded[d * per_rank:(d + 1) * per_rank]
+        ends = torch.cumsum(sizes, 0)
+        cu[d] = ends
+        base[d * per_rank:(d + 1) * per_rank] = (ends - sizes)[d * per_rank:(d + 1) * per_rank]
+    nvs = max(S * K + (token_padding - 1) * 2 * per_rank, int(cu[:, -1].max())) + slack_rows
+    # ordinal of a route among its source's routes to the same expert, in table order
+    order = torch.argsort(ids, dim=1, stable=True)
+    sorted_ids = torch.gather(ids, 1, order)
+    first = torch.searchsorted(sorted_ids, sorted_ids, right=False)      # start of each expert's run per source
+    ordinal = torch.empty_like(ids)
+    ordinal.scatter_(1, order, torch.arange(S * K).expand(R, -1) - first)
+    src_index = torch.arange(R).unsqueeze(1).expand(R, S * K)
+    row = base[ids] + seg_begin[src_index, ids] + ordinal
+    raw = home * nvs + row
+    # a route is a duplicate when an earlier route of its token goes to the same rank
+    hk = home.reshape(R, S, K)
+    same = hk.unsqueeze(3) == hk.unsqueeze(2)                            # [R, S, k, j]
+    earlier = torch.tril(torch.ones(K, K, dtype=torch.bool), diagonal=-1)
+    dup = (same & earlier).any(dim=3).reshape(R, S * K)
+    dst = torch.where(dup, -raw - 1, raw)
+    assert int(raw.max()) < 2 ** 31
+    return {"dst": dst.to(torch.int32).contiguous(), "cu_seqlens": cu.to(torch.int32), "nvs": int(nvs)}
+
+
+def moonep_algorithmic_bytes(s: int, k: int, h: int, with_weights: bool = True):
+    """Bytes one rank's dispatch and combine must move when every route names its own row:
+       dispatch = S*H*2 (read tokens once) + S*K*4 (route words) + S*K*H*2 (write rows) [+ S*K*8 weights in and out]
+       combine  = S*K*H*2 (read rows) + S*K*4 (reverse routes) + S*H*2 (write tokens) [+ S*K*8 weights]"""
+    w = s * k * 8 if with_weights else 0
+    dispatch = s * h * 2 + s * k * 4 + s * k * h * 2 + w
+    combine = s * k * h * 2 + s * k * 4 + s * h * 2 + w
+    return dispatch, combine
