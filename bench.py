@@ -39,7 +39,14 @@ def parse():
     p.add_argument("--gpus", type=int, default=1)
     p.add_argument("--steps", type=int, default=100)
     p.add_argument("--warmup", type=int, default=20)
-    p.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5"])
+    p.add_argument("--workload", default="C3", choices=["C2", "C3", "C4", "C5", "M1"],
+                   help="C2-C5: dispatch / combine by expert ids; M1: the plan-driven (MoonEP) stages at S=4096, K=8, "
+                        "H=7168")
+    p.add_argument("--moon-ranks", type=int, default=1,
+                   help="M1: logical ranks of the world on this device (1 = one rank's share with every route local, "
+                        "8 = the whole 8-rank world of the published shape)")
+    p.add_argument("--moon-saved", action="store_true",
+                   help="M1: dispatch with the saved duplicate plan instead of building it on every call")
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-kernel-events", action="store_true",
                    help="do not record per-kernel HIP events inside the timed region")
@@ -90,12 +97,192 @@ def cpu_baseline(w, x, ids, weights, kept_rows):
     }
 
 
+def moonep_cpu_baseline(world, s, k, h, experts):
+    """The CPU oracle of the plan-driven stages on one host core, at a sample of the workload's tokens."""
+    import numpy as np
+    import torch
+
+    from oracle import moonep as M
+    from tilexr_amd import workloads
+
+    sample = max(64, min(s, 4096 // world))
+    g = torch.Generator().manual_seed(99)
+    ids = torch.topk(torch.rand(world, sample, experts, generator=g), k, dim=2).indices.to(torch.int32)
+    plan = workloads.moonep_home_plan(ids, experts)
+    sh = M.Shape(world, sample, k, h, plan["nvs"])
+    dst = plan["dst"].numpy()
+    hidden = np.random.default_rng(1).integers(0, 0x4000, size=(world, sample, h), dtype=np.uint16)
+    weights = np.ones((world, sample * k), np.float32)
+    best = None
+    for _ in range(3):
+        t0 = time.perf_counter()
+        out, wout, _, dup = M.dispatch_world(sh, dst, hidden, weights, flags=M.FLAG_BUILD_DEDUP)
+        t1 = time.perf_counter()
+        M.combine_world(sh, M.build_dst_local(sh, dst), dup, out, wout)
+        t2 = time.perf_counter()
+        if best is None or t2 - t0 < best[0]:
+            best = (t2 - t0, t1 - t0, t2 - t1)
+    db, cb = workloads.moonep_algorithmic_bytes(sample, k, h)
+    return {
+        "value": round(world * (db + cb) / best[0] / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
+        "us_per_layer": round(best[0] * 1e6, 1), "dispatch_us": round(best[1] * 1e6, 1),
+        "combine_us": round(best[2] * 1e6, 1), "host_cores_available": os.cpu_count(),
+        "sample": f"{sample} of {s} tokens per rank, {world} rank(s), oracle C port, single thread, best of 3",
+    }
+
+
+def main_moonep(args):
+    """Plan-driven stages: a step is one Dispatch (every rank of the world) followed by one Combine, identity expert."""
+    import numpy as np
+    import torch
+
+    from oracle import moonep as M
+    from tilexr_amd import ep, moonep as mp, workloads
+
+    w = workloads.MOONEP_CONFIGS[args.workload]
+    world = args.moon_ranks
+    s, k, h = w.bs, w.top_k, w.h
+    experts = w.experts if world > 1 else max(k, w.experts // w.ranks)    # one rank's share keeps its own experts
+    g = torch.Generator().manual_seed(w.seed)
+    ids = torch.topk(torch.rand(world, s, experts, generator=g), k, dim=2).indices.to(torch.int32)
+    plan = workloads.moonep_home_plan(ids, experts)
+    nvs = plan["nvs"]
+    dst = plan["dst"]
+    sh = M.Shape(world, s, k, h, nvs)
+    dst_local = torch.from_numpy(M.build_dst_local(sh, dst.numpy()))
+    torch.cuda.set_device(0)
+    dev = "cuda:0"
+    comms = [ep.Comm(world, r) for r in range(world)]
+    streams = [torch.cuda.Stream() for _ in range(world)]
+    ranks = []
+    for r in range(world):
+        t = dict(dst=dst[r].to(dev), dl=dst_local[r].to(dev),
+                 groups=torch.zeros((nvs, 3), dtype=torch.int32, device=dev), loffs=torch.zeros(nvs, dtype=torch.int32, device=dev),
+                 counts=torch.zeros(2, dtype=torch.int32, device=dev), status=torch.zeros(8, dtype=torch.int32, device=dev),
+                 x=torch.randn(s, h, generator=g).to(torch.bfloat16).to(dev), wsk=torch.rand(s, k, generator=g).to(dev),
+                 rows=torch.empty((nvs, h), dtype=torch.bfloat16, device=dev), wnv=torch.empty(nvs, dtype=torch.float32, device=dev),
+                 y=torch.empty((s, h), dtype=torch.bfloat16, device=dev), wy=torch.empty((s, k), dtype=torch.float32, device=dev))
+        t["plan"] = mp.plan(s * k, world, experts, 1, nvs, k, t["dst"], t["groups"], t["loffs"], t["counts"], t["status"])
+        t["d_args"] = (mp.tensor(t["x"], mp.DT_BF16, (s, h)), mp.tensor(t["rows"], mp.DT_BF16, (nvs, h)))
+        t["d_w"] = dict(weights_sk=mp.tensor(t["wsk"], mp.DT_FP32, (s, k)), weights_nvs=mp.tensor(t["wnv"], mp.DT_FP32, (nvs,)))
+        t["c_args"] = (mp.tensor(t["rows"], mp.DT_BF16, (nvs, h)), mp.tensor(t["y"], mp.DT_BF16, (s, h)))
+        t["c_w"] = dict(weights_nvs=mp.tensor(t["wnv"], mp.DT_FP32, (nvs,)), weights_sk=mp.tensor(t["wy"], mp.DT_FP32, (s, k)))
+        ranks.append(t)
+
+    def dispatch(flags):
+        for r, t in enumerate(ranks):
+            ep.check(mp.dispatch_v1(comms[r], t["plan"], *t["d_args"], streams[r], flags=flags, **t["d_w"]), "dispatch")
+
+    def combine():
+        for r, t in enumerate(ranks):
+            ep.check(mp.combine_v1(comms[r], t["plan"], t["dl"], *t["c_args"], streams[r], **t["c_w"]), "combine")
+
+    flags = 0 if args.moon_saved else mp.FLAG_BUILD_DEDUP
+
+    def step():
+        dispatch(flags)
+        combine()
+
+    torch.cuda.synchronize()
+    dispatch(mp.FLAG_BUILD_DEDUP)       # the saved plan of a --moon-saved run
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    for t in ranks:
+        assert int(t["status"][0].item()) == 0
+    # identity expert: every token comes back as the sum of its routes, duplicate groups rounded first
+    r0 = ranks[0]
+    peer = torch.from_numpy(np.where(dst[0].numpy() >= 0, dst[0].numpy(), -dst[0].numpy().astype(np.int64) - 1) // nvs).reshape(s, k)
+    per_rank = torch.zeros(s, world, dtype=torch.int64).scatter_add_(1, peer, torch.ones_like(peer)).to(dev)
+    want = torch.zeros((s, h), dtype=torch.float32, device=dev)
+    for q in range(world):
+        want += (r0["x"].float() * per_rank[:, q:q + 1].float()).to(torch.bfloat16).float()
+    if not torch.equal(want.to(torch.bfloat16).view(torch.int16), r0["y"].view(torch.int16)):
+        print("combine(dispatch(x)) differs from the closed form", file=sys.stderr)
+        sys.exit(1)
+
+    dispatch_bytes, combine_bytes = workloads.moonep_algorithmic_bytes(s, k, h)
+    use_events = not args.no_kernel_events
+    stride = max(1, args.event_stride)
+    sampled = [i for i in range(args.steps) if i % stride == 0] if use_events else []
+    pairs = {i: [(ep.HipEvent(timing=True), ep.HipEvent(timing=True)) for _ in range(2)] for i in sampled}
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        if i in pairs:       # the events are set on rank 0's communicator and bracket the launch for the whole world
+            ep.set_kernel_timing_events(comms[0], ep.K_SCATTER, *pairs[i][0])
+            ep.set_kernel_timing_events(comms[0], ep.K_REDUCE, *pairs[i][1])
+            step()
+            ep.set_kernel_timing_events(comms[0], ep.K_SCATTER, None, None)
+            ep.set_kernel_timing_events(comms[0], ep.K_REDUCE, None, None)
+        else:
+            step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - t0
+    names = {"scatter": ep.last_kernel_name(comms[0], ep.K_SCATTER), "reduce": ep.last_kernel_name(comms[0], ep.K_REDUCE)}
+
+    ev = [ep.HipEvent(timing=True) for _ in range(3)]
+    if world == 1:
+        ev[0].record(streams[0])
+        dispatch(flags)
+        ev[1].record(streams[0])
+        combine()
+        ev[2].record(streams[0])
+        torch.cuda.synchronize()
+        split = (round(ev[0].elapsed_ms(ev[1]) * 1e3, 2), round(ev[1].elapsed_ms(ev[2]) * 1e3, 2))
+    else:
+        split = (None, None)
+
+    ms_per_step = elapsed / args.steps * 1e3
+    total_bytes = world * (dispatch_bytes + combine_bytes)
+    gbps = total_bytes / (ms_per_step * 1e-3) / 1e9
+    kernels, roofline = {}, None
+    if use_events:
+        # one launch of the scatter / reduce kernel covers every rank of the world
+        for which, (name, nbytes) in enumerate((("scatter", world * dispatch_bytes), ("reduce", world * combine_bytes))):
+            times = sorted(pairs[i][which][0].elapsed_ms(pairs[i][which][1]) * 1e3 for i in sampled)
+            avg = sum(times) / len(times)
+            kernels[name] = {"avg_us": round(avg, 2), "min_us": round(times[0], 2), "p50_us": round(times[len(times) // 2], 2),
+                             "max_us": round(times[-1], 2), "launches_timed": len(times), "algorithmic_bytes": nbytes,
+                             "achieved_GBps": round(nbytes / (avg * 1e-6) / 1e9, 1)}
+        dom = "scatter" if kernels["scatter"]["avg_us"] >= kernels["reduce"]["avg_us"] else "reduce"
+        roofline = {"bound": "hbm", "kernel": names[dom], "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS,
+                    "unit": "GB/s", "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4),
+                    "traffic": measured_traffic(f"{w.name}_r{world}", dom), "avg_launch_us": kernels[dom]["avg_us"],
+                    "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
+    result = {
+        "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",
+        "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5), "us_per_layer": round(ms_per_step * 1e3, 2),
+        "us_per_layer_per_rank": round(ms_per_step * 1e3 / world, 2),
+        "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{w.name}: plan-driven Dispatch + Combine, {world} logical rank(s) x {s} tokens x {h} bf16, "
+                               f"top-{k} of {experts} experts, home plan, fp32 route weights",
+                   "logical_ranks": world, "tokens_per_rank": s, "hidden": h, "top_k": k, "experts": experts, "nvs": nvs,
+                   "duplicate_routes": int((dst < 0).sum()), "routes": int(dst.numel()),
+                   "dispatch": "saved duplicate plan" if args.moon_saved else "builds the duplicate plan",
+                   "dispatch_bytes_per_rank": dispatch_bytes, "combine_bytes_per_rank": combine_bytes,
+                   "dispatch_us": split[0], "combine_us": split[1], "seed": w.seed,
+                   "dst_sha256": __import__("hashlib").sha256(dst.numpy().tobytes()).hexdigest()[:16]},
+        "roofline": roofline, "kernels": kernels,
+    }
+    if not args.no_cpu_baseline:
+        result["cpu_baseline"] = moonep_cpu_baseline(world, s, k, h, experts)
+    torch.cuda.synchronize()
+    for c in comms:
+        c.destroy()
+    print(json.dumps(result))
+
+
 def main():
     args = parse()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one device's share of the dispatch/combine path: run it with --gpus 1 "
               "(no collective or second GPU is part of this build)", file=sys.stderr)
         sys.exit(2)
+    if args.workload.startswith("M"):
+        return main_moonep(args)
 
     import torch
 

@@ -176,6 +176,7 @@ int TileXRMoeEpCombineMemoryEx(void *expertOut, int32_t *assistInfoForCombine, i
 // Measurement aid without a reference counterpart: while a pair of hipEvent_t is set for a kernel, every call on
 // `comm` that launches that kernel records `startEvent` immediately before and `stopEvent` immediately after it, on
 // the stream of the call.  Pass null events to clear.  Kernel ids: 0 count, 1 place, 2 scatter, 3 invert, 4 reduce.
+// Ids 2 and 4 also cover the scatter and reduce kernels of the plan-driven stages (tilexr_moonep.h).
 int TileXREpSetKernelTimingEvents(TileXRCommPtr comm, int kernel, void *startEvent, void *stopEvent);
 
 // Measurement aid without a reference counterpart: name of the kernel template the last call on `comm` launched

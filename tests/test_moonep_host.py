@@ -94,6 +94,9 @@ def test_dispatch_argument_rules(comms):
     assert mp.dispatch_v1(c, _plan(), hid, out, FAKE, struct_size=56) == INV                   # shorter than the oldest layout
     assert mp.dispatch_v1(c, _plan(), hid, out, FAKE, registered_workspace=FAKE) == NS
     assert mp.dispatch_v1(c, _plan(), hid, out, FAKE, registered_workspace_bytes=64) == NS
+    # a caller built before `trace` was added still selects the registered-workspace variant
+    # (reference: tests/moonep/unit/test_tilexr_moonep_host.cpp:302-306)
+    assert mp.dispatch_v1(c, _plan(), hid, out, FAKE, struct_size=80, registered_workspace=FAKE) == NS
     assert mp.dispatch_v1(c, _plan(), hid, out, FAKE, trace=mp.DispatchTraceV1()) == INV
     assert mp.dispatch_v1(c, _plan(), hid, out, FAKE, flags=mp.FLAG_ZERO_COPY) == NS
     assert mp.dispatch_v1(0xdead0, _plan(), hid, out, FAKE) == ep.ERR_NOT_INITIALIZED          # not a communicator

@@ -1,12 +1,13 @@
 // Host side of the plan-driven (MoonEP) Dispatch and Combine stages: the C entry points, argument validation in the
-// reference's order, and the ordering of the kernels of all logical ranks that share the device.
+// reference's order, and the ordering of the exchange among the logical ranks that share the device.
 //
 // The reference runs one process per rank and lets its kernels meet at magic-tagged barriers in each other's peer
 // windows (src/moonep/dispatch/kernels/tilexr_moonep_dispatch_kernel.cpp:108-147).  With every rank in one process on
 // one device the host orders the exchange instead: a call records what its rank asked for; when the last rank of the
-// world has called, every rank's kernels are enqueued on that rank's own stream, with events where one rank's kernels
-// read or write what another rank's kernels produced.  A rank's outputs are therefore complete once every rank has
-// made the call and the rank's stream has been synchronised.
+// world has called, the kernels -- each launched once for all ranks -- are enqueued on the world's own stream behind an
+// event of every rank's stream, and every rank's stream then waits for the end of the exchange.  A rank's outputs are
+// therefore complete once every rank has made the call and the rank's stream has been synchronised.  A world of one
+// rank runs directly on the caller's stream.
 #include <cstddef>
 #include <limits>
 #include <mutex>
@@ -153,8 +154,8 @@ bool PrepareTables(WorldState *st, int world, int64_t nvS, int64_t n, WorldTable
     const int64_t stride = (rows + kRowsPerGroup - 1) / kRowsPerGroup * kRowsPerGroup;
     const int64_t groups = stride / kRowsPerGroup;
     const int64_t perRank8 = stride * 8;
-    // six 8-byte tables, two 4-byte tables, then the per-rank words
-    const int64_t bytes = world * (6 * perRank8 + 2 * stride * 4) + world * 8 + world * groups * 4 + 256;
+    // six 8-byte tables, three 4-byte tables, then the per-rank words
+    const int64_t bytes = world * (6 * perRank8 + 3 * stride * 4) + world * 8 + world * groups * 12 + 256;
     if (!st->tables.Reserve(static_cast<size_t>(bytes), true)) {
         return false;
     }
@@ -167,13 +168,15 @@ bool PrepareTables(WorldState *st, int world, int64_t nvS, int64_t n, WorldTable
     out->rowTag = reinterpret_cast<uint64_t *>(take(world * perRank8));
     out->parentTag = reinterpret_cast<uint64_t *>(take(world * perRank8));
     out->groupStart = reinterpret_cast<uint64_t *>(take(world * perRank8));
-    out->dupMask = reinterpret_cast<uint64_t *>(take(world * perRank8));
-    out->groupOf = reinterpret_cast<uint64_t *>(take(world * perRank8));
     out->slotSrc = reinterpret_cast<uint64_t *>(take(world * perRank8));
+    out->slotDup = reinterpret_cast<uint64_t *>(take(world * perRank8));
+    out->slotGroup = reinterpret_cast<uint64_t *>(take(world * perRank8));
     out->fail = reinterpret_cast<uint64_t *>(take(world * 8));
     out->sibling = reinterpret_cast<uint32_t *>(take(world * stride * 4));
     out->workList = reinterpret_cast<int32_t *>(take(world * stride * 4));
+    out->slotCount = reinterpret_cast<int32_t *>(take(world * stride * 4));
     out->workCount = reinterpret_cast<int32_t *>(take(world * groups * 4));
+    out->chunkTotals = reinterpret_cast<int32_t *>(take(world * groups * 8));
     out->stride = stride;
     out->groupStride = groups;
     return true;
@@ -224,18 +227,64 @@ bool SameShape(const StageCall &a, const StageCall &b)
         (a.weightsSk != nullptr) == (b.weightsSk != nullptr);
 }
 
-// Every stream first waits for what the previous exchange left running on any stream of the world: the tables are
-// shared, and a kernel of this exchange must not overwrite an entry a kernel of the last one has yet to read.
-int WaitForPreviousExchange(WorldState *st, const std::vector<StageCall> &calls)
+// The stream the exchange runs on, and what it has to wait for first.  A one-rank world runs on the caller's stream.  A
+// larger world runs on a stream of its own that waits until every rank's stream has reached its call (`arrived`): the
+// kernels read and write all ranks' tensors.  Either way the stream also waits for the previous exchange of the world,
+// whose kernels may still be reading the shared tables.
+int BeginExchange(EpWorld *world, WorldState *st, const std::vector<StageCall> &calls, hipStream_t *stream)
 {
-    for (const StageCall &c : calls) {
-        for (RankEvents &e : st->events) {
-            if (e.doneArmed) {
-                MOON_TRY(hipStreamWaitEvent(c.stream, e.done, 0), "waiting for the previous exchange");
-            }
+    const int R = world->rankSize;
+    if (R == 1) {
+        *stream = calls[0].stream;
+    } else {
+        if (st->stream == nullptr) {
+            MOON_TRY(hipStreamCreateWithFlags(&st->stream, hipStreamNonBlocking), "creating the world's stream");
+        }
+        *stream = st->stream;
+        for (int r = 0; r < R; ++r) {
+            MOON_TRY(hipStreamWaitEvent(*stream, st->events[static_cast<size_t>(r)].arrived, 0), "waiting for a rank's call");
+        }
+    }
+    if (st->doneArmed) {
+        MOON_TRY(hipStreamWaitEvent(*stream, st->done, 0), "waiting for the previous exchange");
+    }
+    return kOk;
+}
+
+// Marks the end of the exchange and makes every rank's stream wait for it.
+int EndExchange(EpWorld *world, WorldState *st, const std::vector<StageCall> &calls, hipStream_t stream)
+{
+    if (st->done == nullptr) {
+        MOON_TRY(hipEventCreateWithFlags(&st->done, hipEventDisableTiming), "creating an event");
+    }
+    MOON_TRY(hipEventRecord(st->done, stream), "recording an event");
+    st->doneArmed = true;
+    if (world->rankSize > 1) {
+        for (const StageCall &c : calls) {
+            MOON_TRY(hipStreamWaitEvent(c.stream, st->done, 0), "waiting for the exchange");
         }
     }
     return kOk;
+}
+
+// Timing events and kernel names are a measurement aid of rank 0's communicator (TileXREpSetKernelTimingEvents): the
+// launch they bracket covers every rank of the world.
+LaunchTiming TimingOf(EpWorld *world, int kernel)
+{
+    EpComm *c = world->comms[0];
+    std::lock_guard<std::mutex> lock(c->mu);
+    LaunchTiming t;
+    t.start = c->timing[kernel][0];
+    t.stop = c->timing[kernel][1];
+    return t;
+}
+
+void NoteKernel(EpWorld *world, int kernel, const char *name)
+{
+    for (EpComm *c : world->comms) {
+        std::lock_guard<std::mutex> lock(c->mu);
+        c->lastKernel[kernel] = name;
+    }
 }
 
 int LaunchDispatchWorld(EpWorld *world, WorldState *st)
@@ -243,95 +292,36 @@ int LaunchDispatchWorld(EpWorld *world, WorldState *st)
     const int R = world->rankSize;
     const std::vector<StageCall> &calls = st->dispatch;
     const StageCall &shape = calls[0];
-    WorldTables tables {};
-    uint64_t epoch = 0;
-    if (!PrepareTables(st, R, shape.nvS, shape.s * shape.k, &tables) || !NextEpoch(st, &epoch)) {
+    DispatchWorld w {};
+    if (!PrepareTables(st, R, shape.nvS, shape.s * shape.k, &w.tables) || !NextEpoch(st, &w.epoch)) {
         return TILEXR_MOONEP_ERROR_INTERNAL;
     }
-    int ret = WaitForPreviousExchange(st, calls);
+    w.world = R;
+    w.s = shape.s;
+    w.k = shape.k;
+    w.h = shape.h;
+    w.nvS = shape.nvS;
+    w.fresh = (shape.flags & TILEXR_MOONEP_FLAG_BUILD_DEDUP) != 0;
+    for (int r = 0; r < R; ++r) {
+        const StageCall &c = calls[static_cast<size_t>(r)];
+        w.dst[r] = c.dst;
+        w.hiddenSh[r] = c.hiddenSh;
+        w.weightsSk[r] = c.weightsSk;
+        w.hiddenNvsh[r] = c.hiddenNvsh;
+        w.weightsNvs[r] = c.weightsNvs;
+        w.dupGroups[r] = c.dupGroups;
+        w.dupLoffs[r] = c.dupLoffs;
+        w.dupCounts[r] = c.dupCounts;
+        w.status[r] = c.status;
+    }
+    hipStream_t stream = nullptr;
+    int ret = BeginExchange(world, st, calls, &stream);
     if (ret != kOk) {
         return ret;
     }
-    const bool fresh = (shape.flags & TILEXR_MOONEP_FLAG_BUILD_DEDUP) != 0;
-    ReceiveTable out {};
-    for (int q = 0; q < R; ++q) {
-        out.hidden[q] = calls[static_cast<size_t>(q)].hiddenNvsh;
-        out.weights[q] = calls[static_cast<size_t>(q)].weightsNvs;
-    }
-    for (int s = 0; s < R; ++s) {
-        const StageCall &c = calls[static_cast<size_t>(s)];
-        // rows go straight into the other ranks' receive tensors: not before those ranks' streams have reached the call
-        for (int q = 0; q < R; ++q) {
-            if (q != s) {
-                MOON_TRY(hipStreamWaitEvent(c.stream, st->events[static_cast<size_t>(q)].arrived, 0), "waiting for a peer's call");
-            }
-        }
-        ScatterLaunch l {};
-        l.dst = c.dst;
-        l.hiddenSh = c.hiddenSh;
-        l.weightsSk = c.weightsSk;
-        l.s = c.s;
-        l.k = c.k;
-        l.h = c.h;
-        l.nvS = c.nvS;
-        l.world = R;
-        l.srcRank = s;
-        l.fresh = fresh;
-        l.out = out;
-        l.tables = tables;
-        l.epoch = epoch;
-        l.stream = c.stream;
-        MOON_TRY(LaunchMoonScatter(l), "launching the scatter kernel");
-        MOON_TRY(hipEventRecord(st->events[static_cast<size_t>(s)].sent, c.stream), "recording an event");
-    }
-    for (int q = 0; q < R; ++q) {
-        const StageCall &c = calls[static_cast<size_t>(q)];
-        for (int s = 0; s < R; ++s) {
-            if (s != q) {
-                MOON_TRY(hipStreamWaitEvent(c.stream, st->events[static_cast<size_t>(s)].sent, 0), "waiting for a peer's rows");
-            }
-        }
-        if (fresh) {
-            DedupBuildLaunch b {};
-            b.nvS = c.nvS;
-            b.rank = q;
-            b.tables = tables;
-            b.epoch = epoch;
-            b.dupGroups = c.dupGroups;
-            b.dupLoffs = c.dupLoffs;
-            b.dupCounts = c.dupCounts;
-            b.stream = c.stream;
-            MOON_TRY(LaunchMoonDedupBuild(b), "launching the duplicate-plan kernel");
-        } else {
-            GroupWalkLaunch w {};
-            w.nvS = c.nvS;
-            w.rank = q;
-            w.combine = false;
-            w.dupGroups = c.dupGroups;
-            w.dupLoffs = c.dupLoffs;
-            w.dupCounts = c.dupCounts;
-            w.tables = tables;
-            w.epoch = epoch;
-            w.stream = c.stream;
-            MOON_TRY(LaunchMoonGroupWalk(w), "launching the group-walk kernel");
-        }
-        FillLaunch f {};
-        f.nvS = c.nvS;
-        f.h = c.h;
-        f.world = R;
-        f.rank = q;
-        f.expand = !fresh;
-        f.hiddenNvsh = c.hiddenNvsh;
-        f.weightsNvs = c.weightsNvs;
-        f.tables = tables;
-        f.epoch = epoch;
-        f.status = c.status;
-        f.stream = c.stream;
-        MOON_TRY(LaunchMoonFill(f), "launching the fill kernels");
-        MOON_TRY(hipEventRecord(st->events[static_cast<size_t>(q)].done, c.stream), "recording an event");
-        st->events[static_cast<size_t>(q)].doneArmed = true;
-    }
-    return kOk;
+    MOON_TRY(LaunchMoonDispatch(w, stream, TimingOf(world, TileXREp::kKernelScatter)), "launching the dispatch kernels");
+    NoteKernel(world, TileXREp::kKernelScatter, MoonScatterKernelName());
+    return EndExchange(world, st, calls, stream);
 }
 
 int LaunchCombineWorld(EpWorld *world, WorldState *st)
@@ -339,76 +329,35 @@ int LaunchCombineWorld(EpWorld *world, WorldState *st)
     const int R = world->rankSize;
     const std::vector<StageCall> &calls = st->combine;
     const StageCall &shape = calls[0];
-    WorldTables tables {};
-    uint64_t epoch = 0;
-    if (!PrepareTables(st, R, shape.nvS, shape.s * shape.k, &tables) || !NextEpoch(st, &epoch)) {
+    CombineWorld w {};
+    if (!PrepareTables(st, R, shape.nvS, shape.s * shape.k, &w.tables) || !NextEpoch(st, &w.epoch)) {
         return TILEXR_MOONEP_ERROR_INTERNAL;
     }
-    int ret = WaitForPreviousExchange(st, calls);
+    w.world = R;
+    w.s = shape.s;
+    w.k = shape.k;
+    w.h = shape.h;
+    w.nvS = shape.nvS;
+    for (int r = 0; r < R; ++r) {
+        const StageCall &c = calls[static_cast<size_t>(r)];
+        w.dstLocal[r] = c.dstLocal;
+        w.hiddenNvsh[r] = c.hiddenNvsh;
+        w.weightsNvs[r] = c.weightsNvs;
+        w.dupGroups[r] = c.dupGroups;
+        w.dupLoffs[r] = c.dupLoffs;
+        w.dupCounts[r] = c.dupCounts;
+        w.hiddenSh[r] = c.hiddenShOut;
+        w.weightsSk[r] = c.weightsSkOut;
+        w.status[r] = c.status;
+    }
+    hipStream_t stream = nullptr;
+    int ret = BeginExchange(world, st, calls, &stream);
     if (ret != kOk) {
         return ret;
     }
-    SourceTable src {};
-    for (int q = 0; q < R; ++q) {
-        const StageCall &c = calls[static_cast<size_t>(q)];
-        src.hidden[q] = c.hiddenNvsh;
-        src.weights[q] = c.weightsNvs;
-        src.dupGroups[q] = c.dupGroups;
-        src.dupLoffs[q] = c.dupLoffs;
-    }
-    for (int q = 0; q < R; ++q) {
-        const StageCall &c = calls[static_cast<size_t>(q)];
-        GroupWalkLaunch w {};
-        w.nvS = c.nvS;
-        w.rank = q;
-        w.combine = true;
-        w.dupGroups = c.dupGroups;
-        w.dupLoffs = c.dupLoffs;
-        w.dupCounts = c.dupCounts;
-        w.tables = tables;
-        w.epoch = epoch;
-        w.stream = c.stream;
-        MOON_TRY(LaunchMoonGroupWalk(w), "launching the group-walk kernel");
-        ReverseLaunch r {};
-        r.dstLocal = c.dstLocal;
-        r.nvS = c.nvS;
-        r.n = c.s * c.k;
-        r.world = R;
-        r.rank = q;
-        r.tables = tables;
-        r.epoch = epoch;
-        r.stream = c.stream;
-        MOON_TRY(LaunchMoonReverse(r), "launching the reverse-route kernel");
-        MOON_TRY(hipEventRecord(st->events[static_cast<size_t>(q)].sent, c.stream), "recording an event");
-    }
-    for (int p = 0; p < R; ++p) {
-        const StageCall &c = calls[static_cast<size_t>(p)];
-        // covers both the slot table and the expert ranks' tensors: `sent` follows the expert rank's call on its stream
-        for (int q = 0; q < R; ++q) {
-            if (q != p) {
-                MOON_TRY(hipStreamWaitEvent(c.stream, st->events[static_cast<size_t>(q)].sent, 0), "waiting for a peer's slots");
-            }
-        }
-        MoonReduceLaunch l {};
-        l.s = c.s;
-        l.k = c.k;
-        l.h = c.h;
-        l.nvS = c.nvS;
-        l.world = R;
-        l.rank = p;
-        l.src = src;
-        l.tables = tables;
-        l.epoch = epoch;
-        l.hiddenSh = c.hiddenShOut;
-        l.weightsSk = c.weightsSkOut;
-        l.status = c.status;
-        l.numComputeUnits = world->numComputeUnits;
-        l.stream = c.stream;
-        MOON_TRY(LaunchMoonReduce(l), "launching the reduce kernel");
-        MOON_TRY(hipEventRecord(st->events[static_cast<size_t>(p)].done, c.stream), "recording an event");
-        st->events[static_cast<size_t>(p)].doneArmed = true;
-    }
-    return kOk;
+    MOON_TRY(LaunchMoonCombine(w, stream, TimingOf(world, TileXREp::kKernelReduce)), "launching the combine kernels");
+    NoteKernel(world, TileXREp::kKernelReduce, MoonReduceKernelName());
+    return EndExchange(world, st, calls, stream);
 }
 
 // Files one rank's call; the last rank of the world to arrive enqueues the whole exchange.
@@ -439,7 +388,7 @@ int Arrive(EpComm *comm, const StageCall &call, bool combine)
         }
     }
     RankEvents &ev = st->events[static_cast<size_t>(comm->rank)];
-    if (!EnsureEvent(&ev.arrived) || !EnsureEvent(&ev.sent) || !EnsureEvent(&ev.done)) {
+    if (!EnsureEvent(&ev.arrived)) {
         return TILEXR_MOONEP_ERROR_INTERNAL;
     }
     (void)comm->nextMagic.fetch_add(1);         // one magic per launch, as in the reference (moonep_stage_host.h:75-83)
@@ -466,11 +415,15 @@ void ReleaseWorldState(WorldState *st)
     }
     st->tables.Release();
     for (RankEvents &e : st->events) {
-        for (hipEvent_t ev : {e.arrived, e.sent, e.done}) {
-            if (ev != nullptr) {
-                (void)hipEventDestroy(ev);
-            }
+        if (e.arrived != nullptr) {
+            (void)hipEventDestroy(e.arrived);
         }
+    }
+    if (st->done != nullptr) {
+        (void)hipEventDestroy(st->done);
+    }
+    if (st->stream != nullptr) {
+        (void)hipStreamDestroy(st->stream);
     }
     delete st;
 }

@@ -35,9 +35,6 @@ struct StageCall {
 
 struct RankEvents {
     hipEvent_t arrived = nullptr;   // the rank's stream has reached its call
-    hipEvent_t sent = nullptr;      // what the rank's first kernels produce for its peers is enqueued
-    hipEvent_t done = nullptr;      // the rank's last kernel of the exchange is enqueued
-    bool doneArmed = false;
 };
 
 struct WorldState {
@@ -46,6 +43,9 @@ struct WorldState {
     std::vector<StageCall> dispatch;    // calls waiting for the rest of the world, by rank
     std::vector<StageCall> combine;
     std::vector<RankEvents> events;
+    hipStream_t stream = nullptr;       // worlds of several ranks: the stream their exchanges run on (default priority)
+    hipEvent_t done = nullptr;          // end of the last exchange
+    bool doneArmed = false;
 };
 
 void ReleaseWorldState(WorldState *st);

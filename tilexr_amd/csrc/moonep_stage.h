@@ -3,18 +3,20 @@
 // The reference moves rows through per-rank peer windows with magic-tagged barriers between "window cleared", "data
 // ready" and "window drained" (src/moonep/dispatch/kernels/tilexr_moonep_dispatch_kernel.cpp:108-147,
 // src/moonep/combine/kernels/tilexr_moonep_combine_kernel.cpp:117-177).  Here every rank of the world lives on one
-// device, so a source rank writes straight into the destination rank's receive tensor and the only shared state is a
-// set of small per-row tables in library scratch.  Every table entry carries the epoch of the call that wrote it in
-// its upper 32 bits, so nothing is ever cleared between calls.
+// device, so a source rank writes straight into the destination rank's receive tensor, and one launch of each kernel
+// covers every rank of the world (grid dimension y = rank).  The only shared state is a set of small per-row tables in
+// library scratch; every table entry carries the epoch of the call that wrote it in its upper 32 bits, so nothing is
+// ever cleared between calls.
 //
-//   dispatch  scatter   (per source rank)       rows, weights, row tags, parent / sibling records of duplicates
-//             build     (per destination rank)  fresh plans: dupGroups / dupLoffs / dupCounts from the parent records
-//             walk      (per destination rank)  saved plans: parent records from dupGroups / dupLoffs
-//             classify + fill (per destination) rows nobody named -> zero, duplicate rows of a saved plan -> copy of
-//                                               their primary row; device status
-//   combine   walk      (per expert rank)       duplicate mask and group-of-primary table
-//             reverse   (per expert rank)       dstLocal -> slot table of the origin ranks
-//             reduce    (per origin rank)       K slots per token, duplicate groups pre-summed, fp32 -> bf16
+//   dispatch  walk      saved plans: parent records from dupGroups / dupLoffs
+//             scatter   rows, weights, row tags; fresh plans: parent / sibling records of duplicates
+//             build     fresh plans: dupGroups / dupCounts from the parent records (chunk totals, then group records)
+//             classify  per row: what is left to write (zeros, or a copy of the primary of a saved plan); dupLoffs of
+//                       a fresh plan; weights of unnamed rows; device status
+//             fill      writes what classify listed
+//   combine   prepare   dstLocal and the duplicate plan -> per-slot tables of the origins (which row, duplicate or not,
+//                       its duplicate group)
+//             reduce    K slots per token, duplicate groups pre-summed, fp32 -> bf16; device status
 #ifndef TILEXR_AMD_MOONEP_STAGE_H
 #define TILEXR_AMD_MOONEP_STAGE_H
 
@@ -37,114 +39,68 @@ constexpr int32_t kCombineOk = 0;
 constexpr int32_t kCombineInvalidRoute = 3001;
 constexpr int32_t kCombineRemoteFailureBase = 3100;
 
-// Per-row tables of one world, each [world][nvS] unless noted; `stride` = entries per rank.
+// Per-row tables of one world, each [world][stride] unless noted.
 struct WorldTables {
-    uint64_t *rowTag;        // dispatch: epoch << 32 | 2 (a route names the row) | 1 (a route wrote its hidden values)
+    uint64_t *rowTag;        // dispatch: epoch << 32 | bits: a route names the row, a route wrote its hidden values,
+                             //           the source wrote it as a duplicate the saved plan agrees with
     uint64_t *parentTag;     // dispatch: epoch << 32 | primary row + 1 when the row is a duplicate
     uint32_t *sibling;       // dispatch, fresh plans: rank among the duplicates of its primary | count << 16
     uint64_t *groupStart;    // dispatch, fresh plans: epoch << 32 | first dupLoffs index of the primary's group
-    uint64_t *dupMask;       // combine: epoch << 32 | 1 when the row is a duplicate
-    uint64_t *groupOf;       // combine: epoch << 32 | group index + 1 when the row is a primary with duplicates
-    uint64_t *slotSrc;       // combine: [world][n] epoch << 32 | duplicate << 31 | expert rank * nvS + row
+    uint64_t *slotSrc;       // combine: per origin slot, epoch << 32 | expert rank * nvS + row of the row returned to it
+    uint64_t *slotDup;       // combine: per origin slot, epoch << 32 | 1 when that row is a duplicate (it does not travel)
+    uint64_t *slotGroup;     // combine: per origin slot, epoch << 32 | first dupLoffs index when that row has duplicates
+    int32_t *slotCount;      // combine: per origin slot, number of those duplicates (valid with slotGroup)
     uint64_t *fail;          // [world] epoch << 32 | device status of the rank's own failure
-    int32_t *workList;       // dispatch: [world][nvS] rows the fill kernel has to write, grouped by classify group
+    int32_t *workList;       // dispatch: rows the fill kernel has to write, grouped by classify group
     int32_t *workCount;      // dispatch: [world][groups]
-    int64_t stride;          // >= nvS and >= n
+    int32_t *chunkTotals;    // dispatch, fresh plans: [world][groups][2] group-opening rows and duplicates per 2048 rows
+    int64_t stride;          // >= nvS and >= n, a multiple of kRowsPerGroup
     int64_t groupStride;     // classify groups per rank
 };
 
-struct ReceiveTable {
-    void *hidden[kMaxWorld];       // hiddenNvsh of every rank
-    float *weights[kMaxWorld];     // routeWeightsNvs of every rank (all null when weights are not exchanged)
-};
-
-struct ScatterLaunch {
-    const int32_t *dst;            // [s * k]
-    const void *hiddenSh;          // [s, h] bf16
-    const float *weightsSk;        // [s * k] or null
+// One Dispatch of every rank of a world.
+struct DispatchWorld {
+    int world;
     int64_t s, k, h, nvS;
+    bool fresh;                                // the duplicate plan is built by this call
+    uint64_t epoch;
+    WorldTables tables;
+    const int32_t *dst[kMaxWorld];             // [s * k] route words
+    const void *hiddenSh[kMaxWorld];           // [s, h] bf16
+    const float *weightsSk[kMaxWorld];         // [s * k], or all null
+    void *hiddenNvsh[kMaxWorld];               // out [nvS, h] bf16
+    float *weightsNvs[kMaxWorld];              // out [nvS]
+    int32_t *dupGroups[kMaxWorld];             // [nvS, 3]  out when fresh, else in
+    int32_t *dupLoffs[kMaxWorld];              // [nvS]
+    int32_t *dupCounts[kMaxWorld];             // [2]
+    int32_t *status[kMaxWorld];
+};
+
+// One Combine of every rank of a world.
+struct CombineWorld {
     int world;
-    int srcRank;
-    bool fresh;                    // the duplicate plan is being built: duplicates are written here, with records
-    ReceiveTable out;
-    WorldTables tables;
+    int64_t s, k, h, nvS;
     uint64_t epoch;
-    hipStream_t stream;
-};
-
-struct DedupBuildLaunch {
-    int64_t nvS;
-    int rank;
     WorldTables tables;
-    uint64_t epoch;
-    int32_t *dupGroups;            // out [nvS, 3]
-    int32_t *dupLoffs;             // out [nvS]
-    int32_t *dupCounts;            // out [2]
-    hipStream_t stream;
-};
-
-struct GroupWalkLaunch {
-    int64_t nvS;
-    int rank;
-    bool combine;                  // fills dupMask / groupOf and rejects duplicate == primary; else fills parentTag
-    const int32_t *dupGroups;
-    const int32_t *dupLoffs;
-    const int32_t *dupCounts;
-    WorldTables tables;
-    uint64_t epoch;
-    hipStream_t stream;
-};
-
-struct FillLaunch {
-    int64_t nvS, h;
-    int world;
-    int rank;
-    bool expand;                   // saved plan: duplicate rows take a copy of their primary row
-    void *hiddenNvsh;
-    float *weightsNvs;             // or null
-    WorldTables tables;
-    uint64_t epoch;
-    int32_t *status;               // plan->status
-    hipStream_t stream;
-};
-
-struct ReverseLaunch {
-    const int32_t *dstLocal;       // [nvS]
-    int64_t nvS, n;
-    int world;
-    int rank;
-    WorldTables tables;
-    uint64_t epoch;
-    hipStream_t stream;
-};
-
-struct SourceTable {
-    const void *hidden[kMaxWorld];         // hiddenNvsh of every expert rank
-    const float *weights[kMaxWorld];       // routeWeightsNvs of every expert rank, or null
+    const int32_t *dstLocal[kMaxWorld];        // [nvS]
+    const void *hiddenNvsh[kMaxWorld];         // [nvS, h] bf16
+    const float *weightsNvs[kMaxWorld];        // [nvS], or all null
     const int32_t *dupGroups[kMaxWorld];
     const int32_t *dupLoffs[kMaxWorld];
+    const int32_t *dupCounts[kMaxWorld];
+    void *hiddenSh[kMaxWorld];                 // out [s, h] bf16
+    float *weightsSk[kMaxWorld];               // out [s * k]
+    int32_t *status[kMaxWorld];
 };
 
-struct MoonReduceLaunch {
-    int64_t s, k, h, nvS;
-    int world;
-    int rank;
-    SourceTable src;
-    WorldTables tables;
-    uint64_t epoch;
-    void *hiddenSh;                // out [s, h] bf16
-    float *weightsSk;              // out [s * k] or null
-    int32_t *status;
-    int numComputeUnits;
-    hipStream_t stream;
+// Optional (start, stop) events recorded around the scatter / reduce launch.
+struct LaunchTiming {
+    hipEvent_t start = nullptr;
+    hipEvent_t stop = nullptr;
 };
 
-hipError_t LaunchMoonScatter(const ScatterLaunch &l);
-hipError_t LaunchMoonDedupBuild(const DedupBuildLaunch &l);
-hipError_t LaunchMoonGroupWalk(const GroupWalkLaunch &l);
-hipError_t LaunchMoonFill(const FillLaunch &l);
-hipError_t LaunchMoonReverse(const ReverseLaunch &l);
-hipError_t LaunchMoonReduce(const MoonReduceLaunch &l);
+hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const LaunchTiming &scatterTiming);
+hipError_t LaunchMoonCombine(const CombineWorld &w, hipStream_t stream, const LaunchTiming &reduceTiming);
 
 // Names of the kernel templates the last scatter / reduce launch used (for the benchmark's roofline line).
 const char *MoonScatterKernelName();

@@ -4,6 +4,7 @@
 // count: dispatch is one read of each token row and one write per route; combine is one read per route and one write
 // per token.  Row copies use two 16-byte loads and two 16-byte stores per lane, and the workgroups of one token are
 // given block indices that land on one XCD (block b runs on XCD b % 8) so the token row is read from HBM once.
+// Every kernel is launched once for the whole world: blockIdx.y is the rank whose share the workgroup works on.
 //
 //   what is computed  reference: src/moonep/dispatch/kernels/tilexr_moonep_dispatch_kernel.cpp:108-147, 268-461
 //                                src/moonep/combine/kernels/tilexr_moonep_combine_kernel.cpp:117-177, 285-366, 449-541,
@@ -37,9 +38,11 @@ __device__ __forceinline__ uint64_t Tag(uint64_t epoch, uint32_t value)
     return (epoch << 32) | value;
 }
 
-// Row tag values: a route names the row (its weight is written); a route also wrote the row's hidden values.
-constexpr uint32_t kRowNamed = 2u;
-constexpr uint32_t kRowWritten = 1u;
+// Row tag bits.
+constexpr uint32_t kRowWritten = 1u;    // a route wrote the row's hidden values
+constexpr uint32_t kRowNamed = 2u;      // a route names the row: its weight is written
+constexpr uint32_t kRowDirect = 4u;     // saved plan: a duplicate whose primary is a row of the same token, written by
+                                        // the source like a fresh duplicate
 
 // reference: dispatch kernel :268-279
 struct Route {
@@ -70,19 +73,23 @@ __device__ __forceinline__ void RecordFailure(const WorldTables &t, int rank, ui
 // ---------------------------------------------------------------------------------------------------------------
 // dispatch: scatter
 // ---------------------------------------------------------------------------------------------------------------
-struct ScatterArgs {
-    const int32_t *dst;
-    const void *hiddenSh;
-    const float *weightsSk;
-    int s, k, h;
-    int64_t nvS;
-    int world;
-    int srcRank;
-    int colSlices;
-    ReceiveTable out;
-    WorldTables t;
-    uint64_t epoch;
-};
+
+// Row of the first non-duplicate route of the token, before route k, that goes to `peer`; -1 when there is none.
+// reference: dispatch kernel :281-301
+__device__ __forceinline__ int OwnPrimaryRow(const DispatchWorld &a, const int32_t *words, int k, int peer)
+{
+    for (int j = 0; j < k; ++j) {
+        const int32_t e = words[j];
+        if (e < 0) {
+            continue;
+        }
+        const Route o = Decode(e, a.nvS, a.world);
+        if (o.ok && o.peer == peer) {
+            return o.row;
+        }
+    }
+    return -1;
+}
 
 // What the route's first workgroup records besides the row: the weight, the row tag and -- while the duplicate plan is
 // being built -- which primary a duplicate belongs to and where it stands among that primary's duplicates.  Called by
@@ -91,15 +98,16 @@ struct ScatterArgs {
 //   the plan lists a primary's duplicates in ascending row order (dispatch kernel :393-419), so the rank of a
 //   duplicate within its group is the number of the token's duplicates to that rank with a smaller row
 template <bool FRESH>
-__device__ __forceinline__ void RouteRecords(const ScatterArgs &a, int token, int k, const Route &r, const int32_t *s_dst)
+__device__ __forceinline__ void RouteRecords(const DispatchWorld &a, int src, int token, int k, const Route &r, uint32_t tagBits,
+    const int32_t *s_dst)
 {
     const int lane = threadIdx.x;
-    const int64_t at = static_cast<int64_t>(r.peer) * a.t.stride + r.row;
+    const int64_t at = static_cast<int64_t>(r.peer) * a.tables.stride + r.row;
     if (lane == 0) {
-        if (a.weightsSk != nullptr) {
-            a.out.weights[r.peer][r.row] = a.weightsSk[static_cast<int64_t>(token) * a.k + k];
+        if (a.weightsSk[src] != nullptr) {
+            a.weightsNvs[r.peer][r.row] = a.weightsSk[src][static_cast<int64_t>(token) * a.k + k];
         }
-        a.t.rowTag[at] = Tag(a.epoch, (FRESH || !r.duplicate) ? (kRowNamed | kRowWritten) : kRowNamed);
+        a.tables.rowTag[at] = Tag(a.epoch, tagBits);
     }
     if (!FRESH || !r.duplicate) {
         return;
@@ -114,61 +122,84 @@ __device__ __forceinline__ void RouteRecords(const ScatterArgs &a, int token, in
     const uint64_t before = __ballot(samePeer && other.duplicate && other.row < r.row);
     if (primaries == 0) {
         if (lane == 0) {
-            RecordFailure(a.t, a.srcRank, a.epoch, kDispatchInvalidRoute);
+            RecordFailure(a.tables, src, a.epoch, kDispatchInvalidRoute);
         }
         return;
     }
     const int primaryLane = __ffsll(static_cast<unsigned long long>(primaries)) - 1;
     const int primaryRow = __shfl(other.row, primaryLane);
     if (lane == 0) {
-        a.t.parentTag[at] = Tag(a.epoch, static_cast<uint32_t>(primaryRow) + 1u);
-        a.t.sibling[at] = static_cast<uint32_t>(__popcll(before)) | (static_cast<uint32_t>(__popcll(siblings)) << 16);
+        a.tables.parentTag[at] = Tag(a.epoch, static_cast<uint32_t>(primaryRow) + 1u);
+        a.tables.sibling[at] = static_cast<uint32_t>(__popcll(before)) | (static_cast<uint32_t>(__popcll(siblings)) << 16);
     }
 }
 
-// One workgroup per (token, route, slice of 512 vectors).  FRESH: the duplicate plan is being built from these very
-// route words, so a duplicate row is by construction a copy of this token's row and is written here; otherwise
-// duplicate rows are left to the fill kernel, which copies them from the primary the saved plan names.
+// Whether the source writes the row of this route, and the tag the row gets.
+//   fresh plan   every route: the plan is being built from these very route words, so a duplicate row is by construction
+//                a copy of this token's row
+//   saved plan   non-duplicates; and a duplicate whose primary, according to the plan (parent records written by the walk
+//                kernel), is the row this token's own non-duplicate route to that rank writes -- the copy the fill kernel
+//                would make is a copy of this token's row.  Any other duplicate is left to the fill kernel.
 template <bool FRESH>
-__global__ __launch_bounds__(kThreads) void moon_scatter_kernel(ScatterArgs a)
+__device__ __forceinline__ bool SourceWrites(const DispatchWorld &a, const int32_t *words, int k, const Route &r, uint32_t *tagBits)
+{
+    if (FRESH || !r.duplicate) {
+        *tagBits = kRowNamed | kRowWritten;
+        return true;
+    }
+    const uint64_t p = a.tables.parentTag[static_cast<int64_t>(r.peer) * a.tables.stride + r.row];
+    if (Tagged(p, a.epoch) && static_cast<int>(p & 0xffffffffu) - 1 == OwnPrimaryRow(a, words, k, r.peer)) {
+        *tagBits = kRowNamed | kRowWritten | kRowDirect;
+        return true;
+    }
+    *tagBits = kRowNamed;
+    return false;
+}
+
+// One workgroup per (token, route, slice of 512 vectors) of source rank blockIdx.y.
+template <bool FRESH>
+__global__ __launch_bounds__(kThreads) void moon_scatter_kernel(DispatchWorld a, int colSlices)
 {
     __shared__ int32_t s_dst[kMaxTopK];
+    const int src = blockIdx.y;
     const int xcd = blockIdx.x % kXcds;
     const int j = blockIdx.x / kXcds;
-    const int perToken = a.k * a.colSlices;
+    const int K = static_cast<int>(a.k);
+    const int perToken = K * colSlices;
     const int token = (j / perToken) * kXcds + xcd;
-    const int k = (j % perToken) / a.colSlices;
-    const int slice = (j % perToken) % a.colSlices;
+    const int k = (j % perToken) / colSlices;
+    const int slice = (j % perToken) % colSlices;
     if (token >= a.s) {
         return;
     }
     const int lane = threadIdx.x;
-    const int vecs = a.h / 8;
+    const int h = static_cast<int>(a.h);
+    const int vecs = h / 8;
     const int colBase = slice * (kRowVecs * kThreads);
-    const int32_t *words = a.dst + static_cast<int64_t>(token) * a.k;
+    const int32_t *words = a.dst[src] + static_cast<int64_t>(token) * K;
     const bool records = slice == 0;
-    if (FRESH && records && lane < a.k) {
+    if (FRESH && records && lane < K) {
         s_dst[lane] = words[lane];
     }
     const int32_t encoded = words[k];
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.hiddenSh) +
-        static_cast<int64_t>(token) * a.h * 2);
+    const u32x4 *srcRow = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.hiddenSh[src]) +
+        static_cast<int64_t>(token) * h * 2);
     u32x4 v[kRowVecs];
 #pragma unroll
     for (int i = 0; i < kRowVecs; ++i) {
         const int idx = colBase + i * kThreads + lane;
-        v[i] = idx < vecs ? src[idx] : u32x4{0u, 0u, 0u, 0u};
+        v[i] = idx < vecs ? srcRow[idx] : u32x4{0u, 0u, 0u, 0u};
     }
     const Route r = Decode(encoded, a.nvS, a.world);
     if (!r.ok) {
         if (records && lane == 0) {
-            RecordFailure(a.t, a.srcRank, a.epoch, kDispatchInvalidRoute);
+            RecordFailure(a.tables, src, a.epoch, kDispatchInvalidRoute);
         }
         return;
     }
-    if (FRESH || !r.duplicate) {
-        u32x4 *dstRow = reinterpret_cast<u32x4 *>(static_cast<char *>(a.out.hidden[r.peer]) +
-            static_cast<int64_t>(r.row) * a.h * 2);
+    uint32_t tagBits = 0;
+    if (SourceWrites<FRESH>(a, words, k, r, &tagBits)) {
+        u32x4 *dstRow = reinterpret_cast<u32x4 *>(static_cast<char *>(a.hiddenNvsh[r.peer]) + static_cast<int64_t>(r.row) * h * 2);
 #pragma unroll
         for (int i = 0; i < kRowVecs; ++i) {
             const int idx = colBase + i * kThreads + lane;
@@ -182,177 +213,197 @@ __global__ __launch_bounds__(kThreads) void moon_scatter_kernel(ScatterArgs a)
             TileXREp::LdsBarrier();
         }
         if (lane < kWave) {
-            RouteRecords<FRESH>(a, token, k, r, s_dst);
+            RouteRecords<FRESH>(a, src, token, k, r, tagBits, s_dst);
         }
     }
 }
 
 // Any hidden size and alignment: one workgroup per route, 2-byte elements.
 template <bool FRESH>
-__global__ __launch_bounds__(kThreads) void moon_scatter_generic_kernel(ScatterArgs a)
+__global__ __launch_bounds__(kThreads) void moon_scatter_generic_kernel(DispatchWorld a)
 {
     __shared__ int32_t s_dst[kMaxTopK];
-    const int token = blockIdx.x / a.k;
-    const int k = blockIdx.x % a.k;
+    const int src = blockIdx.y;
+    const int K = static_cast<int>(a.k);
+    const int token = blockIdx.x / K;
+    const int k = blockIdx.x % K;
     const int lane = threadIdx.x;
-    const int32_t *words = a.dst + static_cast<int64_t>(token) * a.k;
-    if (FRESH && lane < a.k) {
+    const int32_t *words = a.dst[src] + static_cast<int64_t>(token) * K;
+    if (FRESH && lane < K) {
         s_dst[lane] = words[lane];
     }
     const Route r = Decode(words[k], a.nvS, a.world);
     if (!r.ok) {
         if (lane == 0) {
-            RecordFailure(a.t, a.srcRank, a.epoch, kDispatchInvalidRoute);
+            RecordFailure(a.tables, src, a.epoch, kDispatchInvalidRoute);
         }
         return;
     }
-    if (FRESH || !r.duplicate) {
-        const uint16_t *src = static_cast<const uint16_t *>(a.hiddenSh) + static_cast<int64_t>(token) * a.h;
-        uint16_t *dstRow = static_cast<uint16_t *>(a.out.hidden[r.peer]) + static_cast<int64_t>(r.row) * a.h;
+    uint32_t tagBits = 0;
+    if (SourceWrites<FRESH>(a, words, k, r, &tagBits)) {
+        const uint16_t *srcRow = static_cast<const uint16_t *>(a.hiddenSh[src]) + static_cast<int64_t>(token) * a.h;
+        uint16_t *dstRow = static_cast<uint16_t *>(a.hiddenNvsh[r.peer]) + static_cast<int64_t>(r.row) * a.h;
         for (int c = lane; c < a.h; c += kThreads) {
-            dstRow[c] = src[c];
+            dstRow[c] = srcRow[c];
         }
     }
     if (FRESH) {
         TileXREp::LdsBarrier();
     }
     if (lane < kWave) {
-        RouteRecords<FRESH>(a, token, k, r, s_dst);
+        RouteRecords<FRESH>(a, src, token, k, r, tagBits, s_dst);
     }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// dispatch: duplicate plan of one destination rank from the parent records (fresh plans)
+// dispatch: duplicate plan of every destination rank from the parent records (fresh plans)
 // ---------------------------------------------------------------------------------------------------------------
-struct BuildArgs {
-    int64_t nvS;
-    int rank;
-    WorldTables t;
-    uint64_t epoch;
-    int32_t *dupGroups;
-    int32_t *dupLoffs;
-    int32_t *dupCounts;
-};
 
 // The reference scans the destination's rows in ascending order: a group is opened by the first duplicate row of its
 // primary, groups take their dupLoffs slices in that order, and each slice lists its duplicates in ascending row order
 // (dispatch kernel :330-424).  With the rank-within-group and group size recorded by the sources, both numberings are
 // exclusive prefix sums over the rows: group index = number of earlier group-opening rows, slice start = sum of their
-// group sizes.  One workgroup walks the rows 2048 at a time with a running carry.
+// group sizes.  Two launches: totals of every chunk of 2048 rows, then group records (a workgroup adds up the totals of
+// the chunks before its own, then scans its chunk).  The slices are filled by the classify kernel, which visits every
+// row anyway.
 constexpr int kBuildRows = 2048;
-__global__ __launch_bounds__(kThreads) void moon_dedup_build_kernel(BuildArgs a)
+constexpr int kBuildPer = kBuildRows / kThreads;
+
+struct ChunkRows {
+    int opens[kBuildPer];
+    int sizes[kBuildPer];
+    int primaries[kBuildPer];
+    int localOpen;
+    int localSize;
+};
+
+__device__ __forceinline__ ChunkRows LoadChunkRows(const DispatchWorld &a, int rank, int64_t base)
 {
-    constexpr int kPer = kBuildRows / kThreads;
+    const uint64_t *parent = a.tables.parentTag + static_cast<int64_t>(rank) * a.tables.stride;
+    const uint32_t *sibling = a.tables.sibling + static_cast<int64_t>(rank) * a.tables.stride;
+    ChunkRows c;
+    c.localOpen = 0;
+    c.localSize = 0;
+#pragma unroll
+    for (int i = 0; i < kBuildPer; ++i) {
+        const int64_t row = base + static_cast<int64_t>(threadIdx.x) * kBuildPer + i;
+        c.opens[i] = 0;
+        c.sizes[i] = 0;
+        c.primaries[i] = -1;
+        if (row < a.nvS) {
+            const uint64_t p = parent[row];
+            if (Tagged(p, a.epoch)) {
+                const uint32_t sib = sibling[row];
+                c.primaries[i] = static_cast<int>(p & 0xffffffffu) - 1;
+                c.opens[i] = (sib & 0xffffu) == 0 ? 1 : 0;
+                c.sizes[i] = c.opens[i] ? static_cast<int>(sib >> 16) : 0;
+            }
+        }
+        c.localOpen += c.opens[i];
+        c.localSize += c.sizes[i];
+    }
+    return c;
+}
+
+// Exclusive prefix of (open, size) over the threads of the workgroup, and the workgroup totals.
+__device__ __forceinline__ void ScanPair(int localOpen, int localSize, int (*s_part)[kThreads / kWave], int *exclOpen,
+    int *exclSize, int *totalOpen, int *totalSize)
+{
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave;
+    int inclOpen = localOpen;
+    int inclSize = localSize;
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+        const int upOpen = __shfl_up(inclOpen, off);
+        const int upSize = __shfl_up(inclSize, off);
+        inclOpen += lane >= off ? upOpen : 0;
+        inclSize += lane >= off ? upSize : 0;
+    }
+    if (lane == kWave - 1) {
+        s_part[0][wave] = inclOpen;
+        s_part[1][wave] = inclSize;
+    }
+    __syncthreads();
+    *exclOpen = inclOpen - localOpen;
+    *exclSize = inclSize - localSize;
+    *totalOpen = 0;
+    *totalSize = 0;
+#pragma unroll
+    for (int w = 0; w < kThreads / kWave; ++w) {
+        *exclOpen += w < wave ? s_part[0][w] : 0;
+        *exclSize += w < wave ? s_part[1][w] : 0;
+        *totalOpen += s_part[0][w];
+        *totalSize += s_part[1][w];
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void moon_dedup_totals_kernel(DispatchWorld a)
+{
     __shared__ int s_part[2][kThreads / kWave];
-    __shared__ int s_carry[2];
+    const int rank = blockIdx.y;
+    const ChunkRows c = LoadChunkRows(a, rank, static_cast<int64_t>(blockIdx.x) * kBuildRows);
+    int exclOpen, exclSize, totalOpen, totalSize;
+    ScanPair(c.localOpen, c.localSize, s_part, &exclOpen, &exclSize, &totalOpen, &totalSize);
+    if (threadIdx.x == 0) {
+        int32_t *totals = a.tables.chunkTotals + (static_cast<int64_t>(rank) * a.tables.groupStride + blockIdx.x) * 2;
+        totals[0] = totalOpen;
+        totals[1] = totalSize;
+    }
+}
+
+__global__ __launch_bounds__(kThreads) void moon_dedup_groups_kernel(DispatchWorld a)
+{
+    __shared__ int s_part[2][kThreads / kWave];
+    __shared__ int s_base[2];
+    const int rank = blockIdx.y;
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
-    const uint64_t *parent = a.t.parentTag + static_cast<int64_t>(a.rank) * a.t.stride;
-    const uint32_t *sibling = a.t.sibling + static_cast<int64_t>(a.rank) * a.t.stride;
-    uint64_t *groupStart = a.t.groupStart + static_cast<int64_t>(a.rank) * a.t.stride;
+    const int32_t *totals = a.tables.chunkTotals + static_cast<int64_t>(rank) * a.tables.groupStride * 2;
+    // totals of the chunks before this one
+    int beforeOpen = 0;
+    int beforeSize = 0;
+    for (int c = tid; c < static_cast<int>(blockIdx.x); c += kThreads) {
+        beforeOpen += totals[2 * c];
+        beforeSize += totals[2 * c + 1];
+    }
+    int exclOpen, exclSize, baseOpen, baseSize;
+    ScanPair(beforeOpen, beforeSize, s_part, &exclOpen, &exclSize, &baseOpen, &baseSize);
     if (tid == 0) {
-        s_carry[0] = 0;
-        s_carry[1] = 0;
+        s_base[0] = baseOpen;
+        s_base[1] = baseSize;
     }
     __syncthreads();
-    for (int64_t base = 0; base < a.nvS; base += kBuildRows) {
-        int opens[kPer];
-        int sizes[kPer];
-        int primaries[kPer];
-        int localOpen = 0;
-        int localSize = 0;
+    const ChunkRows c = LoadChunkRows(a, rank, static_cast<int64_t>(blockIdx.x) * kBuildRows);
+    int totalOpen, totalSize;
+    ScanPair(c.localOpen, c.localSize, s_part, &exclOpen, &exclSize, &totalOpen, &totalSize);
+    int group = s_base[0] + exclOpen;
+    int start = s_base[1] + exclSize;
+    uint64_t *groupStart = a.tables.groupStart + static_cast<int64_t>(rank) * a.tables.stride;
 #pragma unroll
-        for (int i = 0; i < kPer; ++i) {
-            const int64_t row = base + tid * kPer + i;
-            opens[i] = 0;
-            sizes[i] = 0;
-            primaries[i] = -1;
-            if (row < a.nvS) {
-                const uint64_t p = parent[row];
-                if (Tagged(p, a.epoch)) {
-                    const uint32_t sib = sibling[row];
-                    primaries[i] = static_cast<int>(p & 0xffffffffu) - 1;
-                    opens[i] = (sib & 0xffffu) == 0 ? 1 : 0;
-                    sizes[i] = opens[i] ? static_cast<int>(sib >> 16) : 0;
-                }
-            }
-            localOpen += opens[i];
-            localSize += sizes[i];
-        }
-        int inclOpen = localOpen;
-        int inclSize = localSize;
-#pragma unroll
-        for (int off = 1; off < kWave; off <<= 1) {
-            const int upOpen = __shfl_up(inclOpen, off);
-            const int upSize = __shfl_up(inclSize, off);
-            inclOpen += lane >= off ? upOpen : 0;
-            inclSize += lane >= off ? upSize : 0;
-        }
-        if (lane == kWave - 1) {
-            s_part[0][wave] = inclOpen;
-            s_part[1][wave] = inclSize;
-        }
-        __syncthreads();
-        int group = s_carry[0] + inclOpen - localOpen;
-        int start = s_carry[1] + inclSize - localSize;
-        int totalOpen = 0;
-        int totalSize = 0;
-#pragma unroll
-        for (int w = 0; w < kThreads / kWave; ++w) {
-            group += w < wave ? s_part[0][w] : 0;
-            start += w < wave ? s_part[1][w] : 0;
-            totalOpen += s_part[0][w];
-            totalSize += s_part[1][w];
-        }
-#pragma unroll
-        for (int i = 0; i < kPer; ++i) {
-            if (opens[i]) {
-                int32_t *g = a.dupGroups + static_cast<int64_t>(group) * 3;
-                g[0] = primaries[i];
+    for (int i = 0; i < kBuildPer; ++i) {
+        if (c.opens[i]) {
+            // a plan in which duplicates of one token name the same row can claim more slots than there are rows
+            if (group < a.nvS && static_cast<int64_t>(start) + c.sizes[i] <= a.nvS) {
+                int32_t *g = a.dupGroups[rank] + static_cast<int64_t>(group) * 3;
+                g[0] = c.primaries[i];
                 g[1] = start;
-                g[2] = sizes[i];
-                __hip_atomic_store(&groupStart[primaries[i]], Tag(a.epoch, static_cast<uint32_t>(start)), __ATOMIC_RELAXED,
-                    __HIP_MEMORY_SCOPE_AGENT);
-                group += 1;
-                start += sizes[i];
-            }
-        }
-        __syncthreads();
-        if (tid == 0) {
-            s_carry[0] += totalOpen;
-            s_carry[1] += totalSize;
-        }
-        __syncthreads();
-    }
-    if (tid == 0) {
-        a.dupCounts[0] = s_carry[0];
-        a.dupCounts[1] = s_carry[1];
-    }
-    // every group start is written: make the stores complete before any lane of this workgroup reads them back
-    TileXREp::WaitOwnStores();
-    __syncthreads();
-    for (int64_t row = tid; row < a.nvS; row += kThreads) {
-        const uint64_t p = parent[row];
-        if (!Tagged(p, a.epoch)) {
-            continue;
-        }
-        const int primary = static_cast<int>(p & 0xffffffffu) - 1;
-        const uint64_t gs = __hip_atomic_load(&groupStart[primary], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (Tagged(gs, a.epoch)) {
-            // a plan in which two duplicates of a token name the same row can claim more slots than there are rows
-            const int64_t at = static_cast<int64_t>(gs & 0xffffffffu) + (sibling[row] & 0xffffu);
-            if (at < a.nvS) {
-                a.dupLoffs[at] = static_cast<int32_t>(row);
+                g[2] = c.sizes[i];
+                groupStart[c.primaries[i]] = Tag(a.epoch, static_cast<uint32_t>(start));
             } else {
-                RecordFailure(a.t, a.rank, a.epoch, kDispatchInvalidRoute);
+                RecordFailure(a.tables, rank, a.epoch, kDispatchInvalidRoute);
             }
+            group += 1;
+            start += c.sizes[i];
         }
+    }
+    if (blockIdx.x == gridDim.x - 1 && tid == 0) {
+        a.dupCounts[rank][0] = s_base[0] + totalOpen;
+        a.dupCounts[rank][1] = s_base[1] + totalSize;
     }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// saved duplicate plan -> per-row records (dispatch: parentTag; combine: dupMask and groupOf)
+// saved duplicate plan -> records the later kernels follow (dispatch: parentTag per row; combine: per-slot tables)
 // ---------------------------------------------------------------------------------------------------------------
 struct WalkArgs {
     int64_t nvS;
@@ -363,21 +414,38 @@ struct WalkArgs {
     const int32_t *dupCounts;
     WorldTables t;
     uint64_t epoch;
+    const int32_t *dstLocal;     // combine only
+    int world;
+    int64_t n;
 };
 
+// Slot (origin rank * stride + target) a receive row returns to, or -1 (reference: combine kernel :285-298).
+__device__ __forceinline__ int64_t SlotOfRow(const WalkArgs &a, int32_t row)
+{
+    const int32_t encoded = a.dstLocal[row];
+    if (encoded < 0) {
+        return -1;
+    }
+    const int64_t peer = encoded / a.nvS;
+    const int64_t target = encoded % a.nvS;
+    if (peer >= a.world || target >= a.n) {
+        return -1;
+    }
+    return peer * a.t.stride + target;
+}
+
 // One thread per group.  Checks follow the reference (dispatch kernel :428-457, combine kernel :307-345).
-__global__ __launch_bounds__(kThreads) void moon_group_walk_kernel(WalkArgs a)
+__device__ __forceinline__ void WalkGroup(const WalkArgs &a, int64_t g)
 {
     const int32_t groupCount = a.dupCounts[0];
     const int32_t duplicateCount = a.dupCounts[1];
     const int32_t invalid = a.combine ? kCombineInvalidRoute : kDispatchInvalidRoute;
     if (groupCount < 0 || groupCount > a.nvS || duplicateCount < 0 || duplicateCount > a.nvS) {
-        if (blockIdx.x == 0 && threadIdx.x == 0) {
+        if (g == 0) {
             RecordFailure(a.t, a.rank, a.epoch, invalid);
         }
         return;
     }
-    const int64_t g = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (g >= groupCount) {
         return;
     }
@@ -389,7 +457,7 @@ __global__ __launch_bounds__(kThreads) void moon_group_walk_kernel(WalkArgs a)
         return;
     }
     const int64_t base = static_cast<int64_t>(a.rank) * a.t.stride;
-    // nothing is recorded for a group with a bad entry: the reduce kernel follows these records without checking them
+    // nothing is recorded for a group with a bad entry: the kernels that follow these records do not check them again
     for (int32_t i = 0; i < count; ++i) {
         const int32_t dup = a.dupLoffs[start + i];
         if (dup < 0 || dup >= a.nvS || (a.combine && dup == primary)) {
@@ -398,33 +466,36 @@ __global__ __launch_bounds__(kThreads) void moon_group_walk_kernel(WalkArgs a)
         }
     }
     if (a.combine) {
-        a.t.groupOf[base + primary] = Tag(a.epoch, static_cast<uint32_t>(g) + 1u);
+        // the origin reads these per slot, next to the slot's row, so that one round trip tells it everything
+        const int64_t slot = SlotOfRow(a, primary);
+        if (slot >= 0) {
+            a.t.slotCount[slot] = count;
+            a.t.slotGroup[slot] = Tag(a.epoch, static_cast<uint32_t>(start));
+        }
     }
     for (int32_t i = 0; i < count; ++i) {
         const int32_t dup = a.dupLoffs[start + i];
         if (a.combine) {
-            a.t.dupMask[base + dup] = Tag(a.epoch, 1u);
+            const int64_t slot = SlotOfRow(a, dup);
+            if (slot >= 0) {
+                a.t.slotDup[slot] = Tag(a.epoch, 1u);
+            }
         } else {
             a.t.parentTag[base + dup] = Tag(a.epoch, static_cast<uint32_t>(primary) + 1u);
         }
     }
 }
 
+__global__ __launch_bounds__(kThreads) void moon_group_walk_kernel(DispatchWorld a)
+{
+    const int rank = blockIdx.y;
+    WalkArgs w {a.nvS, rank, false, a.dupGroups[rank], a.dupLoffs[rank], a.dupCounts[rank], a.tables, a.epoch, nullptr, a.world, 0};
+    WalkGroup(w, static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x);
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // dispatch: rows nobody wrote
 // ---------------------------------------------------------------------------------------------------------------
-struct FillArgs {
-    int64_t nvS;
-    int h;
-    int world;
-    int rank;
-    bool expand;
-    void *hiddenNvsh;
-    float *weightsNvs;
-    WorldTables t;
-    uint64_t epoch;
-    int32_t *status;
-};
 
 // Work item of the fill kernel: row | kind << 30.
 constexpr int32_t kFillZero = 0;
@@ -432,29 +503,45 @@ constexpr int32_t kFillCopy = 1;
 
 // One thread per row decides what is left to do for it: nothing (a route wrote it), zeros (no route wrote it: the
 // reference clears the whole window first, dispatch kernel :206-230), or -- saved plans -- a copy of its primary row
-// (dispatch kernel :426-461).  The weight of a row no route names is zero for the same reason.  Each workgroup packs its rows' work items into its own segment of the work list, so
-// nothing has to be reset between calls.  Workgroup 0 also writes the device status.
-__global__ __launch_bounds__(kRowsPerGroup) void moon_classify_kernel(FillArgs a)
+// (dispatch kernel :426-461).  The weight of a row no route names is zero for the same reason.  Each workgroup packs its
+// rows' work items into its own segment of the work list, so nothing has to be reset between calls.  The duplicates of a
+// fresh plan also take their places in dupLoffs here, and workgroup 0 of every rank writes the rank's device status.
+__global__ __launch_bounds__(kRowsPerGroup) void moon_classify_kernel(DispatchWorld a)
 {
     __shared__ int s_waveCount[kRowsPerGroup / kWave];
+    const int rank = blockIdx.y;
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    const int64_t base = static_cast<int64_t>(a.rank) * a.t.stride;
+    const int64_t base = static_cast<int64_t>(rank) * a.tables.stride;
     const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerGroup + tid;
     int32_t item = -1;
     if (row < a.nvS) {
-        const uint64_t tag = a.t.rowTag[base + row];
-        const bool named = Tagged(tag, a.epoch) && (tag & kRowNamed) != 0;
-        const bool written = Tagged(tag, a.epoch) && (tag & kRowWritten) != 0;
-        const uint64_t p = a.t.parentTag[base + row];
-        if (a.expand && Tagged(p, a.epoch)) {
+        const uint64_t tag = a.tables.rowTag[base + row];
+        const bool tagged = Tagged(tag, a.epoch);
+        const bool named = tagged && (tag & kRowNamed) != 0;
+        const bool written = tagged && (tag & kRowWritten) != 0;
+        const bool direct = tagged && (tag & kRowDirect) != 0;
+        const uint64_t p = a.tables.parentTag[base + row];
+        if (!a.fresh && Tagged(p, a.epoch) && !direct) {
             item = static_cast<int32_t>(row) | (kFillCopy << 30);
         } else if (!written) {
             item = static_cast<int32_t>(row) | (kFillZero << 30);
         }
-        if (!named && a.weightsNvs != nullptr) {
-            a.weightsNvs[row] = 0.0f;
+        if (!named && a.weightsNvs[rank] != nullptr) {
+            a.weightsNvs[rank][row] = 0.0f;
+        }
+        if (a.fresh && Tagged(p, a.epoch)) {
+            // slot of this duplicate in its group's slice (dispatch kernel :393-419)
+            const uint64_t gs = a.tables.groupStart[base + static_cast<int64_t>(p & 0xffffffffu) - 1];
+            if (Tagged(gs, a.epoch)) {
+                const int64_t at = static_cast<int64_t>(gs & 0xffffffffu) + (a.tables.sibling[base + row] & 0xffffu);
+                if (at < a.nvS) {
+                    a.dupLoffs[rank][at] = static_cast<int32_t>(row);
+                } else {
+                    RecordFailure(a.tables, rank, a.epoch, kDispatchInvalidRoute);
+                }
+            }
         }
     }
     const uint64_t have = __ballot(item >= 0);
@@ -471,65 +558,67 @@ __global__ __launch_bounds__(kRowsPerGroup) void moon_classify_kernel(FillArgs a
     }
     if (item >= 0) {
         const int at = before + __popcll(have & ((1ull << lane) - 1ull));
-        a.t.workList[base + static_cast<int64_t>(blockIdx.x) * kRowsPerGroup + at] = item;
+        a.tables.workList[base + static_cast<int64_t>(blockIdx.x) * kRowsPerGroup + at] = item;
     }
     if (tid == 0) {
-        a.t.workCount[static_cast<int64_t>(a.rank) * a.t.groupStride + blockIdx.x] = total;
+        a.tables.workCount[static_cast<int64_t>(rank) * a.tables.groupStride + blockIdx.x] = total;
     }
     if (blockIdx.x == 0 && tid == 0) {
         // own failure first, then the first failed peer walking upwards from this rank (dispatch kernel :559-574)
         int32_t status = kDispatchOk;
-        const uint64_t own = __hip_atomic_load(&a.t.fail[a.rank], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const uint64_t own = __hip_atomic_load(&a.tables.fail[rank], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         if (Tagged(own, a.epoch)) {
             status = static_cast<int32_t>(own & 0xffffffffu);
         } else {
             for (int o = 1; o < a.world; ++o) {
-                const int peer = (a.rank + o) % a.world;
-                const uint64_t f = __hip_atomic_load(&a.t.fail[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                const int peer = (rank + o) % a.world;
+                const uint64_t f = __hip_atomic_load(&a.tables.fail[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 if (Tagged(f, a.epoch)) {
                     status = kDispatchRemoteFailureBase + peer;
                     break;
                 }
             }
         }
-        a.status[0] = status;
+        a.status[rank][0] = status;
     }
 }
 
 // kFillSplit workgroups share the work items of one classify group; a workgroup writes whole rows.
 template <bool VEC>
-__global__ __launch_bounds__(kThreads) void moon_fill_kernel(FillArgs a)
+__global__ __launch_bounds__(kThreads) void moon_fill_kernel(DispatchWorld a)
 {
+    const int rank = blockIdx.y;
     const int group = blockIdx.x / kFillSplit;
     const int part = blockIdx.x % kFillSplit;
-    const int64_t base = static_cast<int64_t>(a.rank) * a.t.stride;
-    const int count = a.t.workCount[static_cast<int64_t>(a.rank) * a.t.groupStride + group];
-    const int32_t *items = a.t.workList + base + static_cast<int64_t>(group) * kRowsPerGroup;
+    const int64_t base = static_cast<int64_t>(rank) * a.tables.stride;
+    const int count = a.tables.workCount[static_cast<int64_t>(rank) * a.tables.groupStride + group];
+    const int32_t *items = a.tables.workList + base + static_cast<int64_t>(group) * kRowsPerGroup;
     const int lane = threadIdx.x;
+    const int h = static_cast<int>(a.h);
+    char *tensor = static_cast<char *>(a.hiddenNvsh[rank]);
     for (int i = part; i < count; i += kFillSplit) {
         const int32_t item = items[i];
         const int row = item & 0x3fffffff;
         bool copy = (item >> 30) == kFillCopy;
         int primary = 0;
         if (copy) {
-            primary = static_cast<int>(a.t.parentTag[base + row] & 0xffffffffu) - 1;
+            primary = static_cast<int>(a.tables.parentTag[base + row] & 0xffffffffu) - 1;
             // a primary no route wrote is all zeros in the reference too (the window was cleared)
-            const uint64_t tag = a.t.rowTag[base + primary];
+            const uint64_t tag = a.tables.rowTag[base + primary];
             copy = Tagged(tag, a.epoch) && (tag & kRowWritten) != 0;
         }
         if (VEC) {
-            const int vecs = a.h / 8;
-            u32x4 *dstRow = reinterpret_cast<u32x4 *>(static_cast<char *>(a.hiddenNvsh) + static_cast<int64_t>(row) * a.h * 2);
-            const u32x4 *srcRow = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.hiddenNvsh) +
-                static_cast<int64_t>(primary) * a.h * 2);
+            const int vecs = h / 8;
+            u32x4 *dstRow = reinterpret_cast<u32x4 *>(tensor + static_cast<int64_t>(row) * h * 2);
+            const u32x4 *srcRow = reinterpret_cast<const u32x4 *>(tensor + static_cast<int64_t>(primary) * h * 2);
             for (int idx = lane; idx < vecs; idx += kThreads) {
                 const u32x4 v = copy ? srcRow[idx] : u32x4{0u, 0u, 0u, 0u};
                 __builtin_nontemporal_store(v, dstRow + idx);
             }
         } else {
-            uint16_t *dstRow = static_cast<uint16_t *>(a.hiddenNvsh) + static_cast<int64_t>(row) * a.h;
-            const uint16_t *srcRow = static_cast<const uint16_t *>(a.hiddenNvsh) + static_cast<int64_t>(primary) * a.h;
-            for (int c = lane; c < a.h; c += kThreads) {
+            uint16_t *dstRow = reinterpret_cast<uint16_t *>(tensor) + static_cast<int64_t>(row) * h;
+            const uint16_t *srcRow = reinterpret_cast<const uint16_t *>(tensor) + static_cast<int64_t>(primary) * h;
+            for (int c = lane; c < h; c += kThreads) {
                 dstRow[c] = copy ? srcRow[c] : static_cast<uint16_t>(0);
             }
         }
@@ -537,55 +626,57 @@ __global__ __launch_bounds__(kThreads) void moon_fill_kernel(FillArgs a)
 }
 
 // ---------------------------------------------------------------------------------------------------------------
-// combine: reverse routes -> slot table of the origin ranks
+// combine: prepare
 // ---------------------------------------------------------------------------------------------------------------
-struct ReverseArgs {
-    const int32_t *dstLocal;
-    int64_t nvS, n;
-    int world;
-    int rank;
-    WorldTables t;
-    uint64_t epoch;
-};
 
+// Thread i of expert rank blockIdx.y walks duplicate group i (marks the slots of its duplicates, leaves the group's extent
+// at the slot of its primary) and files receive row i under the slot of the origin it returns to.
 // reference: combine kernel :285-298 (decode), :350-366 (validation), :568-606 (which rows travel)
-__global__ __launch_bounds__(kThreads) void moon_reverse_kernel(ReverseArgs a)
+__global__ __launch_bounds__(kThreads) void moon_combine_prepare_kernel(CombineWorld a)
 {
+    const int rank = blockIdx.y;
     const int64_t row = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    WalkArgs w {a.nvS, rank, true, a.dupGroups[rank], a.dupLoffs[rank], a.dupCounts[rank], a.tables, a.epoch, a.dstLocal[rank],
+        a.world, a.s * a.k};
+    WalkGroup(w, row);
     if (row >= a.nvS) {
         return;
     }
-    const int32_t encoded = a.dstLocal[row];
+    const int32_t encoded = a.dstLocal[rank][row];
     if (encoded == -1) {
         return;
     }
     const int64_t peer = encoded / a.nvS;
     const int64_t target = encoded % a.nvS;
-    if (encoded < 0 || peer >= a.world || target >= a.n) {
-        RecordFailure(a.t, a.rank, a.epoch, kCombineInvalidRoute);
+    if (encoded < 0 || peer >= a.world || target >= a.s * a.k) {
+        RecordFailure(a.tables, rank, a.epoch, kCombineInvalidRoute);
         return;
     }
-    const int64_t base = static_cast<int64_t>(a.rank) * a.t.stride;
-    const uint32_t duplicate = Tagged(a.t.dupMask[base + row], a.epoch) ? 0x80000000u : 0u;
-    a.t.slotSrc[peer * a.t.stride + target] = Tag(a.epoch, duplicate | static_cast<uint32_t>(a.rank * a.nvS + row));
+    a.tables.slotSrc[peer * a.tables.stride + target] = Tag(a.epoch, static_cast<uint32_t>(rank * a.nvS + row));
 }
 
 // ---------------------------------------------------------------------------------------------------------------
 // combine: reduce
 // ---------------------------------------------------------------------------------------------------------------
-struct ReduceArgs {
-    int s, k, h;
-    int64_t nvS;
-    int world;
-    int rank;
-    int colSlices;
-    SourceTable src;
-    WorldTables t;
-    uint64_t epoch;
-    void *hiddenSh;
-    float *weightsSk;
-    int32_t *status;
-};
+
+// Device status of combine: own failure, else the first failed peer in rank order (combine kernel :391-411), else 0.
+__device__ __forceinline__ void WriteCombineStatus(const CombineWorld &a, int rank)
+{
+    int32_t value = kCombineOk;
+    const uint64_t own = __hip_atomic_load(&a.tables.fail[rank], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (Tagged(own, a.epoch)) {
+        value = static_cast<int32_t>(own & 0xffffffffu);
+    } else {
+        for (int peer = 0; peer < a.world; ++peer) {
+            const uint64_t f = __hip_atomic_load(&a.tables.fail[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (Tagged(f, a.epoch)) {
+                value = kCombineRemoteFailureBase + peer;
+                break;
+            }
+        }
+    }
+    a.status[rank][0] = value;
+}
 
 __device__ __forceinline__ void AddRow(float (&acc)[kRowVecs][8], const u32x4 (&v)[kRowVecs])
 {
@@ -599,57 +690,74 @@ __device__ __forceinline__ void AddRow(float (&acc)[kRowVecs][8], const u32x4 (&
     }
 }
 
-template <bool VEC>
-struct RowReader;
-
-// 16-byte vectors, two per lane; a unit is one slice of G * kRowVecs vectors of one token.
-template <>
-struct RowReader<true> {
-    __device__ static __forceinline__ void Load(const void *tensor, int64_t row, int h, int colBase, int lane, int lanes,
-        u32x4 (&v)[kRowVecs])
-    {
-        const u32x4 *p = reinterpret_cast<const u32x4 *>(static_cast<const char *>(tensor) + row * h * 2);
-        const int vecs = h / 8;
-#pragma unroll
-        for (int j = 0; j < kRowVecs; ++j) {
-            const int idx = colBase + j * lanes + lane;
-            v[j] = idx < vecs ? __builtin_nontemporal_load(p + idx) : u32x4{0u, 0u, 0u, 0u};
-        }
-    }
-};
-
-// Slot sum of one token slice.  Slots are taken in slot order from zero (combine kernel :664-699); a slot that holds a
-// primary with duplicates contributes bf16(fp32(primary) + fp32(dup) + ...) in the plan's list order (combine kernel
-// :489-530); duplicate rows and slots nothing was returned to contribute nothing (their receive row stays zero).
-template <int G>
-__global__ __launch_bounds__(G) void moon_reduce_kernel(ReduceArgs a)
+__device__ __forceinline__ void LoadRowSlice(const void *tensor, int64_t row, int h, int colBase, int lane, int lanes,
+    u32x4 (&v)[kRowVecs])
 {
-    __shared__ uint64_t s_slot[kMaxTopK];
-    const int xcdUnits = a.s * a.colSlices;
-    const int unit = blockIdx.x;
-    if (unit >= xcdUnits) {
+    const u32x4 *p = reinterpret_cast<const u32x4 *>(static_cast<const char *>(tensor) + row * h * 2);
+    const int vecs = h / 8;
+#pragma unroll
+    for (int j = 0; j < kRowVecs; ++j) {
+        const int idx = colBase + j * lanes + lane;
+        v[j] = idx < vecs ? __builtin_nontemporal_load(p + idx) : u32x4{0u, 0u, 0u, 0u};
+    }
+}
+
+// What the reduce kernels need to know about the K slots of a token, gathered by K lanes at once so that the table
+// lookups of all slots overlap (done slot after slot they would be K dependent round trips to memory).
+struct TokenSlots {
+    uint32_t where[kMaxTopK];   // expert rank * nvS + row of the slot's row; kNoRow when the slot contributes nothing
+    int32_t start[kMaxTopK];    // first dupLoffs index of the row's duplicate group
+    int32_t count[kMaxTopK];    // duplicates in the group; 0 for a row without duplicates
+};
+constexpr uint32_t kNoRow = 0xffffffffu;
+
+// A slot contributes nothing when nothing was returned to it or when the row filed under it is a duplicate (a
+// duplicate row does not travel: its values are part of its primary's slot, combine kernel :583-590).  Weights come
+// back for every receive row, duplicates included (combine kernel :593-600).
+__device__ __forceinline__ void LoadSlots(const CombineWorld &a, int rank, int token, bool writeWeights, TokenSlots *s)
+{
+    const int lane = threadIdx.x;
+    const int K = static_cast<int>(a.k);
+    if (lane >= K) {
         return;
     }
-    const int token = unit / a.colSlices;
-    const int colBase = (unit % a.colSlices) * (G * kRowVecs);
+    const int64_t slot = static_cast<int64_t>(rank) * a.tables.stride + static_cast<int64_t>(token) * K + lane;
+    const uint64_t w = a.tables.slotSrc[slot];
+    const uint64_t dup = a.tables.slotDup[slot];
+    const uint64_t group = a.tables.slotGroup[slot];
+    const int32_t groupCount = a.tables.slotCount[slot];
+    const bool present = Tagged(w, a.epoch);
+    const uint32_t low = static_cast<uint32_t>(w);
+    if (writeWeights && a.weightsSk[rank] != nullptr) {
+        a.weightsSk[rank][static_cast<int64_t>(token) * K + lane] = present ? a.weightsNvs[low / a.nvS][low % a.nvS] : 0.0f;
+    }
+    const bool travels = present && !Tagged(dup, a.epoch);
+    const bool grouped = travels && Tagged(group, a.epoch);
+    s->where[lane] = travels ? low : kNoRow;
+    s->start[lane] = grouped ? static_cast<int32_t>(group & 0xffffffffu) : 0;
+    s->count[lane] = grouped ? groupCount : 0;
+}
+
+// Slot sum of one token slice of origin rank blockIdx.y.  Slots are taken in slot order from zero (combine kernel
+// :664-699); a slot that holds a primary with duplicates contributes bf16(fp32(primary) + fp32(dup) + ...) in the plan's
+// list order (combine kernel :489-530); slots that contribute nothing leave the sum as it is (their receive row stays
+// zero in the reference).
+template <int G>
+__global__ __launch_bounds__(G) void moon_reduce_kernel(CombineWorld a, int colSlices)
+{
+    __shared__ TokenSlots s_slots;
+    const int rank = blockIdx.y;
+    const int unit = blockIdx.x;
+    const int token = unit / colSlices;
+    const int colBase = (unit % colSlices) * (G * kRowVecs);
     const int lane = threadIdx.x;
-    const int vecs = a.h / 8;
-    const uint64_t *slots = a.t.slotSrc + static_cast<int64_t>(a.rank) * a.t.stride + static_cast<int64_t>(token) * a.k;
-    if (lane < a.k) {
-        const uint64_t w = slots[lane];
-        s_slot[lane] = w;
-        if (colBase == 0 && a.weightsSk != nullptr) {
-            float weight = 0.0f;
-            if (Tagged(w, a.epoch)) {
-                const uint32_t where = static_cast<uint32_t>(w) & 0x7fffffffu;
-                weight = a.src.weights[where / a.nvS][where % a.nvS];
-            }
-            a.weightsSk[static_cast<int64_t>(token) * a.k + lane] = weight;
-        }
+    const int h = static_cast<int>(a.h);
+    const int vecs = h / 8;
+    if (unit == 0 && lane == 0) {
+        WriteCombineStatus(a, rank);
     }
-    if (G > kWave) {
-        __syncthreads();
-    }
+    LoadSlots(a, rank, token, colBase == 0, &s_slots);
+    TileXREp::LdsBarrier();
     float acc[kRowVecs][8];
 #pragma unroll
     for (int j = 0; j < kRowVecs; ++j) {
@@ -658,24 +766,24 @@ __global__ __launch_bounds__(G) void moon_reduce_kernel(ReduceArgs a)
             acc[j][e] = 0.0f;
         }
     }
-    for (int k = 0; k < a.k; ++k) {
-        const uint64_t w = s_slot[k];
-        const uint32_t low = static_cast<uint32_t>(w);
-        if (!Tagged(w, a.epoch) || (low & 0x80000000u) != 0u) {
+    const int K = static_cast<int>(a.k);
+    const uint32_t nvS = static_cast<uint32_t>(a.nvS);
+    for (int k = 0; k < K; ++k) {
+        // the lanes of the workgroup share one token: everything read from s_slots is uniform
+        const uint32_t where = __builtin_amdgcn_readfirstlane(s_slots.where[k]);
+        if (where == kNoRow) {
             continue;
         }
-        const int q = static_cast<int>(low / a.nvS);
-        const int64_t row = low % a.nvS;
+        const int q = static_cast<int>(where / nvS);
+        const int64_t row = where % nvS;
+        const int count = __builtin_amdgcn_readfirstlane(s_slots.count[k]);
         u32x4 v[kRowVecs];
-        RowReader<true>::Load(a.src.hidden[q], row, a.h, colBase, lane, G, v);
-        const uint64_t gw = a.t.groupOf[static_cast<int64_t>(q) * a.t.stride + row];
-        if (!Tagged(gw, a.epoch)) {
+        LoadRowSlice(a.hiddenNvsh[q], row, h, colBase, lane, G, v);
+        if (count == 0) {
             AddRow(acc, v);
             continue;
         }
-        const int64_t g = static_cast<int64_t>(gw & 0xffffffffu) - 1;
-        const int32_t start = a.src.dupGroups[q][g * 3 + 1];
-        const int32_t count = a.src.dupGroups[q][g * 3 + 2];
+        const int start = __builtin_amdgcn_readfirstlane(s_slots.start[k]);
         float sub[kRowVecs][8];
 #pragma unroll
         for (int j = 0; j < kRowVecs; ++j) {
@@ -691,7 +799,7 @@ __global__ __launch_bounds__(G) void moon_reduce_kernel(ReduceArgs a)
 #pragma unroll
             for (int u = 0; u < kBatch; ++u) {
                 if (i0 + u < count) {
-                    RowReader<true>::Load(a.src.hidden[q], a.src.dupLoffs[q][start + i0 + u], a.h, colBase, lane, G, d[u]);
+                    LoadRowSlice(a.hiddenNvsh[q], a.dupLoffs[q][start + i0 + u], h, colBase, lane, G, d[u]);
                 }
             }
 #pragma unroll
@@ -711,7 +819,7 @@ __global__ __launch_bounds__(G) void moon_reduce_kernel(ReduceArgs a)
             }
         }
     }
-    u32x4 *out = reinterpret_cast<u32x4 *>(static_cast<char *>(a.hiddenSh) + static_cast<int64_t>(token) * a.h * 2);
+    u32x4 *out = reinterpret_cast<u32x4 *>(static_cast<char *>(a.hiddenSh[rank]) + static_cast<int64_t>(token) * h * 2);
 #pragma unroll
     for (int j = 0; j < kRowVecs; ++j) {
         const int idx = colBase + j * G + lane;
@@ -727,78 +835,58 @@ __global__ __launch_bounds__(G) void moon_reduce_kernel(ReduceArgs a)
 }
 
 // Any hidden size and alignment: one workgroup per token, one element per thread step.
-__global__ __launch_bounds__(kThreads) void moon_reduce_generic_kernel(ReduceArgs a)
+__global__ __launch_bounds__(kThreads) void moon_reduce_generic_kernel(CombineWorld a)
 {
-    __shared__ uint64_t s_slot[kMaxTopK];
+    __shared__ TokenSlots s_slots;
+    const int rank = blockIdx.y;
     const int token = blockIdx.x;
     const int lane = threadIdx.x;
-    const uint64_t *slots = a.t.slotSrc + static_cast<int64_t>(a.rank) * a.t.stride + static_cast<int64_t>(token) * a.k;
-    if (lane < a.k) {
-        const uint64_t w = slots[lane];
-        s_slot[lane] = w;
-        if (a.weightsSk != nullptr) {
-            float weight = 0.0f;
-            if (Tagged(w, a.epoch)) {
-                const uint32_t where = static_cast<uint32_t>(w) & 0x7fffffffu;
-                weight = a.src.weights[where / a.nvS][where % a.nvS];
-            }
-            a.weightsSk[static_cast<int64_t>(token) * a.k + lane] = weight;
-        }
+    if (token == 0 && lane == 0) {
+        WriteCombineStatus(a, rank);
     }
+    LoadSlots(a, rank, token, true, &s_slots);
     __syncthreads();
+    const int K = static_cast<int>(a.k);
+    const uint32_t nvS = static_cast<uint32_t>(a.nvS);
     for (int c = lane; c < a.h; c += kThreads) {
         float acc = 0.0f;
-        for (int k = 0; k < a.k; ++k) {
-            const uint64_t w = s_slot[k];
-            const uint32_t low = static_cast<uint32_t>(w);
-            if (!Tagged(w, a.epoch) || (low & 0x80000000u) != 0u) {
+        for (int k = 0; k < K; ++k) {
+            const uint32_t where = s_slots.where[k];
+            if (where == kNoRow) {
                 continue;
             }
-            const int q = static_cast<int>(low / a.nvS);
-            const int64_t row = low % a.nvS;
-            const uint16_t *tensor = static_cast<const uint16_t *>(a.src.hidden[q]);
+            const int q = static_cast<int>(where / nvS);
+            const int64_t row = where % nvS;
+            const uint16_t *tensor = static_cast<const uint16_t *>(a.hiddenNvsh[q]);
             float value = __uint_as_float(static_cast<uint32_t>(tensor[row * a.h + c]) << 16);
-            const uint64_t gw = a.t.groupOf[static_cast<int64_t>(q) * a.t.stride + row];
-            if (Tagged(gw, a.epoch)) {
-                const int64_t g = static_cast<int64_t>(gw & 0xffffffffu) - 1;
-                const int32_t start = a.src.dupGroups[q][g * 3 + 1];
-                const int32_t count = a.src.dupGroups[q][g * 3 + 2];
-                for (int32_t i = 0; i < count; ++i) {
-                    const int64_t dup = a.src.dupLoffs[q][start + i];
+            const int count = s_slots.count[k];
+            if (count != 0) {
+                const int start = s_slots.start[k];
+                for (int i = 0; i < count; ++i) {
+                    const int64_t dup = a.dupLoffs[q][start + i];
                     value = __fadd_rn(value, __uint_as_float(static_cast<uint32_t>(tensor[dup * a.h + c]) << 16));
                 }
                 value = __uint_as_float(TileXREp::FloatToBf16Rne(value) << 16);
             }
             acc = __fadd_rn(acc, value);
         }
-        static_cast<uint16_t *>(a.hiddenSh)[static_cast<int64_t>(token) * a.h + c] =
+        static_cast<uint16_t *>(a.hiddenSh[rank])[static_cast<int64_t>(token) * a.h + c] =
             static_cast<uint16_t>(TileXREp::FloatToBf16Rne(acc));
     }
 }
 
-// Device status of combine: own failure, else the first failed peer in rank order (combine kernel :391-411), else 0.
-__global__ void moon_combine_status_kernel(WorldTables t, int world, int rank, uint64_t epoch, int32_t *status)
+hipError_t RecordIf(hipEvent_t e, hipStream_t stream)
 {
-    int32_t value = kCombineOk;
-    const uint64_t own = __hip_atomic_load(&t.fail[rank], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (Tagged(own, epoch)) {
-        value = static_cast<int32_t>(own & 0xffffffffu);
-    } else {
-        for (int peer = 0; peer < world; ++peer) {
-            const uint64_t f = __hip_atomic_load(&t.fail[peer], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (Tagged(f, epoch)) {
-                value = kCombineRemoteFailureBase + peer;
-                break;
-            }
-        }
-    }
-    status[0] = value;
+    return e == nullptr ? hipSuccess : hipEventRecord(e, stream);
 }
 
-bool VectorRows(int64_t h, const void *a, const void *b)
-{
-    return h % 8 == 0 && TileXREp::Aligned16(a) && TileXREp::Aligned16(b);
-}
+#define MOON_LAUNCH_CHECK()                \
+    do {                                   \
+        const hipError_t launchErr = hipGetLastError(); \
+        if (launchErr != hipSuccess) {     \
+            return launchErr;              \
+        }                                  \
+    } while (0)
 
 } // namespace
 
@@ -812,155 +900,91 @@ const char *MoonReduceKernelName()
     return gReduceName;
 }
 
-hipError_t LaunchMoonScatter(const ScatterLaunch &l)
+hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const LaunchTiming &timing)
 {
-    ScatterArgs a {};
-    a.dst = l.dst;
-    a.hiddenSh = l.hiddenSh;
-    a.weightsSk = l.weightsSk;
-    a.s = static_cast<int>(l.s);
-    a.k = static_cast<int>(l.k);
-    a.h = static_cast<int>(l.h);
-    a.nvS = l.nvS;
-    a.world = l.world;
-    a.srcRank = l.srcRank;
-    a.out = l.out;
-    a.t = l.tables;
-    a.epoch = l.epoch;
-    bool vec = l.h % 8 == 0 && TileXREp::Aligned16(l.hiddenSh);
-    for (int r = 0; r < l.world; ++r) {
-        vec = vec && TileXREp::Aligned16(l.out.hidden[r]);
+    const unsigned R = static_cast<unsigned>(w.world);
+    const unsigned rowBlocks = static_cast<unsigned>((w.nvS + kThreads - 1) / kThreads);
+    if (!w.fresh) {
+        hipLaunchKernelGGL(moon_group_walk_kernel, dim3(rowBlocks, R), dim3(kThreads), 0, stream, w);
+        MOON_LAUNCH_CHECK();
     }
-    const int64_t vecs = l.h / 8;
-    a.colSlices = static_cast<int>((vecs + kRowVecs * kThreads - 1) / (kRowVecs * kThreads));
-    const int64_t blocks = (l.s + kXcds - 1) / kXcds * kXcds * l.k * a.colSlices;
+    bool vec = w.h % 8 == 0;
+    for (int r = 0; r < w.world; ++r) {
+        vec = vec && TileXREp::Aligned16(w.hiddenSh[r]) && TileXREp::Aligned16(w.hiddenNvsh[r]);
+    }
+    const int64_t vecs = w.h / 8;
+    const int colSlices = static_cast<int>((vecs + kRowVecs * kThreads - 1) / (kRowVecs * kThreads));
+    const int64_t blocks = (w.s + kXcds - 1) / kXcds * kXcds * w.k * colSlices;
+    hipError_t err = RecordIf(timing.start, stream);
+    if (err != hipSuccess) {
+        return err;
+    }
     if (vec && blocks <= 0x7fffffff) {
         gScatterName = "moon_scatter_kernel";
-        if (l.fresh) {
-            hipLaunchKernelGGL(moon_scatter_kernel<true>, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, l.stream, a);
+        if (w.fresh) {
+            hipLaunchKernelGGL(moon_scatter_kernel<true>, dim3(static_cast<unsigned>(blocks), R), dim3(kThreads), 0, stream, w, colSlices);
         } else {
-            hipLaunchKernelGGL(moon_scatter_kernel<false>, dim3(static_cast<unsigned>(blocks)), dim3(kThreads), 0, l.stream, a);
+            hipLaunchKernelGGL(moon_scatter_kernel<false>, dim3(static_cast<unsigned>(blocks), R), dim3(kThreads), 0, stream, w, colSlices);
         }
     } else {
         gScatterName = "moon_scatter_generic_kernel";
-        const unsigned grid = static_cast<unsigned>(l.s * l.k);
-        if (l.fresh) {
-            hipLaunchKernelGGL(moon_scatter_generic_kernel<true>, dim3(grid), dim3(kThreads), 0, l.stream, a);
+        const unsigned grid = static_cast<unsigned>(w.s * w.k);
+        if (w.fresh) {
+            hipLaunchKernelGGL(moon_scatter_generic_kernel<true>, dim3(grid, R), dim3(kThreads), 0, stream, w);
         } else {
-            hipLaunchKernelGGL(moon_scatter_generic_kernel<false>, dim3(grid), dim3(kThreads), 0, l.stream, a);
+            hipLaunchKernelGGL(moon_scatter_generic_kernel<false>, dim3(grid, R), dim3(kThreads), 0, stream, w);
         }
     }
-    return hipGetLastError();
-}
-
-hipError_t LaunchMoonDedupBuild(const DedupBuildLaunch &l)
-{
-    BuildArgs a {};
-    a.nvS = l.nvS;
-    a.rank = l.rank;
-    a.t = l.tables;
-    a.epoch = l.epoch;
-    a.dupGroups = l.dupGroups;
-    a.dupLoffs = l.dupLoffs;
-    a.dupCounts = l.dupCounts;
-    hipLaunchKernelGGL(moon_dedup_build_kernel, dim3(1), dim3(kThreads), 0, l.stream, a);
-    return hipGetLastError();
-}
-
-hipError_t LaunchMoonGroupWalk(const GroupWalkLaunch &l)
-{
-    WalkArgs a {};
-    a.nvS = l.nvS;
-    a.rank = l.rank;
-    a.combine = l.combine;
-    a.dupGroups = l.dupGroups;
-    a.dupLoffs = l.dupLoffs;
-    a.dupCounts = l.dupCounts;
-    a.t = l.tables;
-    a.epoch = l.epoch;
-    const unsigned grid = static_cast<unsigned>((l.nvS + kThreads - 1) / kThreads);
-    hipLaunchKernelGGL(moon_group_walk_kernel, dim3(grid), dim3(kThreads), 0, l.stream, a);
-    return hipGetLastError();
-}
-
-hipError_t LaunchMoonFill(const FillLaunch &l)
-{
-    FillArgs a {};
-    a.nvS = l.nvS;
-    a.h = static_cast<int>(l.h);
-    a.world = l.world;
-    a.rank = l.rank;
-    a.expand = l.expand;
-    a.hiddenNvsh = l.hiddenNvsh;
-    a.weightsNvs = l.weightsNvs;
-    a.t = l.tables;
-    a.epoch = l.epoch;
-    a.status = l.status;
-    const unsigned groups = static_cast<unsigned>((l.nvS + kRowsPerGroup - 1) / kRowsPerGroup);
-    hipLaunchKernelGGL(moon_classify_kernel, dim3(groups), dim3(kRowsPerGroup), 0, l.stream, a);
-    hipError_t err = hipGetLastError();
+    MOON_LAUNCH_CHECK();
+    err = RecordIf(timing.stop, stream);
     if (err != hipSuccess) {
         return err;
     }
-    if (VectorRows(l.h, l.hiddenNvsh, l.hiddenNvsh)) {
-        hipLaunchKernelGGL(moon_fill_kernel<true>, dim3(groups * kFillSplit), dim3(kThreads), 0, l.stream, a);
+    if (w.fresh) {
+        const unsigned chunks = static_cast<unsigned>((w.nvS + kBuildRows - 1) / kBuildRows);
+        hipLaunchKernelGGL(moon_dedup_totals_kernel, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+        MOON_LAUNCH_CHECK();
+        hipLaunchKernelGGL(moon_dedup_groups_kernel, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+        MOON_LAUNCH_CHECK();
+    }
+    const unsigned groups = static_cast<unsigned>((w.nvS + kRowsPerGroup - 1) / kRowsPerGroup);
+    hipLaunchKernelGGL(moon_classify_kernel, dim3(groups, R), dim3(kRowsPerGroup), 0, stream, w);
+    MOON_LAUNCH_CHECK();
+    if (vec) {
+        hipLaunchKernelGGL(moon_fill_kernel<true>, dim3(groups * kFillSplit, R), dim3(kThreads), 0, stream, w);
     } else {
-        hipLaunchKernelGGL(moon_fill_kernel<false>, dim3(groups * kFillSplit), dim3(kThreads), 0, l.stream, a);
+        hipLaunchKernelGGL(moon_fill_kernel<false>, dim3(groups * kFillSplit, R), dim3(kThreads), 0, stream, w);
     }
     return hipGetLastError();
 }
 
-hipError_t LaunchMoonReverse(const ReverseLaunch &l)
+hipError_t LaunchMoonCombine(const CombineWorld &w, hipStream_t stream, const LaunchTiming &timing)
 {
-    ReverseArgs a {};
-    a.dstLocal = l.dstLocal;
-    a.nvS = l.nvS;
-    a.n = l.n;
-    a.world = l.world;
-    a.rank = l.rank;
-    a.t = l.tables;
-    a.epoch = l.epoch;
-    const unsigned grid = static_cast<unsigned>((l.nvS + kThreads - 1) / kThreads);
-    hipLaunchKernelGGL(moon_reverse_kernel, dim3(grid), dim3(kThreads), 0, l.stream, a);
-    return hipGetLastError();
-}
-
-hipError_t LaunchMoonReduce(const MoonReduceLaunch &l)
-{
-    ReduceArgs a {};
-    a.s = static_cast<int>(l.s);
-    a.k = static_cast<int>(l.k);
-    a.h = static_cast<int>(l.h);
-    a.nvS = l.nvS;
-    a.world = l.world;
-    a.rank = l.rank;
-    a.src = l.src;
-    a.t = l.tables;
-    a.epoch = l.epoch;
-    a.hiddenSh = l.hiddenSh;
-    a.weightsSk = l.weightsSk;
-    a.status = l.status;
-    bool vec = l.h % 8 == 0 && TileXREp::Aligned16(l.hiddenSh);
-    for (int r = 0; r < l.world; ++r) {
-        vec = vec && TileXREp::Aligned16(l.src.hidden[r]);
+    const unsigned R = static_cast<unsigned>(w.world);
+    const unsigned rowBlocks = static_cast<unsigned>((w.nvS + kThreads - 1) / kThreads);
+    hipLaunchKernelGGL(moon_combine_prepare_kernel, dim3(rowBlocks, R), dim3(kThreads), 0, stream, w);
+    MOON_LAUNCH_CHECK();
+    bool vec = w.h % 8 == 0;
+    for (int r = 0; r < w.world; ++r) {
+        vec = vec && TileXREp::Aligned16(w.hiddenSh[r]) && TileXREp::Aligned16(w.hiddenNvsh[r]);
     }
-    const int64_t vecs = l.h / 8;
+    const int64_t vecs = w.h / 8;
     constexpr int G = kWave;
-    a.colSlices = static_cast<int>((vecs + G * kRowVecs - 1) / (G * kRowVecs));
-    const int64_t units = l.s * a.colSlices;
+    const int colSlices = static_cast<int>((vecs + G * kRowVecs - 1) / (G * kRowVecs));
+    const int64_t units = w.s * colSlices;
+    hipError_t err = RecordIf(timing.start, stream);
+    if (err != hipSuccess) {
+        return err;
+    }
     if (vec && units <= 0x7fffffff) {
         gReduceName = "moon_reduce_kernel";
-        hipLaunchKernelGGL(moon_reduce_kernel<G>, dim3(static_cast<unsigned>(units)), dim3(G), 0, l.stream, a);
+        hipLaunchKernelGGL(moon_reduce_kernel<G>, dim3(static_cast<unsigned>(units), R), dim3(G), 0, stream, w, colSlices);
     } else {
         gReduceName = "moon_reduce_generic_kernel";
-        hipLaunchKernelGGL(moon_reduce_generic_kernel, dim3(static_cast<unsigned>(l.s)), dim3(kThreads), 0, l.stream, a);
+        hipLaunchKernelGGL(moon_reduce_generic_kernel, dim3(static_cast<unsigned>(w.s), R), dim3(kThreads), 0, stream, w);
     }
-    hipError_t err = hipGetLastError();
-    if (err != hipSuccess) {
-        return err;
-    }
-    hipLaunchKernelGGL(moon_combine_status_kernel, dim3(1), dim3(1), 0, l.stream, l.tables, l.world, l.rank, l.epoch, l.status);
-    return hipGetLastError();
+    MOON_LAUNCH_CHECK();
+    return RecordIf(timing.stop, stream);
 }
 
 } // namespace TileXRMoon
