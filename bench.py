@@ -183,6 +183,13 @@ def main_moonep(args):
         dispatch(flags)
         combine()
 
+    if args.calibrate_copy:
+        src = torch.zeros((64 << 20,), dtype=torch.int32, device=dev)
+        dst_copy = torch.empty_like(src)
+        for _ in range(3):
+            torch.add(src, 1, out=dst_copy)      # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del src, dst_copy
     torch.cuda.synchronize()
     dispatch(mp.FLAG_BUILD_DEDUP)       # the saved plan of a --moon-saved run
     for _ in range(args.warmup):

@@ -151,11 +151,11 @@ int Internal(hipError_t err, const char *what)
 bool PrepareTables(WorldState *st, int world, int64_t nvS, int64_t n, WorldTables *out)
 {
     const int64_t rows = nvS > n ? nvS : n;
-    const int64_t stride = (rows + kRowsPerGroup - 1) / kRowsPerGroup * kRowsPerGroup;
-    const int64_t groups = stride / kRowsPerGroup;
+    const int64_t stride = (rows + kTableAlign - 1) / kTableAlign * kTableAlign;
+    const int64_t groups = (rows + kChunkRows - 1) / kChunkRows;
     const int64_t perRank8 = stride * 8;
-    // six 8-byte tables, three 4-byte tables, then the per-rank words
-    const int64_t bytes = world * (6 * perRank8 + 3 * stride * 4) + world * 8 + world * groups * 12 + 256;
+    // six 8-byte tables, two 4-byte tables, then the per-rank words
+    const int64_t bytes = world * (6 * perRank8 + 2 * stride * 4) + world * 8 + world * groups * 8 + 256;
     if (!st->tables.Reserve(static_cast<size_t>(bytes), true)) {
         return false;
     }
@@ -173,9 +173,7 @@ bool PrepareTables(WorldState *st, int world, int64_t nvS, int64_t n, WorldTable
     out->slotGroup = reinterpret_cast<uint64_t *>(take(world * perRank8));
     out->fail = reinterpret_cast<uint64_t *>(take(world * 8));
     out->sibling = reinterpret_cast<uint32_t *>(take(world * stride * 4));
-    out->workList = reinterpret_cast<int32_t *>(take(world * stride * 4));
     out->slotCount = reinterpret_cast<int32_t *>(take(world * stride * 4));
-    out->workCount = reinterpret_cast<int32_t *>(take(world * groups * 4));
     out->chunkTotals = reinterpret_cast<int32_t *>(take(world * groups * 8));
     out->stride = stride;
     out->groupStride = groups;

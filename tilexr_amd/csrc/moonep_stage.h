@@ -10,10 +10,9 @@
 //
 //   dispatch  walk      saved plans: parent records from dupGroups / dupLoffs
 //             scatter   rows, weights, row tags; fresh plans: parent / sibling records of duplicates
-//             build     fresh plans: dupGroups / dupCounts from the parent records (chunk totals, then group records)
-//             classify  per row: what is left to write (zeros, or a copy of the primary of a saved plan); dupLoffs of
-//                       a fresh plan; weights of unnamed rows; device status
-//             fill      writes what classify listed
+//             build     fresh plans: dupGroups / dupCounts from the parent records
+//             finish    per row: what is left to write (zeros, or a copy of the primary of a saved plan) and writing it;
+//                       dupLoffs of a fresh plan; weights of unnamed rows; device status
 //   combine   prepare   dstLocal and the duplicate plan -> per-slot tables of the origins (which row, duplicate or not,
 //                       its duplicate group)
 //             reduce    K slots per token, duplicate groups pre-summed, fp32 -> bf16; device status
@@ -28,8 +27,8 @@ namespace TileXRMoon {
 
 constexpr int kMaxWorld = 16;       // ranks of a world this library runs the stages for
 constexpr int kMaxTopK = 32;        // reference: src/moonep/common/moonep_stage_layout.h:78
-constexpr int kRowsPerGroup = 256;  // rows one classify workgroup looks at
-constexpr int kFillSplit = 16;      // fill workgroups per classify group
+constexpr int kTableAlign = 256;    // per-rank table strides are a multiple of this many entries
+constexpr int kChunkRows = 2048;    // rows per workgroup of the duplicate-plan build
 
 // Device status values (reference: src/moonep/common/moonep_peer_window.h:36-43).
 constexpr int32_t kDispatchOk = 2000;
@@ -51,11 +50,9 @@ struct WorldTables {
     uint64_t *slotGroup;     // combine: per origin slot, epoch << 32 | first dupLoffs index when that row has duplicates
     int32_t *slotCount;      // combine: per origin slot, number of those duplicates (valid with slotGroup)
     uint64_t *fail;          // [world] epoch << 32 | device status of the rank's own failure
-    int32_t *workList;       // dispatch: rows the fill kernel has to write, grouped by classify group
-    int32_t *workCount;      // dispatch: [world][groups]
-    int32_t *chunkTotals;    // dispatch, fresh plans: [world][groups][2] group-opening rows and duplicates per 2048 rows
-    int64_t stride;          // >= nvS and >= n, a multiple of kRowsPerGroup
-    int64_t groupStride;     // classify groups per rank
+    int32_t *chunkTotals;    // dispatch, fresh plans: [world][groupStride][2] group-opening rows and duplicates per chunk
+    int64_t stride;          // >= nvS and >= n, a multiple of kTableAlign
+    int64_t groupStride;     // chunks per rank
 };
 
 // One Dispatch of every rank of a world.

@@ -263,11 +263,13 @@ __global__ __launch_bounds__(kThreads) void moon_scatter_generic_kernel(Dispatch
 // primary, groups take their dupLoffs slices in that order, and each slice lists its duplicates in ascending row order
 // (dispatch kernel :330-424).  With the rank-within-group and group size recorded by the sources, both numberings are
 // exclusive prefix sums over the rows: group index = number of earlier group-opening rows, slice start = sum of their
-// group sizes.  Two launches: totals of every chunk of 2048 rows, then group records (a workgroup adds up the totals of
-// the chunks before its own, then scans its chunk).  The slices are filled by the classify kernel, which visits every
-// row anyway.
-constexpr int kBuildRows = 2048;
+// group sizes.  A workgroup scans one chunk of 2048 rows after adding up the chunks before its own -- from the rows
+// themselves while the chunks are few, from the totals a first launch leaves otherwise.  The slices are filled by the
+// finish kernel, which visits every row anyway.
+constexpr int kBuildRows = kChunkRows;
 constexpr int kBuildPer = kBuildRows / kThreads;
+constexpr unsigned kSelfTotalChunks = 2;    // up to this many chunks a workgroup sums the earlier ones itself (one after
+                                            // the other: measured 30 us for 17 chunks against 5 us for the extra launch)
 
 struct ChunkRows {
     int opens[kBuildPer];
@@ -352,19 +354,30 @@ __global__ __launch_bounds__(kThreads) void moon_dedup_totals_kernel(DispatchWor
     }
 }
 
+// SELF: the workgroup adds up the chunks before its own from the row records themselves, which is cheaper than a launch
+// of the totals kernel while there are few chunks (the work grows with the square of their number).
+template <bool SELF>
 __global__ __launch_bounds__(kThreads) void moon_dedup_groups_kernel(DispatchWorld a)
 {
     __shared__ int s_part[2][kThreads / kWave];
     __shared__ int s_base[2];
     const int rank = blockIdx.y;
     const int tid = threadIdx.x;
-    const int32_t *totals = a.tables.chunkTotals + static_cast<int64_t>(rank) * a.tables.groupStride * 2;
     // totals of the chunks before this one
     int beforeOpen = 0;
     int beforeSize = 0;
-    for (int c = tid; c < static_cast<int>(blockIdx.x); c += kThreads) {
-        beforeOpen += totals[2 * c];
-        beforeSize += totals[2 * c + 1];
+    if (SELF) {
+        for (int c = 0; c < static_cast<int>(blockIdx.x); ++c) {
+            const ChunkRows earlier = LoadChunkRows(a, rank, static_cast<int64_t>(c) * kBuildRows);
+            beforeOpen += earlier.localOpen;
+            beforeSize += earlier.localSize;
+        }
+    } else {
+        const int32_t *totals = a.tables.chunkTotals + static_cast<int64_t>(rank) * a.tables.groupStride * 2;
+        for (int c = tid; c < static_cast<int>(blockIdx.x); c += kThreads) {
+            beforeOpen += totals[2 * c];
+            beforeSize += totals[2 * c + 1];
+        }
     }
     int exclOpen, exclSize, baseOpen, baseSize;
     ScanPair(beforeOpen, beforeSize, s_part, &exclOpen, &exclSize, &baseOpen, &baseSize);
@@ -497,71 +510,62 @@ __global__ __launch_bounds__(kThreads) void moon_group_walk_kernel(DispatchWorld
 // dispatch: rows nobody wrote
 // ---------------------------------------------------------------------------------------------------------------
 
-// Work item of the fill kernel: row | kind << 30.
+// Work item of the finish kernel: row | kind << 30.
 constexpr int32_t kFillZero = 0;
 constexpr int32_t kFillCopy = 1;
+constexpr int kFinishRows = 64;     // rows one workgroup looks after
 
-// One thread per row decides what is left to do for it: nothing (a route wrote it), zeros (no route wrote it: the
-// reference clears the whole window first, dispatch kernel :206-230), or -- saved plans -- a copy of its primary row
-// (dispatch kernel :426-461).  The weight of a row no route names is zero for the same reason.  Each workgroup packs its
-// rows' work items into its own segment of the work list, so nothing has to be reset between calls.  The duplicates of a
-// fresh plan also take their places in dupLoffs here, and workgroup 0 of every rank writes the rank's device status.
-__global__ __launch_bounds__(kRowsPerGroup) void moon_classify_kernel(DispatchWorld a)
+// What is left to do once every source has scattered.  The first wave of a workgroup looks at 64 rows, one per lane:
+// nothing (a route wrote the row), zeros (no route wrote it: the reference clears the whole window first, dispatch kernel
+// :206-230), or -- saved plans -- a copy of its primary row (dispatch kernel :426-461); the weight of a row no route
+// names is zero for the same reason; the duplicates of a fresh plan take their places in dupLoffs.  Then the whole
+// workgroup writes the rows that need writing.  Workgroup 0 of every rank writes the rank's device status.
+template <bool VEC>
+__global__ __launch_bounds__(kThreads) void moon_finish_kernel(DispatchWorld a)
 {
-    __shared__ int s_waveCount[kRowsPerGroup / kWave];
+    __shared__ int32_t s_items[kFinishRows];
+    __shared__ int s_count;
     const int rank = blockIdx.y;
     const int tid = threadIdx.x;
-    const int lane = tid & (kWave - 1);
-    const int wave = tid / kWave;
     const int64_t base = static_cast<int64_t>(rank) * a.tables.stride;
-    const int64_t row = static_cast<int64_t>(blockIdx.x) * kRowsPerGroup + tid;
-    int32_t item = -1;
-    if (row < a.nvS) {
-        const uint64_t tag = a.tables.rowTag[base + row];
-        const bool tagged = Tagged(tag, a.epoch);
-        const bool named = tagged && (tag & kRowNamed) != 0;
-        const bool written = tagged && (tag & kRowWritten) != 0;
-        const bool direct = tagged && (tag & kRowDirect) != 0;
-        const uint64_t p = a.tables.parentTag[base + row];
-        if (!a.fresh && Tagged(p, a.epoch) && !direct) {
-            item = static_cast<int32_t>(row) | (kFillCopy << 30);
-        } else if (!written) {
-            item = static_cast<int32_t>(row) | (kFillZero << 30);
-        }
-        if (!named && a.weightsNvs[rank] != nullptr) {
-            a.weightsNvs[rank][row] = 0.0f;
-        }
-        if (a.fresh && Tagged(p, a.epoch)) {
-            // slot of this duplicate in its group's slice (dispatch kernel :393-419)
-            const uint64_t gs = a.tables.groupStart[base + static_cast<int64_t>(p & 0xffffffffu) - 1];
-            if (Tagged(gs, a.epoch)) {
-                const int64_t at = static_cast<int64_t>(gs & 0xffffffffu) + (a.tables.sibling[base + row] & 0xffffu);
-                if (at < a.nvS) {
-                    a.dupLoffs[rank][at] = static_cast<int32_t>(row);
-                } else {
-                    RecordFailure(a.tables, rank, a.epoch, kDispatchInvalidRoute);
+    if (tid < kWave) {
+        const int64_t row = static_cast<int64_t>(blockIdx.x) * kFinishRows + tid;
+        int32_t item = -1;
+        if (row < a.nvS) {
+            const uint64_t tag = a.tables.rowTag[base + row];
+            const bool tagged = Tagged(tag, a.epoch);
+            const bool named = tagged && (tag & kRowNamed) != 0;
+            const bool written = tagged && (tag & kRowWritten) != 0;
+            const bool direct = tagged && (tag & kRowDirect) != 0;
+            const uint64_t p = a.tables.parentTag[base + row];
+            if (!a.fresh && Tagged(p, a.epoch) && !direct) {
+                item = static_cast<int32_t>(row) | (kFillCopy << 30);
+            } else if (!written) {
+                item = static_cast<int32_t>(row) | (kFillZero << 30);
+            }
+            if (!named && a.weightsNvs[rank] != nullptr) {
+                a.weightsNvs[rank][row] = 0.0f;
+            }
+            if (a.fresh && Tagged(p, a.epoch)) {
+                // slot of this duplicate in its group's slice (dispatch kernel :393-419)
+                const uint64_t gs = a.tables.groupStart[base + static_cast<int64_t>(p & 0xffffffffu) - 1];
+                if (Tagged(gs, a.epoch)) {
+                    const int64_t at = static_cast<int64_t>(gs & 0xffffffffu) + (a.tables.sibling[base + row] & 0xffffu);
+                    if (at < a.nvS) {
+                        a.dupLoffs[rank][at] = static_cast<int32_t>(row);
+                    } else {
+                        RecordFailure(a.tables, rank, a.epoch, kDispatchInvalidRoute);
+                    }
                 }
             }
         }
-    }
-    const uint64_t have = __ballot(item >= 0);
-    if (lane == 0) {
-        s_waveCount[wave] = __popcll(have);
-    }
-    __syncthreads();
-    int before = 0;
-    int total = 0;
-#pragma unroll
-    for (int w = 0; w < kRowsPerGroup / kWave; ++w) {
-        before += w < wave ? s_waveCount[w] : 0;
-        total += s_waveCount[w];
-    }
-    if (item >= 0) {
-        const int at = before + __popcll(have & ((1ull << lane) - 1ull));
-        a.tables.workList[base + static_cast<int64_t>(blockIdx.x) * kRowsPerGroup + at] = item;
-    }
-    if (tid == 0) {
-        a.tables.workCount[static_cast<int64_t>(rank) * a.tables.groupStride + blockIdx.x] = total;
+        const uint64_t have = __ballot(item >= 0);
+        if (item >= 0) {
+            s_items[__popcll(have & ((1ull << tid) - 1ull))] = item;
+        }
+        if (tid == 0) {
+            s_count = __popcll(have);
+        }
     }
     if (blockIdx.x == 0 && tid == 0) {
         // own failure first, then the first failed peer walking upwards from this rank (dispatch kernel :559-574)
@@ -581,23 +585,12 @@ __global__ __launch_bounds__(kRowsPerGroup) void moon_classify_kernel(DispatchWo
         }
         a.status[rank][0] = status;
     }
-}
-
-// kFillSplit workgroups share the work items of one classify group; a workgroup writes whole rows.
-template <bool VEC>
-__global__ __launch_bounds__(kThreads) void moon_fill_kernel(DispatchWorld a)
-{
-    const int rank = blockIdx.y;
-    const int group = blockIdx.x / kFillSplit;
-    const int part = blockIdx.x % kFillSplit;
-    const int64_t base = static_cast<int64_t>(rank) * a.tables.stride;
-    const int count = a.tables.workCount[static_cast<int64_t>(rank) * a.tables.groupStride + group];
-    const int32_t *items = a.tables.workList + base + static_cast<int64_t>(group) * kRowsPerGroup;
-    const int lane = threadIdx.x;
+    __syncthreads();
+    const int count = s_count;
     const int h = static_cast<int>(a.h);
     char *tensor = static_cast<char *>(a.hiddenNvsh[rank]);
-    for (int i = part; i < count; i += kFillSplit) {
-        const int32_t item = items[i];
+    for (int i = 0; i < count; ++i) {
+        const int32_t item = s_items[i];
         const int row = item & 0x3fffffff;
         bool copy = (item >> 30) == kFillCopy;
         int primary = 0;
@@ -611,14 +604,14 @@ __global__ __launch_bounds__(kThreads) void moon_fill_kernel(DispatchWorld a)
             const int vecs = h / 8;
             u32x4 *dstRow = reinterpret_cast<u32x4 *>(tensor + static_cast<int64_t>(row) * h * 2);
             const u32x4 *srcRow = reinterpret_cast<const u32x4 *>(tensor + static_cast<int64_t>(primary) * h * 2);
-            for (int idx = lane; idx < vecs; idx += kThreads) {
+            for (int idx = tid; idx < vecs; idx += kThreads) {
                 const u32x4 v = copy ? srcRow[idx] : u32x4{0u, 0u, 0u, 0u};
                 __builtin_nontemporal_store(v, dstRow + idx);
             }
         } else {
             uint16_t *dstRow = reinterpret_cast<uint16_t *>(tensor) + static_cast<int64_t>(row) * h;
             const uint16_t *srcRow = reinterpret_cast<const uint16_t *>(tensor) + static_cast<int64_t>(primary) * h;
-            for (int c = lane; c < h; c += kThreads) {
+            for (int c = tid; c < h; c += kThreads) {
                 dstRow[c] = copy ? srcRow[c] : static_cast<uint16_t>(0);
             }
         }
@@ -942,18 +935,20 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
     }
     if (w.fresh) {
         const unsigned chunks = static_cast<unsigned>((w.nvS + kBuildRows - 1) / kBuildRows);
-        hipLaunchKernelGGL(moon_dedup_totals_kernel, dim3(chunks, R), dim3(kThreads), 0, stream, w);
-        MOON_LAUNCH_CHECK();
-        hipLaunchKernelGGL(moon_dedup_groups_kernel, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+        if (chunks <= kSelfTotalChunks) {
+            hipLaunchKernelGGL(moon_dedup_groups_kernel<true>, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+        } else {
+            hipLaunchKernelGGL(moon_dedup_totals_kernel, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+            MOON_LAUNCH_CHECK();
+            hipLaunchKernelGGL(moon_dedup_groups_kernel<false>, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+        }
         MOON_LAUNCH_CHECK();
     }
-    const unsigned groups = static_cast<unsigned>((w.nvS + kRowsPerGroup - 1) / kRowsPerGroup);
-    hipLaunchKernelGGL(moon_classify_kernel, dim3(groups, R), dim3(kRowsPerGroup), 0, stream, w);
-    MOON_LAUNCH_CHECK();
+    const unsigned groups = static_cast<unsigned>((w.nvS + kFinishRows - 1) / kFinishRows);
     if (vec) {
-        hipLaunchKernelGGL(moon_fill_kernel<true>, dim3(groups * kFillSplit, R), dim3(kThreads), 0, stream, w);
+        hipLaunchKernelGGL(moon_finish_kernel<true>, dim3(groups, R), dim3(kThreads), 0, stream, w);
     } else {
-        hipLaunchKernelGGL(moon_fill_kernel<false>, dim3(groups * kFillSplit, R), dim3(kThreads), 0, stream, w);
+        hipLaunchKernelGGL(moon_finish_kernel<false>, dim3(groups, R), dim3(kThreads), 0, stream, w);
     }
     return hipGetLastError();
 }
