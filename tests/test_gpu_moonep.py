@@ -191,6 +191,43 @@ def test_dispatch_and_combine_match_oracle(world, s, k, h, slack, with_weights, 
                 np.testing.assert_array_equal(cres[r]["wy"].cpu().numpy(), wy[r], err_msg=f"rank {r} routeWeightsSk")
 
 
+@pytest.mark.parametrize("seed", range(24))
+def test_random_shapes(seed):
+    """Small random worlds, hidden sizes on both sides of the vector / element-wise split, fresh and saved plans."""
+    rng = np.random.default_rng(1000 + seed)
+    world = int(rng.choice([1, 2, 3, 5, 8]))
+    s = int(rng.integers(1, 70))
+    k = int(rng.integers(1, 13))
+    h = int(rng.choice([8, 16, 24, 40, 64, 136, 17, 33, 1]))
+    slack = int(rng.integers(0, 20))
+    with_weights = bool(rng.integers(0, 2))
+    sh = M.Shape(world, s, k, h, s * k + slack)
+    dst = MC.random_dst(sh, rng, duplicates=bool(rng.integers(0, 4)))
+    hidden = random_rows(rng, (world, s, h))
+    weights = rng.standard_normal((world, s * k)).astype(np.float32) if with_weights else None
+    want = M.dispatch_world(sh, dst, hidden, weights, flags=M.FLAG_BUILD_DEDUP)
+    with World(world) as w:
+        plans = w.plan_tensors(sh, dst)
+        res = w.dispatch(sh, plans, hidden, weights, flags=mp.FLAG_BUILD_DEDUP, order=list(rng.permutation(world)))
+        w.sync()
+        check_dispatch(sh, res, plans, want, fresh=True)
+        res2 = w.dispatch(sh, plans, hidden, weights, flags=0, order=list(rng.permutation(world)))
+        w.sync()
+        check_dispatch(sh, res2, plans, want, fresh=False)
+        out, wout, _, dup = want
+        expert = random_rows(rng, (world, sh.nvs, h))
+        dst_local = M.build_dst_local(sh, dst)
+        cres = w.combine(sh, plans, dst_local, [dev_bits16(expert[r]) for r in range(world)],
+                         None if weights is None else [res[r]["wout"] for r in range(world)])
+        w.sync()
+        y, wy, cstatus = M.combine_world(sh, dst_local, dup, expert, wout)
+        for r in range(world):
+            assert int(plans[r]["status"][0].item()) == int(cstatus[r])
+            np.testing.assert_array_equal(host_bits16(cres[r]["y"]), y[r], err_msg=f"rank {r} hiddenSh")
+            if wy is not None:
+                np.testing.assert_array_equal(cres[r]["wy"].cpu().numpy(), wy[r], err_msg=f"rank {r} routeWeightsSk")
+
+
 def test_home_plans_with_padding():
     """Plans as the reference's planner lays them out (expert groups padded to 8 rows, duplicates marked), fresh and
     saved, three exchanges back to back on one world without waiting in between."""

@@ -155,7 +155,7 @@ bool PrepareTables(WorldState *st, int world, int64_t nvS, int64_t n, WorldTable
     const int64_t groups = (rows + kChunkRows - 1) / kChunkRows;
     const int64_t perRank8 = stride * 8;
     // six 8-byte tables, two 4-byte tables, then the per-rank words
-    const int64_t bytes = world * (6 * perRank8 + 2 * stride * 4) + world * 8 + world * groups * 8 + 256;
+    const int64_t bytes = world * (6 * perRank8 + 2 * stride * 4 + stride) + world * 8 + world * groups * 8 + 256;
     if (!st->tables.Reserve(static_cast<size_t>(bytes), true)) {
         return false;
     }
@@ -175,6 +175,7 @@ bool PrepareTables(WorldState *st, int world, int64_t nvS, int64_t n, WorldTable
     out->sibling = reinterpret_cast<uint32_t *>(take(world * stride * 4));
     out->slotCount = reinterpret_cast<int32_t *>(take(world * stride * 4));
     out->chunkTotals = reinterpret_cast<int32_t *>(take(world * groups * 8));
+    out->direct = reinterpret_cast<uint8_t *>(take(world * stride));
     out->stride = stride;
     out->groupStride = groups;
     return true;

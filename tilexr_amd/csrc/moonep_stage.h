@@ -9,6 +9,7 @@
 // ever cleared between calls.
 //
 //   dispatch  walk      saved plans: parent records from dupGroups / dupLoffs
+//             agree     saved plans: per duplicate route, whether the plan's primary is the token's own primary row
 //             scatter   rows, weights, row tags; fresh plans: parent / sibling records of duplicates
 //             build     fresh plans: dupGroups / dupCounts from the parent records
 //             finish    per row: what is left to write (zeros, or a copy of the primary of a saved plan) and writing it;
@@ -49,6 +50,8 @@ struct WorldTables {
     uint64_t *slotDup;       // combine: per origin slot, epoch << 32 | 1 when that row is a duplicate (it does not travel)
     uint64_t *slotGroup;     // combine: per origin slot, epoch << 32 | first dupLoffs index when that row has duplicates
     int32_t *slotCount;      // combine: per origin slot, number of those duplicates (valid with slotGroup)
+    uint8_t *direct;         // dispatch, saved plans: per source route, 1 when the source writes the duplicate's row itself
+                             //           (rewritten for every route by every saved-plan dispatch)
     uint64_t *fail;          // [world] epoch << 32 | device status of the rank's own failure
     int32_t *chunkTotals;    // dispatch, fresh plans: [world][groupStride][2] group-opening rows and duplicates per chunk
     int64_t stride;          // >= nvS and >= n, a multiple of kTableAlign

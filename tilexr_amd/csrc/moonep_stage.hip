@@ -138,22 +138,44 @@ __device__ __forceinline__ void RouteRecords(const DispatchWorld &a, int src, in
 //   fresh plan   every route: the plan is being built from these very route words, so a duplicate row is by construction
 //                a copy of this token's row
 //   saved plan   non-duplicates; and a duplicate whose primary, according to the plan (parent records written by the walk
-//                kernel), is the row this token's own non-duplicate route to that rank writes -- the copy the fill kernel
-//                would make is a copy of this token's row.  Any other duplicate is left to the fill kernel.
+//                kernel), is the row this token's own non-duplicate route to that rank writes -- the copy the finish
+//                kernel would make is a copy of this token's row (`direct`, worked out by the agree kernel).  Any other
+//                duplicate is left to the finish kernel.
 template <bool FRESH>
-__device__ __forceinline__ bool SourceWrites(const DispatchWorld &a, const int32_t *words, int k, const Route &r, uint32_t *tagBits)
+__device__ __forceinline__ bool SourceWrites(const Route &r, uint8_t direct, uint32_t *tagBits)
 {
     if (FRESH || !r.duplicate) {
         *tagBits = kRowNamed | kRowWritten;
         return true;
     }
-    const uint64_t p = a.tables.parentTag[static_cast<int64_t>(r.peer) * a.tables.stride + r.row];
-    if (Tagged(p, a.epoch) && static_cast<int>(p & 0xffffffffu) - 1 == OwnPrimaryRow(a, words, k, r.peer)) {
+    if (direct != 0) {
         *tagBits = kRowNamed | kRowWritten | kRowDirect;
         return true;
     }
     *tagBits = kRowNamed;
     return false;
+}
+
+// Saved plans, one thread per route of source rank blockIdx.y: whether the source may write a duplicate's row itself
+// (see SourceWrites).  Done ahead of the scatter so that its workgroups find the answer with the route word, in one
+// round trip, instead of looking up the parent record after decoding it.
+__global__ __launch_bounds__(kThreads) void moon_agree_kernel(DispatchWorld a)
+{
+    const int src = blockIdx.y;
+    const int64_t route = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (route >= a.s * a.k) {
+        return;
+    }
+    const int K = static_cast<int>(a.k);
+    const int k = static_cast<int>(route % K);
+    const int32_t *words = a.dst[src] + route - k;
+    uint8_t direct = 0;
+    const Route r = Decode(words[k], a.nvS, a.world);
+    if (r.ok && r.duplicate) {
+        const uint64_t p = a.tables.parentTag[static_cast<int64_t>(r.peer) * a.tables.stride + r.row];
+        direct = Tagged(p, a.epoch) && static_cast<int>(p & 0xffffffffu) - 1 == OwnPrimaryRow(a, words, k, r.peer) ? 1 : 0;
+    }
+    a.tables.direct[static_cast<int64_t>(src) * a.tables.stride + route] = direct;
 }
 
 // One workgroup per (token, route, slice of 512 vectors) of source rank blockIdx.y.
@@ -182,6 +204,7 @@ __global__ __launch_bounds__(kThreads) void moon_scatter_kernel(DispatchWorld a,
         s_dst[lane] = words[lane];
     }
     const int32_t encoded = words[k];
+    const uint8_t direct = FRESH ? 0 : a.tables.direct[static_cast<int64_t>(src) * a.tables.stride + static_cast<int64_t>(token) * K + k];
     const u32x4 *srcRow = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.hiddenSh[src]) +
         static_cast<int64_t>(token) * h * 2);
     u32x4 v[kRowVecs];
@@ -198,7 +221,7 @@ __global__ __launch_bounds__(kThreads) void moon_scatter_kernel(DispatchWorld a,
         return;
     }
     uint32_t tagBits = 0;
-    if (SourceWrites<FRESH>(a, words, k, r, &tagBits)) {
+    if (SourceWrites<FRESH>(r, direct, &tagBits)) {
         u32x4 *dstRow = reinterpret_cast<u32x4 *>(static_cast<char *>(a.hiddenNvsh[r.peer]) + static_cast<int64_t>(r.row) * h * 2);
 #pragma unroll
         for (int i = 0; i < kRowVecs; ++i) {
@@ -240,7 +263,8 @@ __global__ __launch_bounds__(kThreads) void moon_scatter_generic_kernel(Dispatch
         return;
     }
     uint32_t tagBits = 0;
-    if (SourceWrites<FRESH>(a, words, k, r, &tagBits)) {
+    const uint8_t direct = FRESH ? 0 : a.tables.direct[static_cast<int64_t>(src) * a.tables.stride + static_cast<int64_t>(token) * K + k];
+    if (SourceWrites<FRESH>(r, direct, &tagBits)) {
         const uint16_t *srcRow = static_cast<const uint16_t *>(a.hiddenSh[src]) + static_cast<int64_t>(token) * a.h;
         uint16_t *dstRow = static_cast<uint16_t *>(a.hiddenNvsh[r.peer]) + static_cast<int64_t>(r.row) * a.h;
         for (int c = lane; c < a.h; c += kThreads) {
@@ -899,6 +923,9 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
     const unsigned rowBlocks = static_cast<unsigned>((w.nvS + kThreads - 1) / kThreads);
     if (!w.fresh) {
         hipLaunchKernelGGL(moon_group_walk_kernel, dim3(rowBlocks, R), dim3(kThreads), 0, stream, w);
+        MOON_LAUNCH_CHECK();
+        const unsigned routeBlocks = static_cast<unsigned>((w.s * w.k + kThreads - 1) / kThreads);
+        hipLaunchKernelGGL(moon_agree_kernel, dim3(routeBlocks, R), dim3(kThreads), 0, stream, w);
         MOON_LAUNCH_CHECK();
     }
     bool vec = w.h % 8 == 0;
