@@ -93,3 +93,35 @@ def test_layer_quantised_round_trip(quant):
         padded[:n] = deq.to(torch.bfloat16)
         ref = torch_combine_k_ordered(padded, d.row_map, weights)
         assert torch.equal(y.view(torch.int16), ref.to(torch.bfloat16).view(torch.int16))
+
+
+def test_plan_driven_layer_round_trip():
+    """The torch-facing wrapper of the plan-driven stages on a one-rank world: dispatch builds the duplicate plan on the
+    first call and follows it on the second; with an identity expert combine returns bf16(K * x); weights come back."""
+    from tilexr_amd.layer import PlanDrivenLayer
+    s, k, h = 300, 4, 1024
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(s, h, generator=g).to(torch.bfloat16).to(DEV)
+    w = torch.rand(s, k, generator=g).to(DEV)
+    nvs = s * k + 17
+    rows_of = torch.randperm(nvs, generator=g)[:s * k].to(torch.int32)
+    dst = rows_of.clone().reshape(s, k)
+    dst[:, 1:] = -dst[:, 1:] - 1                       # one rank: every route after a token's first is a duplicate
+    dst = dst.reshape(-1).to(DEV)
+    with PlanDrivenLayer(s, k, h, nvs=nvs) as layer:
+        layer.set_plan(dst)
+        for call in range(2):
+            rows, rw = layer.dispatch(x, w)
+            torch.cuda.synchronize()
+            assert int(layer.status[0].item()) == 2000
+            raw = rows_of.to(torch.int64).to(DEV)
+            assert torch.equal(rows[raw].view(torch.int16), x.repeat_interleave(k, dim=0).view(torch.int16)), f"call {call}"
+            assert torch.equal(rw[raw], w.reshape(-1))
+            unused = torch.ones(nvs, dtype=torch.bool, device=DEV)
+            unused[raw] = False
+            assert not rows[unused].view(torch.int16).any() and not rw[unused].any()
+        y, wy = layer.combine(rows, rw)
+        torch.cuda.synchronize()
+        assert int(layer.status[0].item()) == 0
+        assert torch.equal(y.view(torch.int16), (x.float() * k).to(torch.bfloat16).view(torch.int16))
+        assert torch.equal(wy, w)

@@ -127,3 +127,108 @@ class MoeEpLayer:
         ep.check(st, "TileXRMoeEpCombineMemoryEx")
         self._leave(expert_out, weights, y, mask, shared_expert_x, expert_out_scales)
         return y
+
+
+class PlanDrivenLayer:
+    """The plan-driven Dispatch / Combine stages (include/tilexr_moonep.h) for a world of one rank, as torch-style
+    methods: every route of the plan stays on this device.
+
+    A plan is the int32 tensor `dst [S * K]` of signed route words (row of the receive tensor, negated as `-row - 1` for
+    a duplicate: a later route of a token that already has one).  `dispatch` builds the duplicate plan on the first call
+    for a plan and follows the saved one afterwards; `combine` is its inverse with an fp32 sum per token."""
+
+    def __init__(self, tokens: int, top_k: int, hidden: int, nvs: int = 0, device="cuda:0"):
+        from . import moonep as mp
+        self._mp = mp
+        self.s, self.k, self.h = tokens, top_k, hidden
+        self.nvs = nvs if nvs > 0 else tokens * top_k
+        self.device = torch.device(device)
+        torch.cuda.set_device(self.device)
+        self.comm = ep.Comm(1, 0)
+        self.stream = torch.cuda.Stream(device=self.device)
+        dev = self.device
+        self._groups = torch.zeros((self.nvs, 3), dtype=torch.int32, device=dev)
+        self._loffs = torch.zeros((self.nvs,), dtype=torch.int32, device=dev)
+        self._counts = torch.zeros((2,), dtype=torch.int32, device=dev)
+        self.status = torch.zeros((4,), dtype=torch.int32, device=dev)
+        self._dst = None
+        self._dst_local = None
+        self._plan = None
+        self._built = False
+
+    def close(self):
+        if self.comm is not None:
+            torch.cuda.synchronize(self.device)
+            self.comm.destroy()
+            self.comm = None
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close()
+
+    def set_plan(self, dst: torch.Tensor):
+        """dst int32 [S * K] on the device; rows must lie in [0, nvs)."""
+        if dst.dtype != torch.int32 or dst.numel() != self.s * self.k:
+            raise ValueError("dst must be int32 with S * K entries")
+        mp = self._mp
+        self._dst = dst.contiguous()
+        raw = torch.where(self._dst >= 0, self._dst, -self._dst - 1).to(torch.int64)
+        # reverse routes: receive row -> rank * nvs + route (rank 0 here), -1 where no route lands
+        self._dst_local = torch.full((self.nvs,), -1, dtype=torch.int32, device=self.device)
+        self._dst_local[raw] = torch.arange(self.s * self.k, dtype=torch.int32, device=self.device)
+        self._plan = mp.plan(self.s * self.k, 1, self.k, 1, self.nvs, self.k, self._dst, self._groups, self._loffs,
+                             self._counts, self.status)
+        self._built = False
+
+    def _enter(self):
+        self.stream.wait_stream(torch.cuda.current_stream(self.device))
+
+    def _leave(self, *tensors):
+        torch.cuda.current_stream(self.device).wait_stream(self.stream)
+        for t in tensors:
+            if t is not None:
+                t.record_stream(self.stream)
+
+    def dispatch(self, x: torch.Tensor, weights: Optional[torch.Tensor] = None):
+        """x [S, hidden] bf16, weights [S, K] fp32 or None -> (rows [nvs, hidden] bf16, row_weights [nvs] fp32 or None)."""
+        mp = self._mp
+        if self._plan is None:
+            raise RuntimeError("set_plan() first")
+        if x.dtype != torch.bfloat16 or tuple(x.shape) != (self.s, self.h):
+            raise ValueError("x must be bfloat16 [S, hidden]")
+        x = x.contiguous()
+        rows = torch.empty((self.nvs, self.h), dtype=torch.bfloat16, device=self.device)
+        wsk = wnv = None
+        kwargs = {}
+        if weights is not None:
+            wsk = weights.to(torch.float32).contiguous()
+            wnv = torch.empty((self.nvs,), dtype=torch.float32, device=self.device)
+            kwargs = dict(weights_sk=mp.tensor(wsk, mp.DT_FP32, (self.s, self.k)), weights_nvs=mp.tensor(wnv, mp.DT_FP32, (self.nvs,)))
+        self._enter()
+        ep.check(mp.dispatch_v1(self.comm, self._plan, mp.tensor(x, mp.DT_BF16, (self.s, self.h)),
+                                mp.tensor(rows, mp.DT_BF16, (self.nvs, self.h)), self.stream,
+                                flags=0 if self._built else mp.FLAG_BUILD_DEDUP, **kwargs), "TileXRMoonEpDispatchV1")
+        self._built = True
+        self._leave(x, rows, wsk, wnv)
+        return rows, wnv
+
+    def combine(self, rows: torch.Tensor, row_weights: Optional[torch.Tensor] = None):
+        """rows [nvs, hidden] bf16 (expert outputs in the receive layout) -> (y [S, hidden] bf16, weights [S, K] or None)."""
+        mp = self._mp
+        if not self._built:
+            raise RuntimeError("dispatch() builds the duplicate plan combine needs")
+        rows = rows.contiguous()
+        y = torch.empty((self.s, self.h), dtype=torch.bfloat16, device=self.device)
+        wy = None
+        kwargs = {}
+        if row_weights is not None:
+            row_weights = row_weights.to(torch.float32).contiguous()
+            wy = torch.empty((self.s, self.k), dtype=torch.float32, device=self.device)
+            kwargs = dict(weights_nvs=mp.tensor(row_weights, mp.DT_FP32, (self.nvs,)), weights_sk=mp.tensor(wy, mp.DT_FP32, (self.s, self.k)))
+        self._enter()
+        ep.check(mp.combine_v1(self.comm, self._plan, self._dst_local, mp.tensor(rows, mp.DT_BF16, (self.nvs, self.h)),
+                               mp.tensor(y, mp.DT_BF16, (self.s, self.h)), self.stream, **kwargs), "TileXRMoonEpCombineV1")
+        self._leave(rows, row_weights, y, wy)
+        return y, wy
