@@ -76,24 +76,40 @@ def cpu_baseline(w, x, ids, weights, kept_rows):
     quant = {"none": O.Q_NONE, "int8": O.Q_TOKEN_INT8, "fp8_block128": O.Q_FP8_BLOCK128}[w.quant]
     case = O.Case(1, w.bs, w.h, w.top_k, w.experts, dtype=O.DT_BF16, quant_mode=quant, capacity=w.capacity)
     idn = ids.numpy()
-    best = None
-    for _ in range(3):
+    wn = weights.numpy()
+
+    def layer():
         t0 = time.perf_counter()
         d = O.mem_dispatch(case, 0, xb[None], idn[None])
         t1 = time.perf_counter()
         O.mem_combine(O.Case(1, w.bs, w.h, w.top_k, w.experts, dtype=O.DT_BF16), 0, d["expand_x"][None]
                       if quant else d["expand_x"].view(np.uint16)[None], d["assist"][None], d["send_counts"][None],
-                      expert_scales=weights.numpy(), in_quant=quant if quant else 0,
+                      expert_scales=wn, in_quant=quant if quant else 0,
                       in_scales=d["dyn_scales"] if quant else None)
         t2 = time.perf_counter()
-        if best is None or t2 - t0 < best[0]:
-            best = (t2 - t0, t1 - t0, t2 - t1)
+        return (t2 - t0, t1 - t0, t2 - t1)
+
+    best = min(layer() for _ in range(3))
     db, cb = workloads.algorithmic_bytes(w, kept_rows, inverse_index=True)
+    # All cores: the port is scalar, so the host's cores are used the way a host would use them for this path -- one
+    # independent layer per thread (the calls into the C library release the interpreter lock).
+    from concurrent.futures import ThreadPoolExecutor
+    threads = max(1, min(16, os.cpu_count() or 1))
+    many = None
+    with ThreadPoolExecutor(threads) as pool:
+        for _ in range(2):
+            t0 = time.perf_counter()
+            list(pool.map(lambda _i: layer(), range(threads)))
+            dt = time.perf_counter() - t0
+            many = dt if many is None else min(many, dt)
     return {
         "value": round((db + cb) / best[0] / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
         "us_per_layer": round(best[0] * 1e6, 1), "dispatch_us": round(best[1] * 1e6, 1),
         "combine_us": round(best[2] * 1e6, 1), "host_cores_available": os.cpu_count(),
         "sample": f"full {w.name} layer ({w.bs} tokens), oracle C port, single thread, best of 3",
+        "all_cores": {"value": round(threads * (db + cb) / many / 1e9, 3), "unit": "GB/s", "cores": threads,
+                      "us_per_layer": round(many / threads * 1e6, 1),
+                      "sample": f"{threads} independent {w.name} layers at once, one per thread, best of 2"},
     }
 
 
@@ -113,17 +129,29 @@ def moonep_cpu_baseline(world, s, k, h, experts):
     dst = plan["dst"].numpy()
     hidden = np.random.default_rng(1).integers(0, 0x4000, size=(world, sample, h), dtype=np.uint16)
     weights = np.ones((world, sample * k), np.float32)
-    best = None
-    for _ in range(3):
+    def layer():
         t0 = time.perf_counter()
         out, wout, _, dup = M.dispatch_world(sh, dst, hidden, weights, flags=M.FLAG_BUILD_DEDUP)
         t1 = time.perf_counter()
         M.combine_world(sh, M.build_dst_local(sh, dst), dup, out, wout)
         t2 = time.perf_counter()
-        if best is None or t2 - t0 < best[0]:
-            best = (t2 - t0, t1 - t0, t2 - t1)
+        return (t2 - t0, t1 - t0, t2 - t1)
+
+    best = min(layer() for _ in range(3))
     db, cb = workloads.moonep_algorithmic_bytes(sample, k, h)
+    from concurrent.futures import ThreadPoolExecutor
+    threads = max(1, min(16, os.cpu_count() or 1))
+    many = None
+    with ThreadPoolExecutor(threads) as pool:       # one independent layer per thread; the C calls release the lock
+        for _ in range(2):
+            t0 = time.perf_counter()
+            list(pool.map(lambda _i: layer(), range(threads)))
+            dt = time.perf_counter() - t0
+            many = dt if many is None else min(many, dt)
     return {
+        "all_cores": {"value": round(threads * world * (db + cb) / many / 1e9, 3), "unit": "GB/s", "cores": threads,
+                      "us_per_layer": round(many / threads * 1e6, 1),
+                      "sample": f"{threads} independent layers of the same sample at once, one per thread, best of 2"},
         "value": round(world * (db + cb) / best[0] / 1e9, 3), "unit": "GB/s", "cores": 1, "kind": "port",
         "us_per_layer": round(best[0] * 1e6, 1), "dispatch_us": round(best[1] * 1e6, 1),
         "combine_us": round(best[2] * 1e6, 1), "host_cores_available": os.cpu_count(),

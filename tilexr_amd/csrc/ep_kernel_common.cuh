@@ -46,6 +46,7 @@ __device__ __forceinline__ void LdsBarrier()
 // stays on: without it the written-through rows are also allocated in L2 and push out the input rows the sibling
 // workgroups of a token share (measured: 132 us instead of 93 us for the scatter).
 constexpr int kAuxAgentScope = 16 | 2;      // sc1 nt
+constexpr int kAuxNonTemporal = 2;          // nt
 constexpr unsigned kRawBufferWord3 = 0x00020000u;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t RowResource(const void *row, int bytes)

@@ -353,15 +353,21 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
                 const int k = k0 + u;
                 const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
                 rowOfK[u] = row;
-                const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
-                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
+                // Bounds are the buffer resources' business: an absent row gets resources of zero bytes, so its loads, like
+                // those of the lanes past the end of a row, return zeros without a branch (and without the register
+                // clears a branch would need).
+                const int64_t rowAt = row < 0 ? 0 : row;
+                const char *base = static_cast<const char *>(a.expertOut) + rowAt * a.rowBytes;
+                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, row < 0 ? 0 : vecs * 16);
+                const bool perRow = INQ == TILEXR_EP_QUANT_TOKEN_INT8;
+                const float *scaleBase = a.inScales + (perRow ? rowAt : rowAt * b128);
+                const __amdgpu_buffer_rsrc_t scaleRsrc = RowResource(scaleBase, row < 0 ? 0 : (perRow ? 4 : b128 * 4));
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
                     const int idx = j * G + lane;
-                    const bool live = row >= 0 && idx < vecs;
-                    q[u][j] = live ? RowLoad<FL>(base, rsrc, idx * 16) : u32x4{0u, 0u, 0u, 0u};
-                    sc[u][j] = !live ? 0.0f : (INQ == TILEXR_EP_QUANT_TOKEN_INT8 ? ScaleLoad<FL>(a.inScales + row) :
-                        ScaleLoad<FL>(a.inScales + static_cast<int64_t>(row) * b128 + (idx >> 3)));
+                    q[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 16, 0, FL ? kAuxAgentScope : kAuxNonTemporal);
+                    sc[u][j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scaleRsrc, perRow ? 0 : (idx >> 3) * 4, 0,
+                        FL ? kAuxAgentScope : 0));
                 }
             }
 #pragma unroll
