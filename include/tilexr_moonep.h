@@ -27,7 +27,12 @@
  * All tensors are caller-owned device memory; every call is asynchronous on `stream` (a hipStream_t carried as the
  * reference's opaque aclrtStream); validation happens before a magic is drawn or anything is enqueued.  With more than
  * one rank in the communicator's world every rank must make the call (any order, any host thread, its own stream): a
- * rank's outputs are complete once all ranks have called and its stream has been synchronised.
+ * rank's outputs are complete once all ranks have called and its stream has been synchronised.  The ranks of a world
+ * must agree on S, K, H, NvS, the flags and on whether weights travel.  A call that disagrees with the calls already
+ * filed for the same exchange returns INVALID_ARGUMENT and cancels them: each cancelled rank finds the remote-failure
+ * status naming the disagreeing rank in its plan->status[0] (stored in the order of its stream), its outputs are left
+ * as they were, and every rank has to call again.  A second call of one rank while its first still waits for its
+ * peers returns INTERNAL.
  *
  * Differences from the reference, all deliberate:
  *   - a world of ONE rank is accepted by both stages (the reference's combine needs at least two,

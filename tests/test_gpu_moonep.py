@@ -347,17 +347,24 @@ def test_argument_rules_on_the_device():
         assert mp.dispatch_v1(*args, flags=mp.FLAG_ZERO_COPY) == mp.ERR_NOT_SUPPORTED
         assert mp.dispatch_v1(*args, flags=1 << 20) == mp.ERR_INVALID_ARGUMENT
         assert mp.dispatch_v1(*args[:4], None) == mp.ERR_INVALID_ARGUMENT
-        # rank 0 files a call; rank 1 disagrees about the flags and is refused; then agrees and the exchange runs
+        # rank 0 files a call and may not file another while it waits; rank 1 disagrees about the flags: it is refused
+        # and rank 0's call is cancelled with rank 1 named as the failed peer; then both call again and the exchange runs
         assert mp.dispatch_v1(*args, flags=mp.FLAG_BUILD_DEDUP) == mp.SUCCESS
+        assert mp.dispatch_v1(*args, flags=mp.FLAG_BUILD_DEDUP) == mp.ERR_INTERNAL
         x1 = dev_bits16(hidden[1])
         out1 = torch.zeros((sh.nvs, h), dtype=torch.bfloat16, device=DEV)
         torch.cuda.synchronize()
         args1 = (w.comms[1], plans[1]["desc"], mp.tensor(x1, mp.DT_BF16, (s, h)), mp.tensor(out1, mp.DT_BF16, (sh.nvs, h)),
                  w.streams[1])
         assert mp.dispatch_v1(*args1, flags=0) == mp.ERR_INVALID_ARGUMENT
-        assert mp.dispatch_v1(*args, flags=mp.FLAG_BUILD_DEDUP) == mp.ERR_INTERNAL      # rank 0 already has a call waiting
-        assert mp.dispatch_v1(*args1, flags=mp.FLAG_BUILD_DEDUP) == mp.SUCCESS
         w.sync()
+        assert int(plans[0]["status"][0].item()) == mp.DISPATCH_STATUS_REMOTE_FAILURE_BASE + 1
+        assert int(plans[1]["status"][0].item()) == -1          # the refused call left nothing behind
+        assert not out.view(torch.int16).any().item()           # and the cancelled one wrote no row
+        assert mp.dispatch_v1(*args1, flags=mp.FLAG_BUILD_DEDUP) == mp.SUCCESS
+        assert mp.dispatch_v1(*args, flags=mp.FLAG_BUILD_DEDUP) == mp.SUCCESS
+        w.sync()
+        assert int(plans[0]["status"][0].item()) == int(plans[1]["status"][0].item()) == mp.DISPATCH_STATUS_SUCCESS
         want = M.dispatch_world(sh, dst, hidden, flags=M.FLAG_BUILD_DEDUP)
         np.testing.assert_array_equal(host_bits16(out), want[0][0])
         np.testing.assert_array_equal(host_bits16(out1), want[0][1])

@@ -383,6 +383,17 @@ int Arrive(EpComm *comm, const StageCall &call, bool combine)
     }
     for (const StageCall &c : calls) {
         if (c.present && !SameShape(c, call)) {
+            // The world cannot run this exchange.  The calls already filed for it are dropped, each with this rank
+            // named in its device status as the peer that failed (what a peer's bad plan leaves there in the
+            // reference: src/moonep/dispatch/kernels/tilexr_moonep_dispatch_kernel.cpp:512,
+            // src/moonep/combine/kernels/tilexr_moonep_combine_kernel.cpp:423), so that the world is usable again.
+            const int32_t failure = (combine ? kCombineRemoteFailureBase : kDispatchRemoteFailureBase) + comm->rank;
+            for (StageCall &waiting : calls) {
+                if (waiting.present && waiting.status != nullptr) {
+                    (void)LaunchMoonStatus(waiting.status, failure, waiting.stream);
+                }
+                waiting.present = false;
+            }
             return kInvalid;
         }
     }

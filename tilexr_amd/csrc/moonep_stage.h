@@ -102,6 +102,9 @@ struct LaunchTiming {
 hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const LaunchTiming &scatterTiming);
 hipError_t LaunchMoonCombine(const CombineWorld &w, hipStream_t stream, const LaunchTiming &reduceTiming);
 
+// Stores one device status word in stream order.
+hipError_t LaunchMoonStatus(int32_t *status, int32_t value, hipStream_t stream);
+
 // Names of the kernel templates the last scatter / reduce launch used (for the benchmark's roofline line).
 const char *MoonScatterKernelName();
 const char *MoonReduceKernelName();

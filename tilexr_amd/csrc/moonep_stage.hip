@@ -907,6 +907,20 @@ hipError_t RecordIf(hipEvent_t e, hipStream_t stream)
 
 } // namespace
 
+// One device status word, written in stream order (a call that was dropped because a peer's call disagreed with it).
+__global__ void moon_status_kernel(int32_t *status, int32_t value)
+{
+    if (threadIdx.x == 0 && blockIdx.x == 0) {
+        status[0] = value;
+    }
+}
+
+hipError_t LaunchMoonStatus(int32_t *status, int32_t value, hipStream_t stream)
+{
+    hipLaunchKernelGGL(moon_status_kernel, dim3(1), dim3(kWave), 0, stream, status, value);
+    return hipGetLastError();
+}
+
 const char *MoonScatterKernelName()
 {
     return gScatterName;
