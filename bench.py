@@ -57,6 +57,8 @@ def parse():
     p.add_argument("--no-overlap-leg", action="store_true",
                    help="skip the extra, separately timed run of the other schedule that is reported under "
                         "config.other_schedule")
+    p.add_argument("--no-rotate-leg", action="store_true",
+                   help="skip the extra leg that feeds every step a different input tensor (inputs not cache-resident)")
     p.add_argument("--event-stride", type=int, default=10,
                    help="record the per-kernel events on every N-th timed step")
     p.add_argument("--calibrate-copy", action="store_true",
@@ -354,7 +356,7 @@ def main():
     status = torch.zeros((1,), dtype=torch.int32, device=dev)
     meta_ready, combined = ep.HipEvent(), ep.HipEvent()
 
-    def step_serial():
+    def step_serial(d_x=d_x):
         st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
                                       ep.DT_BF16, stream, quant_mode=quant, expert_capacity=w.capacity,
                                       dynamic_scales=scales, row_index_map=row_map)
@@ -459,6 +461,26 @@ def main():
                  "steps": other_steps, "us_per_layer": round(other_us, 2),
                  "GBps": round((dispatch_bytes + combine_bytes) / (other_us * 1e-6) / 1e9, 1)}
 
+    # the serial schedule once more with the token rows of every step in a different tensor, enough of them that none
+    # is still in the 256 MiB memory-side cache when its turn comes again: what a caller sees whose x was produced long
+    # before the dispatch.  Not part of `value`.
+    rotating = None
+    if not args.no_rotate_leg:
+        copies = max(2, -(-(384 << 20) // (bs * h * 2)))
+        xs = [d_x] + [d_x.clone() for _ in range(copies - 1)]
+        rot_steps = max(copies, args.steps // 2)
+        for i in range(copies):
+            step_serial(xs[i])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(rot_steps):
+            step_serial(xs[i % copies])
+        torch.cuda.synchronize()
+        rot_us = (time.perf_counter() - t1) / rot_steps * 1e6
+        rotating = {"schedule": "serial", "input_tensors": copies, "steps": rot_steps, "us_per_layer": round(rot_us, 2),
+                    "GBps": round((dispatch_bytes + combine_bytes) / (rot_us * 1e-6) / 1e9, 1)}
+        del xs
+
     ms_per_step = elapsed / args.steps * 1e3
     total_bytes = dispatch_bytes + combine_bytes
     gbps = total_bytes / (ms_per_step * 1e-3) / 1e9
@@ -486,7 +508,7 @@ def main():
         "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": dict(workloads.describe(w, ids), schedule="overlapped via tile flags" if args.overlap else "serial",
-                       other_schedule=other, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+                       other_schedule=other, rotating_inputs=rotating, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
         "roofline": roofline, "kernels": kernels,
     }

@@ -197,6 +197,13 @@ int TileXRMoonEpDispatchV1(const TileXRMoonEpDispatchArgsV1 *args, aclrtStream s
  * (what is computed). */
 int TileXRMoonEpCombineV1(const TileXRMoonEpCombineArgsV1 *args, aclrtStream stream);
 
+/* No counterpart in the reference: a tuning knob of this library.  Dispatch copies token rows with one of two kernels:
+ * the faster one when the rows are still in the device's memory-side cache (256 MiB on MI355X), one that keeps most of
+ * its speed when they have to come from HBM.  It picks by the bytes of token rows of the whole world (ranks * S * H * 2)
+ * against the value set here (default 256 MiB; 0 = always the HBM-tolerant kernel).  Process-wide, thread-safe;
+ * returns the previous value.  Results do not depend on it. */
+int64_t TileXRMoonEpSetCachedRowBytes(int64_t bytes);
+
 #ifdef __cplusplus
 }
 #endif

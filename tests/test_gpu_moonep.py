@@ -155,8 +155,16 @@ CASES = [
 ]
 
 
+@pytest.fixture(params=["rows_cached", "rows_uncached"])
+def row_cache(request):
+    """Both scatter kernels: the library picks by the bytes of token rows against this setting."""
+    previous = mp.set_cached_row_bytes(0 if request.param == "rows_uncached" else 1 << 40)
+    yield "moon_scatter_token_kernel" if request.param == "rows_uncached" else "moon_scatter_kernel"
+    mp.set_cached_row_bytes(previous)
+
+
 @pytest.mark.parametrize("world,s,k,h,slack,with_weights,dups", CASES)
-def test_dispatch_and_combine_match_oracle(world, s, k, h, slack, with_weights, dups):
+def test_dispatch_and_combine_match_oracle(world, s, k, h, slack, with_weights, dups, row_cache):
     rng = np.random.default_rng(world * 1000 + s * 10 + k)
     sh = M.Shape(world, s, k, h, s * k + slack)
     dst = MC.random_dst(sh, rng, duplicates=dups)
@@ -168,6 +176,8 @@ def test_dispatch_and_combine_match_oracle(world, s, k, h, slack, with_weights, 
         res = w.dispatch(sh, plans, hidden, weights, flags=mp.FLAG_BUILD_DEDUP, order=list(rng.permutation(world)))
         w.sync()
         check_dispatch(sh, res, plans, want, fresh=True)
+        if h % 8 == 0:
+            assert ep.last_kernel_name(w.comms[0], ep.K_SCATTER) == row_cache
         # saved plan on the same world: same rows, the plan's arrays are left as they are
         before = [(p["groups"].clone(), p["loffs"].clone(), p["counts"].clone()) for p in plans]
         res2 = w.dispatch(sh, plans, hidden, weights, flags=0)
@@ -192,7 +202,7 @@ def test_dispatch_and_combine_match_oracle(world, s, k, h, slack, with_weights, 
 
 
 @pytest.mark.parametrize("seed", range(24))
-def test_random_shapes(seed):
+def test_random_shapes(seed, row_cache):
     """Small random worlds, hidden sizes on both sides of the vector / element-wise split, fresh and saved plans."""
     rng = np.random.default_rng(1000 + seed)
     world = int(rng.choice([1, 2, 3, 5, 8]))
@@ -258,7 +268,7 @@ def test_home_plans_with_padding():
                 np.testing.assert_array_equal(cres[r]["wy"].cpu().numpy().reshape(-1), weights[r])
 
 
-def test_saved_plan_is_followed_as_given():
+def test_saved_plan_is_followed_as_given(row_cache):
     """A saved plan is data: an empty one leaves duplicate rows zero, and a plan in the CPU model's group order gives
     the same rows as the one the kernels build."""
     world, s, k, h = 2, 12, 4, 64
@@ -283,7 +293,7 @@ def test_saved_plan_is_followed_as_given():
         check_dispatch(sh, res, plans, M.dispatch_world(sh, dst, hidden, flags=0, dup=shuffled), fresh=False)
 
 
-def test_device_status_of_bad_plans():
+def test_device_status_of_bad_plans(row_cache):
     world, s, k, h = 3, 8, 2, 64
     rng = np.random.default_rng(9)
     sh = M.Shape(world, s, k, h, s * k)

@@ -94,6 +94,10 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     count.expertTokenNumsOut = p.expertTokenNumsOut;
     count.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
     count.stream = stream;
+    // the scatter kernel that copies per route wants the token rows close by
+    const bool warm = ScatterCopiesPerRoute(p.x, p.expandXOut, p.bs, p.h, p.topK, static_cast<int>(p.quantMode));
+    count.warmRows = warm ? p.x : nullptr;
+    count.warmBytes = p.bs * p.h * 2;
     int ret = Timed(comm, kKernelCount, stream, "route count", [&] { return LaunchRouteCount(count); });
     if (ret != kOk) {
         return ret;

@@ -63,6 +63,10 @@ struct RouteCountLaunch {
     int32_t *recvCountOut;       // [1] total kept rows
     int64_t *expertTokenNumsOut; // [experts]
     int tokenNumsType;
+    // Token rows the scatter that follows will read: extra workgroups of this launch read them once while the counting
+    // workgroups wait on their own small loads, which leaves the rows in the memory-side cache.  Null or 0: none.
+    const void *warmRows;
+    int64_t warmBytes;
     hipStream_t stream;
 };
 
@@ -193,6 +197,10 @@ hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l);
 hipError_t LaunchRouteCount(const RouteCountLaunch &l);
 hipError_t LaunchRoutePlace(const RoutePlaceLaunch &l);
 hipError_t LaunchScatter(const ScatterLaunch &l);
+// Whether LaunchScatter copies rows with one workgroup per (route, slice), each reading its own copy of the token row
+// (plain payload, wide rows, 1024 tokens and more).  That kernel is the one that needs the token rows close by: it is
+// what RouteCountLaunch::warmRows is for.
+bool ScatterCopiesPerRoute(const void *x, const void *out, int64_t bs, int64_t h, int64_t topK, int quantMode);
 hipError_t LaunchInvert(const InvertLaunch &l);
 hipError_t LaunchReduce(const ReduceLaunch &l);
 

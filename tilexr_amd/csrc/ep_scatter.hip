@@ -480,8 +480,7 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
     switch (l.quantMode) {
         case TILEXR_EP_QUANT_NONE:
             // small batches are latency-bound and gain nothing from the extra workgroups
-            if (G == kThreads && a.topK > 1 && a.bs >= 1024 &&
-                static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK * a.colSlices <= 0x7fffffff) {
+            if (G == kThreads && ScatterCopiesPerRoute(l.x, l.out, l.bs, l.h, l.topK, l.quantMode)) {
                 const dim3 blocks(static_cast<unsigned>(static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK * a.colSlices));
                 if (l.kernelNameOut != nullptr) {
                     *l.kernelNameOut = "ep_scatter_route_kernel";
@@ -533,6 +532,16 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
 }
 
 } // namespace
+
+bool ScatterCopiesPerRoute(const void *x, const void *out, int64_t bs, int64_t h, int64_t topK, int quantMode)
+{
+    const int64_t vecs = h / 8;
+    const int64_t slices = (vecs + kRouteVecs * kThreads - 1) / (kRouteVecs * kThreads);
+    // token rows beyond half the memory-side cache (256 MiB) cannot be kept close by: the per-token kernel takes those
+    return quantMode == TILEXR_EP_QUANT_NONE && h % 8 == 0 && Aligned16(x) && Aligned16(out) && vecs > 4 * kWave &&
+        vecs <= 8 * kThreads && topK > 1 && bs >= 1024 && bs * h * 2 <= (int64_t{128} << 20) &&
+        (bs + 7) / 8 * 8 * topK * slices <= 0x7fffffff;
+}
 
 hipError_t LaunchScatter(const ScatterLaunch &l)
 {

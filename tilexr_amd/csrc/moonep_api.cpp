@@ -542,6 +542,11 @@ int TileXRMoonEpGetCapabilitiesV2(uint64_t *nativeStages, uint64_t *stubStages)
     return TileXRMoonEpGetCapabilitiesV1(nativeStages, stubStages);
 }
 
+int64_t TileXRMoonEpSetCachedRowBytes(int64_t bytes)
+{
+    return TileXRMoon::SetCachedRowBytes(bytes);
+}
+
 int TileXRMoonEpDispatchV1(const TileXRMoonEpDispatchArgsV1 *args, aclrtStream stream)
 {
     TileXREp::EpComm *comm = nullptr;

@@ -105,6 +105,10 @@ hipError_t LaunchMoonCombine(const CombineWorld &w, hipStream_t stream, const La
 // Stores one device status word in stream order.
 hipError_t LaunchMoonStatus(int32_t *status, int32_t value, hipStream_t stream);
 
+// Bytes of token rows (all ranks of a world together) up to which the scatter assumes that they are still in the
+// device's memory-side cache when it runs; returns the previous value.  Default 256 MiB.
+int64_t SetCachedRowBytes(int64_t bytes);
+
 // Names of the kernel templates the last scatter / reduce launch used (for the benchmark's roofline line).
 const char *MoonScatterKernelName();
 const char *MoonReduceKernelName();

@@ -18,7 +18,7 @@ DISPATCH_STATUS_SUCCESS, DISPATCH_STATUS_INVALID_ROUTE, DISPATCH_STATUS_REMOTE_F
 COMBINE_STATUS_SUCCESS, COMBINE_STATUS_INVALID_ROUTE, COMBINE_STATUS_REMOTE_FAILURE_BASE = 0, 3001, 3100
 
 EXPORTS = ("TileXRMoonEpGetAbiVersion", "TileXRMoonEpGetCapabilitiesV1", "TileXRMoonEpGetCapabilitiesV2",
-           "TileXRMoonEpDispatchV1", "TileXRMoonEpCombineV1")
+           "TileXRMoonEpDispatchV1", "TileXRMoonEpCombineV1", "TileXRMoonEpSetCachedRowBytes")
 
 
 class TensorV1(C.Structure):
@@ -77,6 +77,15 @@ def lib():
 
 def abi_version():
     return lib().TileXRMoonEpGetAbiVersion()
+
+
+def set_cached_row_bytes(nbytes):
+    """Bytes of token rows up to which dispatch assumes they are still in the device's memory-side cache (picks the
+    scatter kernel); returns the previous value."""
+    fn = lib().TileXRMoonEpSetCachedRowBytes
+    fn.argtypes = [C.c_int64]
+    fn.restype = C.c_int64
+    return fn(int(nbytes))
 
 
 def capabilities(version=1):
