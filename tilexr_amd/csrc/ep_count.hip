@@ -54,7 +54,7 @@ struct RouteCountArgs {
     int64_t warmVecs;
 };
 
-constexpr int kWarmLoads = 8;    // 16-byte loads in flight per lane of a warming workgroup (32 KiB per workgroup)
+constexpr int kWarmLoads = 2;    // 16-byte loads per lane of a warming workgroup (8 KiB per workgroup; 11.4 us for 58.7 MB, 14.3 us with eight)
 
 // BPW = batches of 64 routes per wave: a workgroup counts 256 * BPW consecutive routes.
 template <int BPW>
@@ -75,7 +75,7 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     const bool expHist = a.s.chunkExpHist != nullptr;
 
     if (a.warmRows != nullptr && chunk >= a.numChunks) {
-        // Not a counting workgroup: reads 32 KiB of the token rows and drops them.  The scatter that follows finds the
+        // Not a counting workgroup: reads 8 KiB of the token rows and drops them.  The scatter that follows finds the
         // rows in the memory-side cache; when it has to fetch them from HBM between its own writes it runs at little
         // more than half its speed (4096 x 7168 x top-8: 140 us instead of 83).
         const int64_t base = static_cast<int64_t>(chunk - a.numChunks) * (kThreads * kWarmLoads) + tid;
