@@ -57,6 +57,9 @@ def parse():
     p.add_argument("--no-overlap-leg", action="store_true",
                    help="skip the extra, separately timed run of the other schedule that is reported under "
                         "config.other_schedule")
+    p.add_argument("--moon-cached-row-bytes", type=int, default=None,
+                   help="M1: value for TileXRMoonEpSetCachedRowBytes (0 = always the scatter kernel that tolerates "
+                        "token rows that come from HBM)")
     p.add_argument("--no-rotate-leg", action="store_true",
                    help="skip the extra leg that feeds every step a different input tensor (inputs not cache-resident)")
     p.add_argument("--event-stride", type=int, default=10,
@@ -208,6 +211,8 @@ def main_moonep(args):
             ep.check(mp.combine_v1(comms[r], t["plan"], t["dl"], *t["c_args"], streams[r], **t["c_w"]), "combine")
 
     flags = 0 if args.moon_saved else mp.FLAG_BUILD_DEDUP
+    if args.moon_cached_row_bytes is not None:
+        mp.set_cached_row_bytes(args.moon_cached_row_bytes)
 
     def step():
         dispatch(flags)
@@ -270,6 +275,32 @@ def main_moonep(args):
     else:
         split = (None, None)
 
+    # one rank once more with the token rows of every step in a different tensor, enough of them that none is still in
+    # the 256 MiB memory-side cache when its turn comes again.  Not part of `value`.
+    rotating = None
+    if world == 1 and not args.no_rotate_leg:
+        copies = max(2, -(-(384 << 20) // (s * h * 2)))
+        xs = [r0["x"]] + [r0["x"].clone() for _ in range(copies - 1)]
+        descs = [mp.tensor(x, mp.DT_BF16, (s, h)) for x in xs]
+        rot_steps = max(copies, args.steps // 2)
+
+        def rot_step(i):
+            ep.check(mp.dispatch_v1(comms[0], r0["plan"], descs[i % copies], r0["d_args"][1], streams[0], flags=flags,
+                                    **r0["d_w"]), "dispatch")
+            combine()
+
+        for i in range(copies):
+            rot_step(i)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(rot_steps):
+            rot_step(i)
+        torch.cuda.synchronize()
+        rot_us = (time.perf_counter() - t1) / rot_steps * 1e6
+        rotating = {"input_tensors": copies, "steps": rot_steps, "us_per_layer": round(rot_us, 2),
+                    "GBps": round((dispatch_bytes + combine_bytes) / (rot_us * 1e-6) / 1e9, 1)}
+        del xs, descs
+
     ms_per_step = elapsed / args.steps * 1e3
     total_bytes = world * (dispatch_bytes + combine_bytes)
     gbps = total_bytes / (ms_per_step * 1e-3) / 1e9
@@ -297,7 +328,7 @@ def main_moonep(args):
         "config": {"workload": f"{w.name}: plan-driven Dispatch + Combine, {world} logical rank(s) x {s} tokens x {h} bf16, "
                                f"top-{k} of {experts} experts, home plan, fp32 route weights",
                    "logical_ranks": world, "tokens_per_rank": s, "hidden": h, "top_k": k, "experts": experts, "nvs": nvs,
-                   "duplicate_routes": int((dst < 0).sum()), "routes": int(dst.numel()),
+                   "duplicate_routes": int((dst < 0).sum()), "routes": int(dst.numel()), "rotating_inputs": rotating,
                    "dispatch": "saved duplicate plan" if args.moon_saved else "builds the duplicate plan",
                    "dispatch_bytes_per_rank": dispatch_bytes, "combine_bytes_per_rank": combine_bytes,
                    "dispatch_us": split[0], "combine_us": split[1], "seed": w.seed,
