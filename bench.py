@@ -512,6 +512,32 @@ def main():
                     "GBps": round((dispatch_bytes + combine_bytes) / (rot_us * 1e-6) / 1e9, 1)}
         del xs
 
+    # the same layer through the reference's own entry points (TileXRMoeEpDispatchMemory / TileXRMoeEpCombineMemoryV2),
+    # which carry no row map from dispatch to combine: combine rebuilds it from the assist tuples first.  Plain
+    # payloads only (the quantised workloads need the extended calls).  Not part of `value`.
+    reference_abi = None
+    if quant == ep.Q_NONE and w.capacity == 0 and not args.no_rotate_leg:
+        ref_steps = max(10, args.steps // 2)
+        ref_x = expand_x.view(torch.bfloat16)
+
+        def step_reference():
+            ep.check(ep.dispatch_memory(d_x, d_ids, comm, bs, h, K, E, ref_x, token_nums, send_counts, assist, ep.DT_BF16,
+                                        stream), "dispatch")
+            ep.check(ep.combine_memory_v2(ref_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
+                                          expert_scales=d_w), "combine")
+
+        for _ in range(5):
+            step_reference()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for _ in range(ref_steps):
+            step_reference()
+        torch.cuda.synchronize()
+        ref_us = (time.perf_counter() - t1) / ref_steps * 1e6
+        reference_abi = {"entry_points": "TileXRMoeEpDispatchMemory + TileXRMoeEpCombineMemoryV2", "steps": ref_steps,
+                         "us_per_layer": round(ref_us, 2),
+                         "GBps": round((dispatch_bytes + combine_bytes + kept_rows * 16 - bs * K * 4) / (ref_us * 1e-6) / 1e9, 1)}
+
     ms_per_step = elapsed / args.steps * 1e3
     total_bytes = dispatch_bytes + combine_bytes
     gbps = total_bytes / (ms_per_step * 1e-3) / 1e9
@@ -539,7 +565,7 @@ def main():
         "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": dict(workloads.describe(w, ids), schedule="overlapped via tile flags" if args.overlap else "serial",
-                       other_schedule=other, rotating_inputs=rotating, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+                       other_schedule=other, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
         "roofline": roofline, "kernels": kernels,
     }
