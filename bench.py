@@ -60,6 +60,8 @@ def parse():
     p.add_argument("--moon-cached-row-bytes", type=int, default=None,
                    help="M1: value for TileXRMoonEpSetCachedRowBytes (0 = always the scatter kernel that tolerates "
                         "token rows that come from HBM)")
+    p.add_argument("--no-ceilings", action="store_true",
+                   help="skip the memory-system yardsticks (probe kernels of the library) reported under `ceilings`")
     p.add_argument("--no-rotate-leg", action="store_true",
                    help="skip the extra leg that feeds every step a different input tensor (inputs not cache-resident)")
     p.add_argument("--event-stride", type=int, default=10,
@@ -68,6 +70,41 @@ def parse():
                    help="also launch a plain 256 MiB read + 256 MiB write kernel before the warm-up, as the known-size "
                         "yardstick for hardware-counter runs")
     return p.parse_args()
+
+
+def measured_ceilings(ep, torch, stream, dev, reps=10):
+    """What this device's memory system delivers for plain access patterns, measured in this run with the library's
+    own probe kernels (HIP events around `reps` launches each): pure read, pure write, copy, and the read : write
+    mixes of the scatter (1 : 8) and the reduce (8 : 1).  GB/s of all bytes moved, reads plus writes.  The mixed
+    patterns depend on how far apart their eight regions lie (5.6 to 6.6 TB/s for the 1 : 8 mix between 56 and 125 MiB),
+    so they are run at three sizes and the best is kept: a ceiling, not an average."""
+    patterns = {"read": ep.PROBE_READ, "write": ep.PROBE_WRITE, "copy": ep.PROBE_COPY, "fan_out_1r8w": ep.PROBE_FAN_OUT,
+                "fan_in_8r1w": ep.PROBE_FAN_IN}
+    sizes = (448, 472, 1000)
+    out = {"buffer_MiB": list(sizes), "launches": reps}
+    for mib in sizes:
+        nbytes = mib << 20
+        src = torch.zeros((nbytes,), dtype=torch.uint8, device=dev)
+        dst = torch.zeros((nbytes,), dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+        moved = {"read": nbytes, "write": nbytes, "copy": 2 * nbytes, "fan_out_1r8w": nbytes + nbytes // 8,
+                 "fan_in_8r1w": nbytes + nbytes // 8}
+        for name, pattern in patterns.items():
+            if mib != sizes[0] and not name.startswith("fan"):
+                continue
+            for _ in range(3):
+                ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+            a, b = ep.HipEvent(timing=True), ep.HipEvent(timing=True)
+            a.record(stream)
+            for _ in range(reps):
+                ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+            b.record(stream)
+            stream.synchronize()
+            us = a.elapsed_ms(b) * 1e3 / reps
+            rate = round(moved[name] / (us * 1e-6) / 1e9, 1)
+            out[name + "_GBps"] = max(rate, out.get(name + "_GBps", 0.0))
+        del src, dst
+    return out
 
 
 def cpu_baseline(w, x, ids, weights, kept_rows):
@@ -318,6 +355,12 @@ def main_moonep(args):
                     "unit": "GB/s", "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4),
                     "traffic": measured_traffic(f"{w.name}_r{world}", dom), "avg_launch_us": kernels[dom]["avg_us"],
                     "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
+    ceilings = None
+    if not args.no_ceilings:
+        ceilings = measured_ceilings(ep, torch, streams[0], dev)
+        if roofline is not None:
+            mix = ceilings["fan_out_1r8w_GBps"] if dom == "scatter" else ceilings["fan_in_8r1w_GBps"]
+            roofline["frac_of_measured_mix"] = round(roofline["achieved"] / mix, 4)
     result = {
         "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -333,7 +376,7 @@ def main_moonep(args):
                    "dispatch_bytes_per_rank": dispatch_bytes, "combine_bytes_per_rank": combine_bytes,
                    "dispatch_us": split[0], "combine_us": split[1], "seed": w.seed,
                    "dst_sha256": __import__("hashlib").sha256(dst.numpy().tobytes()).hexdigest()[:16]},
-        "roofline": roofline, "kernels": kernels,
+        "roofline": roofline, "kernels": kernels, "ceilings": ceilings,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = moonep_cpu_baseline(world, s, k, h, experts)
@@ -558,6 +601,13 @@ def main():
                     "traffic": measured_traffic(w.name, dom),
                     "avg_launch_us": kernels[dom]["avg_us"], "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
 
+    ceilings = None
+    if not args.no_ceilings:
+        ceilings = measured_ceilings(ep, torch, stream, dev)
+        if roofline is not None:
+            mix = ceilings["fan_out_1r8w_GBps"] if dom == "scatter" else ceilings["fan_in_8r1w_GBps"]
+            roofline["frac_of_measured_mix"] = round(roofline["achieved"] / mix, 4)
+
     result = {
         "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -567,7 +617,7 @@ def main():
         "config": dict(workloads.describe(w, ids), schedule="overlapped via tile flags" if args.overlap else "serial",
                        other_schedule=other, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
-        "roofline": roofline, "kernels": kernels,
+        "roofline": roofline, "kernels": kernels, "ceilings": ceilings,
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline(w, x, ids, weights, kept_rows)

@@ -187,6 +187,25 @@ const char *TileXREpLastKernelName(TileXRCommPtr comm, int kernel);
 // Library build identification ("tilexr-ep gfx950 <abi version>").
 const char *TileXREpVersion(void);
 
+// Measurement aid without a reference counterpart: one launch of a kernel that does nothing but the memory traffic of
+// a given pattern, so that a harness can time what this device's memory system delivers for the read : write mix of
+// the scatter and reduce kernels.  `bytes` is the size of the larger side and a multiple of 128; pointers are device
+// memory, 16-byte aligned.
+//   READ     reads `bytes` of src                     (dst: at least 4 bytes, not written in practice)
+//   WRITE    writes `bytes` of dst                    (src unused)
+//   COPY     reads `bytes` of src, writes `bytes` of dst
+//   FAN_OUT  reads bytes / 8 of src, writes `bytes` of dst as eight copies   (the scatter's 1 : 8 mix)
+//   FAN_IN   reads `bytes` of src as eight regions, writes bytes / 8 of dst  (the reduce's 8 : 1 mix)
+// Asynchronous on `stream`; returns 0, -3 for bad arguments, -2 when the launch fails.
+enum TileXREpProbePattern {
+    TILEXR_EP_PROBE_READ = 0,
+    TILEXR_EP_PROBE_WRITE = 1,
+    TILEXR_EP_PROBE_COPY = 2,
+    TILEXR_EP_PROBE_FAN_OUT = 3,
+    TILEXR_EP_PROBE_FAN_IN = 4
+};
+int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int64_t bytes, aclrtStream stream);
+
 }
 
 #endif // __cplusplus

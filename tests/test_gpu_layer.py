@@ -125,3 +125,45 @@ def test_plan_driven_layer_round_trip():
         assert int(layer.status[0].item()) == 0
         assert torch.equal(y.view(torch.int16), (x.float() * k).to(torch.bfloat16).view(torch.int16))
         assert torch.equal(wy, w)
+
+
+@pytest.mark.gpu
+def test_memory_probe_patterns_move_what_they_say():
+    """The yardstick kernels of the benchmark: every pattern writes exactly the bytes it is specified to write."""
+    import torch
+    from tilexr_amd import ep
+
+    dev = "cuda:0"
+    n = 1 << 20
+    stream = torch.cuda.Stream()
+    src = torch.arange(n, dtype=torch.int32, device=dev)
+    dst = torch.full((n + 64,), -1, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    nbytes = n * 4
+    assert ep.memory_probe(ep.PROBE_COPY, src, dst, nbytes, stream) == 0
+    stream.synchronize()
+    assert torch.equal(dst[:n], src) and bool((dst[n:] == -1).all())
+    dst.fill_(-1)
+    torch.cuda.synchronize()
+    assert ep.memory_probe(ep.PROBE_FAN_OUT, src, dst, nbytes, stream) == 0
+    stream.synchronize()
+    assert torch.equal(dst[:n].view(8, n // 8), src[:n // 8].expand(8, n // 8)) and bool((dst[n:] == -1).all())
+    dst.fill_(-1)
+    torch.cuda.synchronize()
+    assert ep.memory_probe(ep.PROBE_FAN_IN, src, dst, nbytes, stream) == 0
+    stream.synchronize()
+    want = src.view(8, n // 8)[0].clone()
+    for k in range(1, 8):
+        want ^= src.view(8, n // 8)[k]
+    assert torch.equal(dst[:n // 8], want) and bool((dst[n // 8:] == -1).all())
+    dst.fill_(-1)
+    torch.cuda.synchronize()
+    assert ep.memory_probe(ep.PROBE_WRITE, None, dst, nbytes, stream) == 0
+    assert ep.memory_probe(ep.PROBE_READ, src, dst[n:], nbytes, stream) == 0
+    stream.synchronize()
+    assert torch.equal(dst[:n].view(-1, 4), torch.tensor([1, 2, 3, 4], dtype=torch.int32, device=dev).expand(n // 4, 4))
+    assert bool((dst[n:] == -1).all())
+    # argument rules
+    assert ep.memory_probe(7, src, dst, nbytes, stream) == -3
+    assert ep.memory_probe(ep.PROBE_COPY, src, dst, nbytes + 4, stream) == -3
+    assert ep.memory_probe(ep.PROBE_COPY, None, dst, nbytes, stream) == -3

@@ -23,7 +23,7 @@ EXPORTS = (
     "TileXRMoeEpDispatch", "TileXRMoeEpDispatchV2", "TileXRMoeEpDispatchMemory", "TileXRMoeEpDispatchMemoryV2",
     "TileXRMoeEpCombine", "TileXRMoeEpCombineV2", "TileXRMoeEpCombineMemory", "TileXRMoeEpCombineMemoryV2",
     "TileXRMoeEpDispatchMemoryEx", "TileXRMoeEpCombineMemoryEx", "TileXREpVersion", "TileXREpSetKernelTimingEvents",
-    "TileXREpLastKernelName",
+    "TileXREpLastKernelName", "TileXREpMemoryProbe",
     "TileXRCommInitRankLocal", "TileXRCommDestroy", "TileXRGetCommArgsHost", "TileXRGetCommArgsDev",
     "TileXRCommNextMagic",
 )
@@ -275,6 +275,16 @@ K_COUNT, K_PLACE, K_SCATTER, K_INVERT, K_REDUCE = range(5)
 def set_kernel_timing_events(comm, kernel, start=None, stop=None):
     return lib().TileXREpSetKernelTimingEvents(_h(comm), kernel, start.handle if start else None,
                                                stop.handle if stop else None)
+
+
+PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_FAN_OUT, PROBE_FAN_IN = range(5)
+
+
+def memory_probe(pattern, src, dst, nbytes, stream):
+    """One launch of a kernel that does nothing but the memory traffic of `pattern` (see tilexr_ep.h)."""
+    fn = lib().TileXREpMemoryProbe
+    fn.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
+    return fn(pattern, _ptr(src), _ptr(dst), int(nbytes), _stream(stream))
 
 
 def last_kernel_name(comm, kernel):
