@@ -159,7 +159,9 @@ struct TileXREpCombineExOptions {
     const uint64_t *tileFlags;    // optional: before a row is read, wait until the upper half of its tile's word
                                   //      equals flagEpoch; the rows are then read from memory, not from a cache.
                                   //      A producer other than the dispatch above (an expert stage) completes its
-                                  //      rows with a release at agent scope, then stores the word
+                                  //      rows with a release at agent scope, then stores the word.  The producer's
+                                  //      work must be enqueued BEFORE this call: streams of a process may share a
+                                  //      hardware queue, where a waiting kernel keeps later kernels behind it
     int64_t tileRows;
     int64_t flagEpoch;            // epoch the producer tags its flag words with
     int64_t waitTimeoutUs;        // bound of every flag wait; 0 = library default (2 s)

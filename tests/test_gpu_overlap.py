@@ -165,8 +165,10 @@ def test_flag_wait_expires_instead_of_hanging():
 def test_combine_follows_an_expert_stage_that_publishes_tiles_in_random_order():
     """The producer here is not the dispatch but an "expert stage" written with torch ops on a second stream: it
     rewrites the rows tile by tile in a random order and stores a tile's readiness word after the tile's rows (a
-    kernel boundary on one stream is a release at device scope).  The combine is enqueued first, so it really waits;
-    it must return the weighted sum of the rewritten rows, never of the rows the buffer held before."""
+    kernel boundary on one stream is a release at device scope).  The producer's stream starts with a few milliseconds
+    of other work, so a combine that runs beside it really waits; it must return the weighted sum of the rewritten
+    rows, never of the rows the buffer held before.  The producer is enqueued first: two streams of a process can share
+    a hardware queue, and a waiting kernel at the head of that queue would keep the kernels it waits for behind it."""
     bs, h, K, E, tile_rows = 2048, 1024, 4, 32, 128
     rng = np.random.default_rng(31)
     n = bs * K
@@ -187,19 +189,22 @@ def test_combine_follows_an_expert_stage_that_publishes_tiles_in_random_order():
         flags = torch.zeros((tiles,), dtype=torch.int64, device=DEV)
         status = torch.zeros((1,), dtype=torch.int32, device=DEV)
         y = torch.full((bs, h), 3.0, dtype=torch.bfloat16, device=DEV)
+        busy = torch.zeros((64 << 20,), dtype=torch.int32, device=DEV)      # 40 passes over 256 MiB: a few milliseconds
         for epoch in (5, 6, 7):
             scale = float(epoch)
             torch.cuda.synchronize()
+            with torch.cuda.stream(producer):
+                for _ in range(40):
+                    busy.add_(1)
+                for tile in rng.permutation(tiles):
+                    lo, hi = int(tile) * tile_rows, min(int(tile + 1) * tile_rows, n)
+                    expert_out[lo:hi] = (rows[lo:hi].float() * scale).to(torch.bfloat16)
+                    flags[int(tile)] = (epoch << 32) | (hi - lo)
             st = ep.combine_memory_ex(expert_out, out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream,
                                       expert_scales=d_w, row_index_map=out["row_map"], tile_flags=flags,
                                       tile_rows=tile_rows, flag_epoch=epoch, wait_timeout_us=10_000_000,
                                       device_status=status)
             assert st == 0
-            with torch.cuda.stream(producer):
-                for tile in rng.permutation(tiles):
-                    lo, hi = int(tile) * tile_rows, min(int(tile + 1) * tile_rows, n)
-                    expert_out[lo:hi] = (rows[lo:hi].float() * scale).to(torch.bfloat16)
-                    flags[int(tile)] = (epoch << 32) | (hi - lo)
             producer.synchronize()
             s.sync()
             assert status.item() == 0
