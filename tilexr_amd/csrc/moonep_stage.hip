@@ -255,7 +255,9 @@ template <bool FRESH>
 __global__ __launch_bounds__(kTokenThreads) void moon_scatter_token_kernel(DispatchWorld a, int colSlices)
 {
     __shared__ int32_t s_dst[kMaxTopK];
-    __shared__ uint8_t s_direct[kMaxTopK];
+    __shared__ Route s_route[kMaxTopK];
+    __shared__ uint32_t s_tag[kMaxTopK];        // row tag bits of the route; 0 = the source does not write the row
+    __shared__ char *s_row[kMaxTopK];           // destination row
     const int src = blockIdx.y;
     const int token = blockIdx.x / colSlices;
     const int slice = blockIdx.x % colSlices;
@@ -265,29 +267,38 @@ __global__ __launch_bounds__(kTokenThreads) void moon_scatter_token_kernel(Dispa
     const int vecs = h / 8;
     const int idx = slice * kTokenThreads + lane;
     if (lane < K) {
+        // one lane per route decodes it (two 64-bit divisions) for the whole workgroup
         const int64_t route = static_cast<int64_t>(token) * K + lane;
-        s_dst[lane] = a.dst[src][route];
-        s_direct[lane] = FRESH ? 0 : a.tables.direct[static_cast<int64_t>(src) * a.tables.stride + route];
+        const int32_t word = a.dst[src][route];
+        const uint8_t direct = FRESH ? 0 : a.tables.direct[static_cast<int64_t>(src) * a.tables.stride + route];
+        const Route r = Decode(word, a.nvS, a.world);
+        uint32_t tagBits = 0;
+        const bool writes = r.ok && SourceWrites<FRESH>(r, direct, &tagBits);
+        s_dst[lane] = word;
+        s_route[lane] = r;
+        s_tag[lane] = r.ok ? tagBits : 0u;
+        s_row[lane] = writes ? static_cast<char *>(a.hiddenNvsh[r.peer]) + static_cast<int64_t>(r.row) * h * 2 : nullptr;
     }
     const u32x4 *srcRow = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.hiddenSh[src]) +
         static_cast<int64_t>(token) * h * 2);
     const u32x4 v = idx < vecs ? srcRow[idx] : u32x4{0u, 0u, 0u, 0u};
     __syncthreads();
     for (int k = 0; k < K; ++k) {
-        const Route r = Decode(s_dst[k], a.nvS, a.world);
-        if (!r.ok) {
-            if (slice == 0 && lane == 0) {
-                RecordFailure(a.tables, src, a.epoch, kDispatchInvalidRoute);
+        char *row = s_row[k];
+        if (row != nullptr && idx < vecs) {
+            __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(row) + idx);
+        }
+    }
+    if (slice == 0 && lane < kWave) {
+        for (int k = 0; k < K; ++k) {
+            const Route r = s_route[k];
+            if (!r.ok) {
+                if (lane == 0) {
+                    RecordFailure(a.tables, src, a.epoch, kDispatchInvalidRoute);
+                }
+                continue;
             }
-            continue;
-        }
-        uint32_t tagBits = 0;
-        if (SourceWrites<FRESH>(r, s_direct[k], &tagBits) && idx < vecs) {
-            u32x4 *dstRow = reinterpret_cast<u32x4 *>(static_cast<char *>(a.hiddenNvsh[r.peer]) + static_cast<int64_t>(r.row) * h * 2);
-            __builtin_nontemporal_store(v, dstRow + idx);
-        }
-        if (slice == 0 && lane < kWave) {
-            RouteRecords<FRESH>(a, src, token, k, r, tagBits, s_dst);
+            RouteRecords<FRESH>(a, src, token, k, r, s_tag[k], s_dst);
         }
     }
 }
