@@ -533,6 +533,8 @@ __device__ __forceinline__ int64_t SlotOfRow(const WalkArgs &a, int32_t row)
     return peer * a.t.stride + target;
 }
 
+constexpr int kWalkBatch = 8;    // entries of a group a thread has in flight
+
 // One thread per group.  Checks follow the reference (dispatch kernel :428-457, combine kernel :307-345).
 __device__ __forceinline__ void WalkGroup(const WalkArgs &a, int64_t g)
 {
@@ -556,13 +558,24 @@ __device__ __forceinline__ void WalkGroup(const WalkArgs &a, int64_t g)
         return;
     }
     const int64_t base = static_cast<int64_t>(a.rank) * a.t.stride;
-    // nothing is recorded for a group with a bad entry: the kernels that follow these records do not check them again
-    for (int32_t i = 0; i < count; ++i) {
-        const int32_t dup = a.dupLoffs[start + i];
-        if (dup < 0 || dup >= a.nvS || (a.combine && dup == primary)) {
-            RecordFailure(a.t, a.rank, a.epoch, invalid);
-            return;
+    // The group's entries are handled eight at a time with all loads of a batch issued together: a thread that took them
+    // one by one would sit out two dependent round trips per duplicate (entry, then the entry's dstLocal word).
+    // Nothing is recorded for a group with a bad entry: the kernels that follow these records do not check them again.
+    bool bad = false;
+    for (int32_t i0 = 0; i0 < count; i0 += kWalkBatch) {
+        int32_t dup[kWalkBatch];
+#pragma unroll
+        for (int j = 0; j < kWalkBatch; ++j) {
+            dup[j] = i0 + j < count ? a.dupLoffs[start + i0 + j] : 0;
         }
+#pragma unroll
+        for (int j = 0; j < kWalkBatch; ++j) {
+            bad = bad || (i0 + j < count && (dup[j] < 0 || dup[j] >= a.nvS || (a.combine && dup[j] == primary)));
+        }
+    }
+    if (bad) {
+        RecordFailure(a.t, a.rank, a.epoch, invalid);
+        return;
     }
     if (a.combine) {
         // the origin reads these per slot, next to the slot's row, so that one round trip tells it everything
@@ -572,15 +585,31 @@ __device__ __forceinline__ void WalkGroup(const WalkArgs &a, int64_t g)
             a.t.slotGroup[slot] = Tag(a.epoch, static_cast<uint32_t>(start));
         }
     }
-    for (int32_t i = 0; i < count; ++i) {
-        const int32_t dup = a.dupLoffs[start + i];
+    for (int32_t i0 = 0; i0 < count; i0 += kWalkBatch) {
+        int32_t dup[kWalkBatch];
+#pragma unroll
+        for (int j = 0; j < kWalkBatch; ++j) {
+            dup[j] = i0 + j < count ? a.dupLoffs[start + i0 + j] : -1;
+        }
         if (a.combine) {
-            const int64_t slot = SlotOfRow(a, dup);
-            if (slot >= 0) {
-                a.t.slotDup[slot] = Tag(a.epoch, 1u);
+            int64_t slot[kWalkBatch];
+#pragma unroll
+            for (int j = 0; j < kWalkBatch; ++j) {
+                slot[j] = dup[j] >= 0 ? SlotOfRow(a, dup[j]) : -1;
+            }
+#pragma unroll
+            for (int j = 0; j < kWalkBatch; ++j) {
+                if (slot[j] >= 0) {
+                    a.t.slotDup[slot[j]] = Tag(a.epoch, 1u);
+                }
             }
         } else {
-            a.t.parentTag[base + dup] = Tag(a.epoch, static_cast<uint32_t>(primary) + 1u);
+#pragma unroll
+            for (int j = 0; j < kWalkBatch; ++j) {
+                if (dup[j] >= 0) {
+                    a.t.parentTag[base + dup[j]] = Tag(a.epoch, static_cast<uint32_t>(primary) + 1u);
+                }
+            }
         }
     }
 }
@@ -717,11 +746,8 @@ __global__ __launch_bounds__(kThreads) void moon_combine_prepare_kernel(CombineW
     const int64_t row = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     WalkArgs w {a.nvS, rank, true, a.dupGroups[rank], a.dupLoffs[rank], a.dupCounts[rank], a.tables, a.epoch, a.dstLocal[rank],
         a.world, a.s * a.k};
+    const int32_t encoded = row < a.nvS ? a.dstLocal[rank][row] : -1;      // in flight while the group is walked
     WalkGroup(w, row);
-    if (row >= a.nvS) {
-        return;
-    }
-    const int32_t encoded = a.dstLocal[rank][row];
     if (encoded == -1) {
         return;
     }
