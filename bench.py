@@ -79,8 +79,8 @@ def measured_ceilings(ep, torch, stream, dev, reps=10):
     patterns depend on how far apart their eight regions lie (5.6 to 6.6 TB/s for the 1 : 8 mix between 56 and 125 MiB),
     so they are run at three sizes and the best is kept: a ceiling, not an average."""
     patterns = {"read": ep.PROBE_READ, "write": ep.PROBE_WRITE, "copy": ep.PROBE_COPY, "fan_out_1r8w": ep.PROBE_FAN_OUT,
-                "fan_in_8r1w": ep.PROBE_FAN_IN}
-    sizes = (448, 472, 1000)
+                "fan_in_8r1w": ep.PROBE_FAN_IN, "gather_rows_8r1w": ep.PROBE_GATHER_ROWS}
+    sizes = (448, 472, 1000)       # MiB, each a multiple of eight rows of 14 KiB
     out = {"buffer_MiB": list(sizes), "launches": reps}
     for mib in sizes:
         nbytes = mib << 20
@@ -88,16 +88,20 @@ def measured_ceilings(ep, torch, stream, dev, reps=10):
         dst = torch.zeros((nbytes,), dtype=torch.uint8, device=dev)
         torch.cuda.synchronize()
         moved = {"read": nbytes, "write": nbytes, "copy": 2 * nbytes, "fan_out_1r8w": nbytes + nbytes // 8,
-                 "fan_in_8r1w": nbytes + nbytes // 8}
+                 "fan_in_8r1w": nbytes + nbytes // 8, "gather_rows_8r1w": nbytes + nbytes // 8}
         for name, pattern in patterns.items():
-            if mib != sizes[0] and not name.startswith("fan"):
+            if mib != sizes[0] and name in ("read", "write", "copy"):
                 continue
+            size = nbytes
+            if name == "gather_rows_8r1w":      # whole groups of eight 14 KiB rows
+                size = nbytes // (8 * 14336) * (8 * 14336)
+                moved[name] = size + size // 8
             for _ in range(3):
-                ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+                ep.check(ep.memory_probe(pattern, src, dst, size, stream), "memory probe")
             a, b = ep.HipEvent(timing=True), ep.HipEvent(timing=True)
             a.record(stream)
             for _ in range(reps):
-                ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+                ep.check(ep.memory_probe(pattern, src, dst, size, stream), "memory probe")
             b.record(stream)
             stream.synchronize()
             us = a.elapsed_ms(b) * 1e3 / reps
@@ -361,6 +365,8 @@ def main_moonep(args):
         if roofline is not None:
             mix = ceilings["fan_out_1r8w_GBps"] if dom == "scatter" else ceilings["fan_in_8r1w_GBps"]
             roofline["frac_of_measured_mix"] = round(roofline["achieved"] / mix, 4)
+            if dom == "reduce":
+                roofline["frac_of_measured_row_gather"] = round(roofline["achieved"] / ceilings["gather_rows_8r1w_GBps"], 4)
     result = {
         "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -607,6 +613,8 @@ def main():
         if roofline is not None:
             mix = ceilings["fan_out_1r8w_GBps"] if dom == "scatter" else ceilings["fan_in_8r1w_GBps"]
             roofline["frac_of_measured_mix"] = round(roofline["achieved"] / mix, 4)
+            if dom == "reduce":
+                roofline["frac_of_measured_row_gather"] = round(roofline["achieved"] / ceilings["gather_rows_8r1w_GBps"], 4)
 
     result = {
         "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",

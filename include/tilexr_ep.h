@@ -198,13 +198,16 @@ const char *TileXREpVersion(void);
 //   COPY     reads `bytes` of src, writes `bytes` of dst
 //   FAN_OUT  reads bytes / 8 of src, writes `bytes` of dst as eight copies   (the scatter's 1 : 8 mix)
 //   FAN_IN   reads `bytes` of src as eight regions, writes bytes / 8 of dst  (the reduce's 8 : 1 mix)
+//   GATHER_ROWS  the same mix with the reduce's addresses: src is rows of 14336 bytes, every output row combines
+//            eight source rows at unrelated positions; `bytes` a multiple of 8 * 14336; writes bytes / 8 of dst
 // Asynchronous on `stream`; returns 0, -3 for bad arguments, -2 when the launch fails.
 enum TileXREpProbePattern {
     TILEXR_EP_PROBE_READ = 0,
     TILEXR_EP_PROBE_WRITE = 1,
     TILEXR_EP_PROBE_COPY = 2,
     TILEXR_EP_PROBE_FAN_OUT = 3,
-    TILEXR_EP_PROBE_FAN_IN = 4
+    TILEXR_EP_PROBE_FAN_IN = 4,
+    TILEXR_EP_PROBE_GATHER_ROWS = 5
 };
 int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int64_t bytes, aclrtStream stream);
 

@@ -167,3 +167,28 @@ def test_memory_probe_patterns_move_what_they_say():
     assert ep.memory_probe(7, src, dst, nbytes, stream) == -3
     assert ep.memory_probe(ep.PROBE_COPY, src, dst, nbytes + 4, stream) == -3
     assert ep.memory_probe(ep.PROBE_COPY, None, dst, nbytes, stream) == -3
+
+
+@pytest.mark.gpu
+def test_memory_probe_row_gather_reads_rows_whole():
+    """The row-gather yardstick: every output row is the xor of eight source rows, taken whole."""
+    import torch
+    from tilexr_amd import ep
+
+    dev = "cuda:0"
+    rows, row_ints = 64, 14336 // 4
+    stream = torch.cuda.Stream()
+    g = torch.Generator().manual_seed(5)
+    src = torch.randint(-2**31, 2**31 - 1, (rows, row_ints), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    dst = torch.full((rows // 8 + 1, row_ints), -1, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    assert ep.memory_probe(ep.PROBE_GATHER_ROWS, src, dst, rows * 14336, stream) == 0
+    stream.synchronize()
+    strides = [1, 7919, 10007, 12289, 15013, 17389, 20011, 22291]
+    for t in range(rows // 8):
+        want = torch.zeros(row_ints, dtype=torch.int32, device=dev)
+        for k in range(8):
+            want ^= src[(t * strides[k] + k * 977) % rows]
+        assert torch.equal(dst[t], want), f"row {t}"
+    assert bool((dst[rows // 8] == -1).all())
+    assert ep.memory_probe(ep.PROBE_GATHER_ROWS, src, dst, rows * 14336 + 128, stream) == -3

@@ -7,6 +7,8 @@
 //   copy      src -> dst, two loads then two stores per lane
 //   fan-out   the scatter's mix: a block of src is loaded once and stored to eight regions of dst (1 read : 8 writes)
 //   fan-in    the reduce's mix: eight regions of src are loaded and one region of dst is stored (8 reads : 1 write)
+//   gather    the same mix with the reduce's addresses: every output row of 14 KiB combines eight rows of src that lie
+//             at unrelated positions
 //
 // No reference counterpart; nothing on the dispatch / combine path calls these.
 #include <hip/hip_runtime.h>
@@ -96,6 +98,31 @@ __global__ __launch_bounds__(kWave) void ep_probe_fan_in_kernel(const u32x4 *src
     __builtin_nontemporal_store(acc, dst + at);
 }
 
+// The reduce's mix with the reduce's addresses: src is rows of kProbeRowBytes; output row t is combined from eight rows
+// at unrelated positions ((t * stride_k + k) mod rows, a bijection per k because the strides are coprime to the row
+// count chosen by the launcher).  One wave per 1 KiB slice of an output row, as in the reduce kernel.
+constexpr int kProbeRowBytes = 14336;
+constexpr int kProbeRowVecs = kProbeRowBytes / 16;
+__global__ __launch_bounds__(kWave) void ep_probe_gather_rows_kernel(const u32x4 *src, u32x4 *dst, int64_t rows)
+{
+    constexpr int kSlices = kProbeRowVecs / kWave;
+    const uint32_t t = blockIdx.x / kSlices;
+    const int at = (blockIdx.x % kSlices) * kWave + threadIdx.x;
+    const uint32_t strides[8] = {1u, 7919u, 10007u, 12289u, 15013u, 17389u, 20011u, 22291u};   // primes; rows < 2^17
+    u32x4 v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const uint32_t row = (t * strides[k] + static_cast<uint32_t>(k) * 977u) % static_cast<uint32_t>(rows);
+        v[k] = __builtin_nontemporal_load(src + static_cast<int64_t>(row) * kProbeRowVecs + at);
+    }
+    u32x4 acc = v[0];
+#pragma unroll
+    for (int k = 1; k < 8; ++k) {
+        acc ^= v[k];
+    }
+    __builtin_nontemporal_store(acc, dst + static_cast<int64_t>(t) * kProbeRowVecs + at);
+}
+
 } // namespace
 } // namespace TileXREp
 
@@ -104,7 +131,10 @@ extern "C" int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int6
     using namespace TileXREp;
     const bool needSrc = pattern != TILEXR_EP_PROBE_WRITE;
     const bool needDst = true;      // the read probe uses dst as a 4-byte sink
-    if (pattern < TILEXR_EP_PROBE_READ || pattern > TILEXR_EP_PROBE_FAN_IN || bytes < 128 || bytes % 128 != 0 ||
+    if (pattern == TILEXR_EP_PROBE_GATHER_ROWS && (bytes % (8 * kProbeRowBytes) != 0 || bytes / kProbeRowBytes >= (1 << 17))) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    if (pattern < TILEXR_EP_PROBE_READ || pattern > TILEXR_EP_PROBE_GATHER_ROWS || bytes < 128 || bytes % 128 != 0 ||
         bytes > (int64_t{1} << 40) || (needSrc && (src == nullptr || !Aligned16(src))) ||
         (needDst && (dst == nullptr || !Aligned16(dst)))) {
         return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
@@ -128,9 +158,14 @@ extern "C" int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int6
         case TILEXR_EP_PROBE_FAN_OUT:
             hipLaunchKernelGGL(ep_probe_fan_out_kernel, blocks(vecs / 8, kWave), dim3(kWave), 0, s, in, out, vecs / 8);
             break;
-        default:
+        case TILEXR_EP_PROBE_FAN_IN:
             hipLaunchKernelGGL(ep_probe_fan_in_kernel, blocks(vecs / 8, kWave), dim3(kWave), 0, s, in, out, vecs / 8);
             break;
+        default: {
+            const int64_t rows = bytes / kProbeRowBytes;
+            hipLaunchKernelGGL(ep_probe_gather_rows_kernel, blocks(vecs / 8, kWave), dim3(kWave), 0, s, in, out, rows);
+            break;
+        }
     }
     return hipGetLastError() == hipSuccess ? TileXR::TILEXR_SUCCESS : TileXR::TILEXR_ERROR_MKIRT;
 }

@@ -277,7 +277,7 @@ def set_kernel_timing_events(comm, kernel, start=None, stop=None):
                                                stop.handle if stop else None)
 
 
-PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_FAN_OUT, PROBE_FAN_IN = range(5)
+PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_FAN_OUT, PROBE_FAN_IN, PROBE_GATHER_ROWS = range(6)
 
 
 def memory_probe(pattern, src, dst, nbytes, stream):
