@@ -15,6 +15,11 @@ def test_exports_and_versions():
     lib = mp.lib()
     for name in mp.EXPORTS:
         assert hasattr(lib, name), name
+    # every function the header declares is in that list
+    import re
+    header = open(os.path.join(ROOT, "include", "tilexr_moonep.h")).read()
+    declared = set(re.findall(r"^(?:int|uint32_t|int64_t)\s+(TileXRMoonEp\w+)\(", header, flags=re.M))
+    assert declared == set(mp.EXPORTS), sorted(declared ^ set(mp.EXPORTS))
     assert mp.abi_version() == 2
     for version in (1, 2):
         ret, native, stub = mp.capabilities(version)
