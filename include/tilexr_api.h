@@ -23,6 +23,7 @@
 #include "comm_args.h"
 
 extern "C" {
+#pragma GCC visibility push(default)   // the entry points below are what the shared library exports
 
 typedef void *TileXRCommPtr;
 
@@ -41,6 +42,7 @@ int TileXRGetCommArgsHost(TileXRCommPtr comm, TileXR::CommArgs *&commArgsPtr);
 // reference: src/include/tilexr_api.h:48
 int TileXRCommNextMagic(TileXRCommPtr comm, int64_t *magic);
 
+#pragma GCC visibility pop
 }
 
 #endif // TILEXR_API_H

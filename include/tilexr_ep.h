@@ -56,6 +56,7 @@ enum TileXREpQuantMode : int64_t {
 } // namespace TileXREp
 
 extern "C" {
+#pragma GCC visibility push(default)   // the entry points below are what the shared library exports
 
 // ---------------------------------------------------------------------------------------------------------
 // Part 1: the reference's entry points
@@ -132,8 +133,11 @@ struct TileXREpDispatchExOptions {
                                   //      becomes (epoch << 32) | rows in the tile, in one store, once every row of
                                   //      the tile (payload and scales) is complete in memory for every compute
                                   //      unit; until then it holds whatever an earlier epoch left (never cleared)
-    int64_t tileRows;
-    int64_t *epochOut;            // optional host pointer: receives the epoch the flags are tagged with
+    int64_t tileRows;             // 1 .. 2^31 - 1 when tileFlagsOut is set; values above bs * topK name one tile
+    int64_t *epochOut;            // optional host pointer: receives the epoch the flags are tagged with.  Epochs
+                                  //      are 32 bits wide, never 0 and drawn from one counter for the whole process,
+                                  //      so flag arrays may be shared by communicators; a zero-filled array is
+                                  //      "not ready" for every epoch
     void *metaReadyEvent;         // optional hipEvent_t recorded on `stream` once counts, assist tuples,
                                   //      rowIndexMapOut and the reset flag words are enqueued (before rows move)
 };
@@ -162,10 +166,16 @@ struct TileXREpCombineExOptions {
                                   //      rows with a release at agent scope, then stores the word.  The producer's
                                   //      work must be enqueued BEFORE this call: streams of a process may share a
                                   //      hardware queue, where a waiting kernel keeps later kernels behind it
-    int64_t tileRows;
+                                  //      Waiting workgroups stay resident (two per compute unit): a producer
+                                  //      that runs beside them needs room for at least one workgroup of its own
+                                  //      on the compute units, or the waits expire
+    int64_t tileRows;             // 1 .. 2^31 - 1 when tileFlags is set
     int64_t flagEpoch;            // epoch the producer tags its flag words with
     int64_t waitTimeoutUs;        // bound of every flag wait; 0 = library default (2 s)
-    int32_t *deviceStatusOut;     // optional device int32: set to 1 when a flag wait expired
+    int32_t *deviceStatusOut;     // device int32, required with tileFlags (-3 without it): set to 1 when a flag
+                                  //      wait expired; the waits that follow in that launch give up at once.  A
+                                  //      token with an expired wait gets a row of zeros in yOut, never a partial sum.
+                                  //      The caller clears the word before the call
 };
 
 // Memory-route combine (same result as TileXRMoeEpCombineMemoryV2) with quantised expert output, a ready-made
@@ -211,6 +221,7 @@ enum TileXREpProbePattern {
 };
 int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int64_t bytes, aclrtStream stream);
 
+#pragma GCC visibility pop
 }
 
 #endif // __cplusplus

@@ -50,6 +50,7 @@
 
 #ifdef __cplusplus
 extern "C" {
+#pragma GCC visibility push(default)   // the entry points below are what the shared library exports
 #endif
 
 #ifndef TILEXR_EP_HAVE_ACL_STREAM
@@ -205,6 +206,7 @@ int TileXRMoonEpCombineV1(const TileXRMoonEpCombineArgsV1 *args, aclrtStream str
 int64_t TileXRMoonEpSetCachedRowBytes(int64_t bytes);
 
 #ifdef __cplusplus
+#pragma GCC visibility pop
 }
 #endif
 

@@ -1,7 +1,13 @@
-"""ctypes view of the host-side hooks of libtilexr-ep.so (tilexr_amd/csrc/hooks.h) for the CPU tests."""
+"""ctypes view of the test-only companion library libtilexr-ep-hooks.so for the CPU tests: the plain-C hooks into the
+host-side rules (tilexr_amd/csrc/hooks.h) and the CPU model of the readiness-flag protocol (tilexr_amd/csrc/flag_trace.h).
+It is linked from the same objects as libtilexr-ep.so, which itself exports the declared entry points only."""
 import ctypes as C
+import os
 
 from tilexr_amd import ep
+
+HOOKS_PATH = os.path.join(os.path.dirname(ep.LIB_PATH), "libtilexr-ep-hooks.so")
+_hooks = None
 
 X, EXPERT_IDS, SCALES, ACTIVE_MASK, EXPERT_SCALES, COMM, EXPAND_X, DYNAMIC_SCALES, ASSIST, TOKEN_NUMS, COUNTS, \
     TP_COUNTS, EXPAND_SCALES, WORKSPACE, STREAM = (1 << i for i in range(15))
@@ -30,7 +36,12 @@ class HookCombine(C.Structure):
 
 
 def lib():
-    l = ep.lib()
+    global _hooks
+    if _hooks is None:
+        if not os.path.exists(HOOKS_PATH):
+            raise ImportError(f"{HOOKS_PATH} is missing: build it with `make -C tilexr_amd/csrc`")
+        _hooks = C.CDLL(HOOKS_PATH)
+    l = _hooks
     if not getattr(l, "_hooks_ready", False):
         i64, i32, u32, vp = C.c_int64, C.c_int, C.c_uint32, C.c_void_p
         l.TileXREpHookValidateDispatch.argtypes = [i32, C.POINTER(HookDispatch), C.POINTER(HookComm)]

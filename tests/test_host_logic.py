@@ -32,6 +32,22 @@ def test_library_exports_every_declared_symbol():
     assert ep.version().startswith("tilexr-ep gfx950")
 
 
+def test_library_exports_nothing_but_the_declared_entry_points():
+    """The dynamic symbol table of libtilexr-ep.so is exactly the functions that include/*.h declare: no C++ internals,
+    no test seams (those live in the companion hooks library)."""
+    import subprocess
+    declared = set()
+    for header in ("tilexr_ep.h", "tilexr_api.h", "tilexr_moonep.h"):
+        text = open(os.path.join(ROOT, "include", header)).read()
+        declared |= set(re.findall(r"^(?:int|uint32_t|int64_t|const char \*)\s*\*?(TileXR\w+)\(", text, flags=re.M))
+    out = subprocess.run(["nm", "-D", "--defined-only", ep.LIB_PATH], check=True, capture_output=True, text=True).stdout
+    exported = {line.split()[-1] for line in out.splitlines() if line.strip()}
+    assert exported == declared, sorted(exported ^ declared)
+    hooks = subprocess.run(["nm", "-D", "--defined-only", H.HOOKS_PATH], check=True, capture_output=True, text=True).stdout
+    names = {line.split()[-1] for line in hooks.splitlines() if line.strip()}
+    assert names and all(n.startswith(("TileXREpHook", "TileXREpTrace")) for n in names), sorted(names)
+
+
 # ---------------------------------------------------------------------------------------------
 # arithmetic: reference known answers
 # ---------------------------------------------------------------------------------------------
@@ -328,6 +344,23 @@ def test_entry_points_reject_before_touching_a_device():
         assert ep.combine(recv_counts=fake, **cargs) == ep.ERR_NOT_INITIALIZED
         assert ep.combine_memory(send_counts=fake, **cargs) == ep.ERR_NOT_INITIALIZED
         assert ep.combine_memory(send_counts=None, **cargs) == ep.ERR_PARA_CHECK_FAIL
+        # readiness flags: tile sizes are checked before anything else of the extended calls, and a combine that
+        # waits on flags must be given the status word an expired wait is reported through
+        ex = (fake, fake, comm, 4, 8, 2, 8, fake, fake, fake, fake, ep.DT_BF16, fake)
+        for tile_rows in (0, -1, 1 << 31, 1 << 40):
+            st, _ = ep.dispatch_memory_ex(*ex, tile_flags=fake, tile_rows=tile_rows)
+            assert st == ep.ERR_PARA_CHECK_FAIL, tile_rows
+        st, _ = ep.dispatch_memory_ex(*ex, tile_flags=fake, tile_rows=(1 << 31) - 1)
+        assert st == ep.ERR_NOT_INITIALIZED
+        cex = (fake, fake, fake, comm, 4, 8, 2, 8, fake, ep.DT_BF16, fake)
+        for tile_rows in (0, -1, 1 << 31):
+            assert ep.combine_memory_ex(*cex, tile_flags=fake, tile_rows=tile_rows, flag_epoch=1,
+                                        device_status=fake) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.combine_memory_ex(*cex, tile_flags=fake, tile_rows=8, flag_epoch=1) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.combine_memory_ex(*cex, tile_flags=fake, tile_rows=8, flag_epoch=1,
+                                    device_status=fake) == ep.ERR_NOT_INITIALIZED
+        assert ep.combine_memory_ex(*cex, tile_flags=fake, tile_rows=8, flag_epoch=1, device_status=fake,
+                                    wait_timeout_us=-5) == ep.ERR_PARA_CHECK_FAIL
         assert comm.next_magic() == 3                                 # no magic was consumed by rejected calls
     # an unknown communicator handle
     args = dict(x=fake, expert_ids=fake, comm=0xdead0, bs=4, h=8, top_k=2, experts=8, expand_x=fake,
@@ -386,7 +419,7 @@ def test_cxx_caller_links_against_the_headers_and_the_library(tmp_path):
 # readiness-tile bookkeeping: the scatter kernels' counting code, run on CPU threads with random landing orders
 # ---------------------------------------------------------------------------------------------
 def _publish_stress(*args):
-    fn = ep.lib().TileXREpHookTilePublishStress
+    fn = H.lib().TileXREpHookTilePublishStress
     fn.argtypes = [C.c_int] * 6 + [C.c_uint32, C.c_int]
     return fn(*args)
 

@@ -4,6 +4,7 @@
 // tilexr_ep_memory_dispatch.cpp:9-23, tilexr_ep_memory_combine.cpp:9-21, ep_kernel_launch.cpp:252-416):
 // basic argument check, communicator lookup, configuration check, magic, launch.  Success means "enqueued on the
 // caller's stream"; nothing here waits for the device.
+#include <algorithm>
 #include <cstdio>
 #include <limits>
 
@@ -26,7 +27,7 @@ constexpr int kOk = TileXR::TILEXR_SUCCESS;
 // ---------------------------------------------------------------------------------------------------------
 // one rank per device: rows go straight from x to expandXOut
 // ---------------------------------------------------------------------------------------------------------
-int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, int64_t magic)
+int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, int64_t magic, uint64_t flagEpoch)
 {
     if (!WithinKernelLimits(p.bs, p.h, p.topK, p.moeExpertNum)) {
         return TileXR::TILEXR_ERROR_NOT_SUPPORT;
@@ -155,11 +156,12 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     scatter.out = p.expandXOut;
     scatter.scalesOut = p.dynamicScalesOut;
     scatter.tileFlags = p.tileFlagsOut;
-    scatter.tileRows = p.tileRows;
-    scatter.epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
+    // a tile never holds more rows than the dispatch can produce: larger values name the same single tile
+    scatter.tileRows = std::min<int64_t>(p.tileRows, std::max<int64_t>(n, 1));
+    scatter.epoch = flagEpoch;
     scatter.totalRowsPtr = scratch.keyOffset + numKeys;
     if (p.tileFlagsOut != nullptr) {
-        if (!comm->tileCounters.Reserve(static_cast<size_t>(TileCounterWords(n, p.tileRows)) * sizeof(uint32_t), true)) {
+        if (!comm->tileCounters.Reserve(static_cast<size_t>(TileCounterWords(n, scatter.tileRows)) * sizeof(uint32_t), true)) {
             return TileXR::TILEXR_ERROR_INTERNAL;
         }
         scatter.tileCounters = static_cast<uint32_t *>(comm->tileCounters.ptr);
@@ -223,7 +225,7 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     red.topK = p.topK;
     red.y = p.yOut;
     red.tileFlags = p.tileFlags;
-    red.tileRows = p.tileRows;
+    red.tileRows = std::min<int64_t>(p.tileRows, std::max<int64_t>(n, 1));
     red.flagEpoch = static_cast<uint64_t>(p.flagEpoch) & 0xffffffffull;
     red.waitTimeoutTicks = (p.waitTimeoutUs > 0 ? p.waitTimeoutUs : kDefaultWaitUs) * kWallClockTicksPerUs;
     red.deviceStatus = p.deviceStatusOut;
@@ -269,7 +271,8 @@ int DispatchMvp(const EpDispatchParams &p)
     if (ret != kOk) {
         return ret;
     }
-    return args->rankSize == 1 ? RunDispatchSingle(comm, p, false, magic) : RunDispatchMulti(comm, p, false, magic);
+    return args->rankSize == 1 ? RunDispatchSingle(comm, p, false, magic, static_cast<uint64_t>(magic) & 0xffffffffull) :
+                                 RunDispatchMulti(comm, p, false, magic);
 }
 
 int DispatchMemory(const EpDispatchParams &p)
@@ -293,7 +296,8 @@ int DispatchMemory(const EpDispatchParams &p)
             p.quantMode != TILEXR_EP_QUANT_MXFP8 && p.quantMode != TILEXR_EP_QUANT_FP8_BLOCK128) {
             return TileXR::TILEXR_ERROR_NOT_SUPPORT;
         }
-        if (p.expertCapacity < 0 || (p.tileFlagsOut != nullptr && p.tileRows <= 0)) {
+        if (p.expertCapacity < 0 ||
+            (p.tileFlagsOut != nullptr && (p.tileRows <= 0 || p.tileRows > std::numeric_limits<int32_t>::max()))) {
             return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
         }
         if (p.quantMode == TILEXR_EP_QUANT_TOKEN_INT8 || p.quantMode == TILEXR_EP_QUANT_FP8_BLOCK128) {
@@ -319,10 +323,13 @@ int DispatchMemory(const EpDispatchParams &p)
     if (ret != kOk) {
         return ret;
     }
+    // Readiness words are tagged from one counter for the whole process, so that two communicators that are handed the
+    // same flag array (one after the other, or a destroyed and re-created one) can never tag it with the same value.
+    const uint64_t flagEpoch = p.tileFlagsOut != nullptr ? NextFlagEpoch() : (static_cast<uint64_t>(magic) & 0xffffffffull);
     if (p.epochOut != nullptr) {
-        *p.epochOut = magic & 0xffffffffll;
+        *p.epochOut = static_cast<int64_t>(flagEpoch);
     }
-    return args->rankSize == 1 ? RunDispatchSingle(comm, p, true, magic) : RunDispatchMulti(comm, p, true, magic);
+    return args->rankSize == 1 ? RunDispatchSingle(comm, p, true, magic, flagEpoch) : RunDispatchMulti(comm, p, true, magic);
 }
 
 int CombineMvp(const EpCombineParams &p)
@@ -372,8 +379,11 @@ int CombineMemory(const EpCombineParams &p)
             p.expertOutQuantMode != TILEXR_EP_QUANT_FP8_BLOCK128) {
             return TileXR::TILEXR_ERROR_NOT_SUPPORT;
         }
+        // a combine that waits on flags must be able to report an expired wait: the status word is required
         if ((p.expertOutQuantMode != 0 && (p.expertOutScales == nullptr || p.quantMode != 0)) ||
-            (p.tileFlags != nullptr && p.tileRows <= 0) || p.waitTimeoutUs < 0) {
+            (p.tileFlags != nullptr && (p.tileRows <= 0 || p.tileRows > std::numeric_limits<int32_t>::max() ||
+                                        p.deviceStatusOut == nullptr)) ||
+            p.waitTimeoutUs < 0) {
             return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
         }
         if (args->rankSize != 1) {

@@ -107,6 +107,16 @@ void DeviceBuffer::Release()
     bytes = 0;
 }
 
+uint64_t NextFlagEpoch()
+{
+    static std::atomic<uint32_t> counter {0};
+    uint32_t v = 0;
+    do {
+        v = counter.fetch_add(1, std::memory_order_relaxed) + 1;
+    } while (v == 0);
+    return v;
+}
+
 EpComm *LookupComm(TileXRCommPtr comm)
 {
     std::lock_guard<std::mutex> lock(gRegistryMutex);

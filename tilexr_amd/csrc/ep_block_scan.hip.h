@@ -1,10 +1,10 @@
 // Workgroup-wide exclusive scan in LDS (256 threads), shared by the routing and exchange kernels.
-#ifndef TILEXR_AMD_EP_BLOCK_SCAN_CUH
-#define TILEXR_AMD_EP_BLOCK_SCAN_CUH
+#ifndef TILEXR_AMD_EP_BLOCK_SCAN_HIP_H
+#define TILEXR_AMD_EP_BLOCK_SCAN_HIP_H
 
 #include <hip/hip_runtime.h>
 
-#include "ep_kernel_common.cuh"
+#include "ep_kernel_common.hip.h"
 
 namespace TileXREp {
 
@@ -52,4 +52,4 @@ __device__ inline int BlockExclusiveScan(int *vals, int m, int *part)
 
 } // namespace TileXREp
 
-#endif // TILEXR_AMD_EP_BLOCK_SCAN_CUH
+#endif // TILEXR_AMD_EP_BLOCK_SCAN_HIP_H

@@ -122,6 +122,10 @@ struct EpComm {
 
 enum KernelId : int { kKernelCount = 0, kKernelPlace = 1, kKernelScatter = 2, kKernelInvert = 3, kKernelReduce = 4 };
 
+// Next tag for tile readiness words: one counter for the whole process, 32 bits wide, never 0 (a zero-filled flag
+// array must read as "not ready" for every epoch).
+uint64_t NextFlagEpoch();
+
 // Returns the communicator when `comm` was created by TileXRCommInitRankLocal and not destroyed, else nullptr.
 EpComm *LookupComm(TileXRCommPtr comm);
 

@@ -7,11 +7,11 @@
 // All integer work; the reference behaviour each kernel restates is cited at the kernel.
 #include <hip/hip_runtime.h>
 
-#include "ep_block_scan.cuh"
-#include "ep_kernel_common.cuh"
+#include "ep_block_scan.hip.h"
+#include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
-#include "ep_numerics.cuh"
-#include "ep_place.cuh"
+#include "ep_numerics.hip.h"
+#include "ep_place.hip.h"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -345,7 +345,7 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
 // -------------------------------------------------------------------------------------------------------------
 // place (stand-alone): destination row of every route + assist tuple + inverse map.  Used when they must be complete
 // before the first row lands (readiness flags, a metadata-ready event) or when the rows go to a staging area;
-// otherwise the scatter kernel resolves the rows of its own tokens (ep_place.cuh).
+// otherwise the scatter kernel resolves the rows of its own tokens (ep_place.hip.h).
 // -------------------------------------------------------------------------------------------------------------
 struct RoutePlaceArgs {
     PlaceArgs p;

@@ -10,9 +10,9 @@
 // On one device the "window" is ordinary HBM owned by the world, and readiness is stream order, not flags.
 #include <hip/hip_runtime.h>
 
-#include "ep_block_scan.cuh"
+#include "ep_block_scan.hip.h"
 #include "ep_exchange.h"
-#include "ep_kernel_common.cuh"
+#include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
 
 namespace TileXREp {

@@ -1,6 +1,6 @@
 // Launch geometry shared by the EP kernels (gfx950: 64-lane wavefronts, 256-thread workgroups).
-#ifndef TILEXR_AMD_EP_KERNEL_COMMON_CUH
-#define TILEXR_AMD_EP_KERNEL_COMMON_CUH
+#ifndef TILEXR_AMD_EP_KERNEL_COMMON_HIP_H
+#define TILEXR_AMD_EP_KERNEL_COMMON_HIP_H
 
 #include <cstdint>
 
@@ -63,4 +63,4 @@ __device__ __forceinline__ void WaitOwnStores()
 
 } // namespace TileXREp
 
-#endif // TILEXR_AMD_EP_KERNEL_COMMON_CUH
+#endif // TILEXR_AMD_EP_KERNEL_COMMON_HIP_H

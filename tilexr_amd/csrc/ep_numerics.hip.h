@@ -9,8 +9,8 @@
 //   int8 rounding      reference: src/ep/kernels/tilexr_ep_dispatch_kernel.cpp:183-193
 //   MXFP8 / fp8 codec  reference: tests/ep/demo/mxfp8_golden.h:45-152
 //   output casts       reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:595 (CAST_RINT, saturating)
-#ifndef TILEXR_AMD_EP_NUMERICS_CUH
-#define TILEXR_AMD_EP_NUMERICS_CUH
+#ifndef TILEXR_AMD_EP_NUMERICS_HIP_H
+#define TILEXR_AMD_EP_NUMERICS_HIP_H
 
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
@@ -219,4 +219,4 @@ __device__ __forceinline__ float Exp2Int(int e)
 
 } // namespace TileXREp
 
-#endif // TILEXR_AMD_EP_NUMERICS_CUH
+#endif // TILEXR_AMD_EP_NUMERICS_HIP_H

@@ -3,8 +3,8 @@
 //   row   = keyOffset[key] + (rank of the route within its key), routes at or beyond `capacity` get none
 //   tuple = {srcRank, token, k, expert id} (reference: src/ep/common/ep_window.h:47-52,
 //           src/ep/kernels/tilexr_ep_dispatch_memory_kernel.h:1240-1258)
-#ifndef TILEXR_AMD_EP_PLACE_CUH
-#define TILEXR_AMD_EP_PLACE_CUH
+#ifndef TILEXR_AMD_EP_PLACE_HIP_H
+#define TILEXR_AMD_EP_PLACE_HIP_H
 
 #include <cstdint>
 
@@ -84,4 +84,4 @@ __device__ __forceinline__ int PlaceRoute(const PlaceArgs &a, int i)
 
 } // namespace TileXREp
 
-#endif // TILEXR_AMD_EP_PLACE_CUH
+#endif // TILEXR_AMD_EP_PLACE_HIP_H

@@ -13,8 +13,8 @@
 // No reference counterpart; nothing on the dispatch / combine path calls these.
 #include <hip/hip_runtime.h>
 
-#include "ep_kernel_common.cuh"
-#include "ep_numerics.cuh"
+#include "ep_kernel_common.hip.h"
+#include "ep_numerics.hip.h"
 #include "tilexr_ep.h"
 #include "tilexr_types.h"
 

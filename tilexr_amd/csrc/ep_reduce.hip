@@ -17,9 +17,10 @@
 //                 type first (no reference counterpart)
 #include <hip/hip_runtime.h>
 
-#include "ep_kernel_common.cuh"
+#include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
-#include "ep_numerics.cuh"
+#include "ep_numerics.hip.h"
+#include "ep_tile_publish.h"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -71,7 +72,7 @@ __device__ bool WaitTile(const ReduceArgs &a, int row)
     int backoff = 0;
     while (true) {
         const uint64_t w = __hip_atomic_load(&a.tileFlags[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((w >> 32) == a.flagEpoch) {
+        if (TileWordReady(w, a.flagEpoch)) {
             return true;
         }
         if (static_cast<int64_t>(wall_clock64() - start) > a.waitTimeoutTicks) {
@@ -144,7 +145,20 @@ __device__ __forceinline__ float ScaleLoad(const float *p)
     return *p;
 }
 
-// Fills s_row / s_w for one token; waits for tile flags when asked to.
+// Fills s_row / s_w for one token; waits for tile flags when asked to.  A wait that expires sets the launch's status
+// word and leaves kRowExpired in the slot: the token then gets a row of zeros (AnyExpired), never the sum of the rows
+// that happened to be ready.
+constexpr int kRowExpired = -2;
+
+__device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
+{
+    bool expired = false;
+    for (int k = 0; k < slots; ++k) {
+        expired |= rows[k] == kRowExpired;
+    }
+    return expired;
+}
+
 template <bool FENCE>
 __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
     float *weights)
@@ -156,7 +170,7 @@ __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool 
             if (a.deviceStatus != nullptr) {
                 atomicExch(a.deviceStatus, 1);
             }
-            row = -1;
+            row = kRowExpired;
         }
         rows[k] = row;
         // shared-expert slots follow the routed ones and carry no gate weight
@@ -204,7 +218,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             }
             __syncthreads();
         }
-        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0);
+        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !(FL && AnyExpired(s_row[tg], a.slots));
 
         float acc[V][8];
 #pragma unroll
@@ -334,7 +348,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
         __syncthreads();
         LoadRoutes<false>(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
         __syncthreads();
-        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0);
+        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !(FL && AnyExpired(s_row[tg], a.slots));
 
         float acc[V][16];
 #pragma unroll
@@ -472,7 +486,8 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
             }
             __syncthreads();
         }
-        const bool active = a.tokenMask == nullptr || a.tokenMask[token] != 0;
+        const bool active = (a.tokenMask == nullptr || a.tokenMask[token] != 0) &&
+            !(a.tileFlags != nullptr && AnyExpired(s_row, a.slots));
         uint16_t *dst = static_cast<uint16_t *>(a.y) + static_cast<int64_t>(token) * a.h;
         const int blocks = (a.h + 31) / 32;
         for (int b = tid; b < blocks; b += kThreads) {

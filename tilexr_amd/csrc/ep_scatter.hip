@@ -19,10 +19,10 @@
 //   QMODE 5  fp8 e4m3, fp32 scale per 128 columns (no reference counterpart)
 #include <hip/hip_runtime.h>
 
-#include "ep_kernel_common.cuh"
+#include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
-#include "ep_numerics.cuh"
-#include "ep_place.cuh"
+#include "ep_numerics.hip.h"
+#include "ep_place.hip.h"
 #include "ep_tile_publish.h"
 #include "tilexr_ep.h"
 

@@ -8,10 +8,10 @@
 // 1159-1168, 1240-1258); only the number of launches differs.
 #include <hip/hip_runtime.h>
 
-#include "ep_block_scan.cuh"
-#include "ep_kernel_common.cuh"
+#include "ep_block_scan.hip.h"
+#include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
-#include "ep_numerics.cuh"
+#include "ep_numerics.hip.h"
 
 namespace TileXREp {
 namespace {

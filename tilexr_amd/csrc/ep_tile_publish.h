@@ -40,6 +40,18 @@ struct TilePublishArgs {
     uint64_t epoch;
 };
 
+// The word a complete tile is published with, and the consumer's test of a polled word: ready means "published for
+// exactly this epoch".  A word of an older epoch, a word of a newer one and a zero-filled word all read as not ready.
+TILEXR_EP_HD uint64_t TileReadyWord(uint64_t epoch, int rowsInTile)
+{
+    return (epoch << 32) | static_cast<uint32_t>(rowsInTile);
+}
+
+TILEXR_EP_HD bool TileWordReady(uint64_t word, uint64_t epoch)
+{
+    return (word >> 32) == epoch;
+}
+
 template <typename Ops>
 TILEXR_EP_HD bool CountLanded(Ops &ops, uint32_t *counter, int target)
 {
@@ -77,7 +89,7 @@ TILEXR_EP_HD void PublishLanded(Ops &ops, const TilePublishArgs &a, int row, int
             }
         }
     }
-    ops.Store(&a.flags[tile], (a.epoch << 32) | static_cast<uint32_t>(rowsInTile));
+    ops.Store(&a.flags[tile], TileReadyWord(a.epoch, rowsInTile));
 }
 
 } // namespace TileXREp

@@ -8,6 +8,7 @@
 
 #ifdef __cplusplus
 extern "C" {
+#pragma GCC visibility push(default)   // the entry points below are what the shared library exports
 #endif
 
 enum {
@@ -91,6 +92,7 @@ int TileXREpHookTilePublishStress(int totalRows, int maxRows, int tileRows, int 
     uint32_t seed, int fault);
 
 #ifdef __cplusplus
+#pragma GCC visibility pop
 }
 #endif
 

@@ -13,8 +13,8 @@
 
 #include <hip/hip_runtime.h>
 
-#include "ep_kernel_common.cuh"
-#include "ep_numerics.cuh"
+#include "ep_kernel_common.hip.h"
+#include "ep_numerics.hip.h"
 #include "moonep_stage.h"
 
 namespace TileXRMoon {
