@@ -19,6 +19,11 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+SCHEDULES = {
+    "flags-serial": "tile flags published by dispatch and awaited by combine, one stream",
+    "flags-overlapped": "tile flags published by dispatch and awaited by combine, combine on a second stream beside dispatch",
+    "plain": "no tile flags, one stream",
+}
 
 
 def measured_traffic(workload, kernel):
@@ -31,6 +36,23 @@ def measured_traffic(workload, kernel):
         parts = line.split("=")
         if len(parts) == 2 and parts[0].strip() == f"{kernel}_bytes_per_launch":
             return int(float(parts[1].strip()))
+    return None
+
+
+def trace_avg_us(workload, kernel):
+    """Average duration of a kernel from the committed rocprofv3 kernel-trace summary of this workload
+    (profiles/ep_dispatch_combine_<workload>_kernel_stats.txt: table rows `<kernel template> calls avg_us ...`), or
+    None.  Event-bracketed times read a few microseconds above it (an event record holds the queue)."""
+    path = os.path.join(ROOT, "profiles", f"ep_dispatch_combine_{workload}_kernel_stats.txt")
+    if not os.path.exists(path) or not kernel:
+        return None
+    for line in open(path):
+        if line.startswith(kernel):
+            parts = line.rsplit(None, 5)
+            try:
+                return float(parts[-4])
+            except (ValueError, IndexError):
+                return None
     return None
 
 
@@ -50,13 +72,16 @@ def parse():
     p.add_argument("--no-cpu-baseline", action="store_true")
     p.add_argument("--no-kernel-events", action="store_true",
                    help="do not record per-kernel HIP events inside the timed region")
-    p.add_argument("--overlap", action="store_true",
-                   help="run combine on a second stream, consuming tiles through readiness flags while dispatch is "
-                        "still writing rows")
+    p.add_argument("--schedule", default="auto", choices=["auto", "flags-serial", "flags-overlapped", "plain"],
+                   help="C2-C5: what a timed step is.  flags-serial: dispatch publishes tile readiness flags, combine "
+                        "waits on them, both on one stream; flags-overlapped: the same with combine on a second "
+                        "stream, reducing tiles while dispatch is still writing rows; plain: no flags; auto (default): "
+                        "the faster of the two flag schedules, decided by a short calibration before the timed steps")
+    p.add_argument("--overlap", action="store_true", help="same as --schedule flags-overlapped")
     p.add_argument("--tile-rows", type=int, default=64)
     p.add_argument("--no-overlap-leg", action="store_true",
-                   help="skip the extra, separately timed run of the other schedule that is reported under "
-                        "config.other_schedule")
+                   help="skip the extra, separately timed runs of the schedules that are not the timed one (reported "
+                        "under config.other_schedules)")
     p.add_argument("--moon-cached-row-bytes", type=int, default=None,
                    help="M1: value for TileXRMoonEpSetCachedRowBytes (0 = always the scatter kernel that tolerates "
                         "token rows that come from HBM)")
@@ -210,7 +235,6 @@ def main_moonep(args):
     import numpy as np
     import torch
 
-    from oracle import moonep as M
     from tilexr_amd import ep, moonep as mp, workloads
 
     w = workloads.MOONEP_CONFIGS[args.workload]
@@ -222,8 +246,7 @@ def main_moonep(args):
     plan = workloads.moonep_home_plan(ids, experts)
     nvs = plan["nvs"]
     dst = plan["dst"]
-    sh = M.Shape(world, s, k, h, nvs)
-    dst_local = torch.from_numpy(M.build_dst_local(sh, dst.numpy()))
+    dst_local = workloads.moonep_dst_local(dst, nvs)
     torch.cuda.set_device(0)
     dev = "cuda:0"
     comms = [ep.Comm(world, r) for r in range(world)]
@@ -436,7 +459,7 @@ def main():
     status = torch.zeros((1,), dtype=torch.int32, device=dev)
     meta_ready, combined = ep.HipEvent(), ep.HipEvent()
 
-    def step_serial(d_x=d_x):
+    def step_plain(d_x=d_x):
         st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
                                       ep.DT_BF16, stream, quant_mode=quant, expert_capacity=w.capacity,
                                       dynamic_scales=scales, row_index_map=row_map)
@@ -444,6 +467,19 @@ def main():
         ep.check(ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
                                       expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
                                       row_index_map=row_map), "combine")
+
+    def step_flags_serial(d_x=d_x):
+        # dispatch publishes a readiness word per tile of rows, combine waits for the tiles of every row it reads;
+        # one stream, so the waits find every tile published
+        st, epoch = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
+                                          ep.DT_BF16, stream, quant_mode=quant, expert_capacity=w.capacity,
+                                          dynamic_scales=scales, row_index_map=row_map, tile_flags=flags,
+                                          tile_rows=args.tile_rows)
+        ep.check(st, "dispatch")
+        ep.check(ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
+                                      expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
+                                      row_index_map=row_map, tile_flags=flags, tile_rows=args.tile_rows,
+                                      flag_epoch=epoch, device_status=status), "combine")
 
     def step_overlapped():
         # dispatch on `stream` publishes tiles; combine on `side` starts once the metadata is enqueued and reduces
@@ -461,7 +497,25 @@ def main():
         combined.record(side)
         combined.wait_on(stream)
 
-    step = step_overlapped if args.overlap else step_serial
+    steps_by_schedule = {"flags-serial": step_flags_serial, "flags-overlapped": step_overlapped, "plain": step_plain}
+    schedule = "flags-overlapped" if args.overlap else args.schedule
+    calibration = None
+    if schedule == "auto":
+        # the faster of the two schedules that publish and consume flags, by a short calibration outside the timed region
+        torch.cuda.synchronize()
+        calibration = {}
+        for name in ("flags-serial", "flags-overlapped"):
+            for _ in range(5):
+                steps_by_schedule[name]()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(20):
+                steps_by_schedule[name]()
+            torch.cuda.synchronize()
+            calibration[name] = round((time.perf_counter() - t0) / 20 * 1e6, 2)
+        schedule = min(calibration, key=calibration.get)
+    step = steps_by_schedule[schedule]
+    uses_flags = schedule != "plain"
 
     if args.calibrate_copy:
         src = torch.zeros((64 << 20,), dtype=torch.int32, device=dev)
@@ -503,43 +557,60 @@ def main():
     elapsed = time.perf_counter() - t0
     kernel_names = {"scatter": ep.last_kernel_name(comm, ep.K_SCATTER), "reduce": ep.last_kernel_name(comm, ep.K_REDUCE)}
 
-    if args.overlap and status.item() != 0:
+    if status.item() != 0:
         print("a tile-flag wait expired during the run", file=sys.stderr)
         sys.exit(1)
+    # the identity expert makes the layer checkable on the device: every kept row is its token's row, so y is the
+    # weighted sum of that row over the token's kept routes
+    if quant == ep.Q_NONE:
+        kept_w = torch.where(row_map >= 0, d_w, torch.zeros_like(d_w)).sum(1, keepdim=True)
+        ref = d_x.float() * kept_w
+        err = (y.float() - ref).abs().max().item()
+        if not err <= 2e-2 * ref.abs().max().item():
+            print(f"combine(dispatch(x)) is off by {err}", file=sys.stderr)
+            sys.exit(1)
+        del ref, kept_w
 
-    # split of one step into its two calls, run back to back on one stream (outside the timed region)
+    # split of one step into its two calls, run back to back on one stream (outside the timed region), with the timed
+    # schedule's flag settings
     d_ev[0].record(stream)
-    st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts, ep.DT_BF16,
-                                  stream, quant_mode=quant, expert_capacity=w.capacity, dynamic_scales=scales,
-                                  row_index_map=row_map)
+    st, epoch = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts, ep.DT_BF16,
+                                      stream, quant_mode=quant, expert_capacity=w.capacity, dynamic_scales=scales,
+                                      row_index_map=row_map, tile_flags=flags if uses_flags else None,
+                                      tile_rows=args.tile_rows if uses_flags else 0)
     d_ev[1].record(stream)
     ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
-                         expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w, row_index_map=row_map)
+                         expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w, row_index_map=row_map,
+                         tile_flags=flags if uses_flags else None, tile_rows=args.tile_rows if uses_flags else 0,
+                         flag_epoch=epoch, device_status=status if uses_flags else None)
     d_ev[2].record(stream)
     torch.cuda.synchronize()
     dispatch_us = d_ev[0].elapsed_ms(d_ev[1]) * 1e3
     combine_us = d_ev[1].elapsed_ms(d_ev[2]) * 1e3
 
-    # the other schedule (overlapped when the timed one is serial, and the other way round), timed on its own after
-    # the main region so that both are on record; it is not part of `value`
+    # the schedules that were not timed, each on its own after the main region so that all three are on record; they
+    # are not part of `value`
     other = None
     if not args.no_overlap_leg:
-        other_step = step_serial if args.overlap else step_overlapped
-        other_steps = max(10, args.steps // 2)
-        for _ in range(5):
-            other_step()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-        for _ in range(other_steps):
-            other_step()
-        torch.cuda.synchronize()
-        other_us = (time.perf_counter() - t1) / other_steps * 1e6
-        if status.item() != 0:
-            print("a tile-flag wait expired during the run", file=sys.stderr)
-            sys.exit(1)
-        other = {"schedule": "serial" if args.overlap else "overlapped via tile flags", "tile_rows": args.tile_rows,
-                 "steps": other_steps, "us_per_layer": round(other_us, 2),
-                 "GBps": round((dispatch_bytes + combine_bytes) / (other_us * 1e-6) / 1e9, 1)}
+        other = []
+        for name, other_step in steps_by_schedule.items():
+            if name == schedule:
+                continue
+            other_steps = max(10, args.steps // 2)
+            for _ in range(5):
+                other_step()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(other_steps):
+                other_step()
+            torch.cuda.synchronize()
+            other_us = (time.perf_counter() - t1) / other_steps * 1e6
+            if status.item() != 0:
+                print("a tile-flag wait expired during the run", file=sys.stderr)
+                sys.exit(1)
+            other.append({"schedule": SCHEDULES[name], "tile_rows": args.tile_rows if name != "plain" else None,
+                          "steps": other_steps, "us_per_layer": round(other_us, 2),
+                          "GBps": round((dispatch_bytes + combine_bytes) / (other_us * 1e-6) / 1e9, 1)})
 
     # the serial schedule once more with the token rows of every step in a different tensor, enough of them that none
     # is still in the 256 MiB memory-side cache when its turn comes again: what a caller sees whose x was produced long
@@ -549,15 +620,16 @@ def main():
         copies = max(2, -(-(384 << 20) // (bs * h * 2)))
         xs = [d_x] + [d_x.clone() for _ in range(copies - 1)]
         rot_steps = max(copies, args.steps // 2)
+        rot_step = step_plain if schedule == "plain" else step_flags_serial
         for i in range(copies):
-            step_serial(xs[i])
+            rot_step(xs[i])
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         for i in range(rot_steps):
-            step_serial(xs[i % copies])
+            rot_step(xs[i % copies])
         torch.cuda.synchronize()
         rot_us = (time.perf_counter() - t1) / rot_steps * 1e6
-        rotating = {"schedule": "serial", "input_tensors": copies, "steps": rot_steps, "us_per_layer": round(rot_us, 2),
+        rotating = {"schedule": SCHEDULES["plain" if schedule == "plain" else "flags-serial"], "input_tensors": copies, "steps": rot_steps, "us_per_layer": round(rot_us, 2),
                     "GBps": round((dispatch_bytes + combine_bytes) / (rot_us * 1e-6) / 1e9, 1)}
         del xs
 
@@ -606,6 +678,12 @@ def main():
                     "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4),
                     "traffic": measured_traffic(w.name, dom),
                     "avg_launch_us": kernels[dom]["avg_us"], "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
+        # the same kernel by the committed rocprofv3 kernel trace of this workload (no event records between kernels)
+        trace_us = trace_avg_us(w.name, kernel_names[dom])
+        if trace_us:
+            roofline["kernel_trace"] = {"avg_launch_us": trace_us, "source": f"profiles/ep_dispatch_combine_{w.name}_kernel_stats.txt",
+                                        "achieved": round(kernels[dom]["algorithmic_bytes"] / (trace_us * 1e-6) / 1e9, 1),
+                                        "frac": round(kernels[dom]["algorithmic_bytes"] / (trace_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
 
     ceilings = None
     if not args.no_ceilings:
@@ -622,8 +700,9 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "us_per_layer": round(ms_per_step * 1e3, 2),
         "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": dict(workloads.describe(w, ids), schedule="overlapped via tile flags" if args.overlap else "serial",
-                       other_schedule=other, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+        "config": dict(workloads.describe(w, ids), schedule=SCHEDULES[schedule],
+                       tile_rows=args.tile_rows if uses_flags else None, schedule_calibration_us=calibration,
+                       other_schedules=other, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
         "roofline": roofline, "kernels": kernels, "ceilings": ceilings,
     }

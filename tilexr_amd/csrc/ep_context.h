@@ -115,6 +115,11 @@ struct EpComm {
     DeviceBuffer combineScratch;
     DeviceBuffer drainScratch;
     DeviceBuffer tileCounters;        // rows landed per readiness tile; all zero whenever no dispatch is in flight
+    // The last dispatch of this communicator that published readiness flags: a combine on the same stream that waits for
+    // the same words and epoch finds every tile published (stream order), so it needs no room left for a producer.
+    const void *lastFlagWords = nullptr;
+    uint64_t lastFlagEpoch = 0;
+    hipStream_t lastFlagStream = nullptr;
     hipEvent_t timing[5][2] = {};     // optional (start, stop) pairs around each kernel, see tilexr_ep.h
     const char *lastKernel[5] = {};   // name of the kernel template last launched for each kernel id
     std::mutex mu;

@@ -669,7 +669,9 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     // A kernel that waits on flags must never crowd out the producer it waits for: its waiting waves keep their
     // registers, and with three or more of these workgroups per compute unit a producer workgroup no longer fits
     // beside them (measured: flag waits expire at six).  Two workgroups per compute unit walk the tokens.
-    const int gridLimit = l.tileFlags != nullptr ? 2 * (l.numComputeUnits > 0 ? l.numComputeUnits : 256) : 0;
+    // A launch whose flags were published earlier on its own stream never waits and gets the ordinary geometry.
+    const bool mayWait = l.tileFlags != nullptr && !l.producerOrdered;
+    const int gridLimit = mayWait ? 2 * (l.numComputeUnits > 0 ? l.numComputeUnits : 256) : 0;
     const int64_t vecs = l.h / 8;
     const bool plain = l.inQuant == 0 && l.h % 8 == 0 && Aligned16(l.y) && vecs <= 8 * kThreads &&
         Aligned16(l.expertOut) && l.rowBytes % 16 == 0 &&
@@ -701,9 +703,9 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
             LaunchByType<kWave, 2>(l, a, gridLimit);
         } else if (vecs <= 4 * kWave) {
             LaunchByType<kWave, 4>(l, a, gridLimit);
-        } else if (a.tileFlags != nullptr) {
-            // readiness flags: one workgroup per token, so that one wave polls the token's tiles instead of one per
-            // slice (waiters on a hot flag word slow down the producer's atomics on it)
+        } else if (mayWait) {
+            // readiness flags that may still be pending: one workgroup per token, so that one wave polls the token's
+            // tiles instead of one per slice, and few enough workgroups that the producer fits beside them
             if (vecs <= 2 * kThreads) {
                 LaunchByType<kThreads, 2>(l, a, gridLimit);
             } else if (vecs <= 4 * kThreads) {

@@ -113,7 +113,22 @@ class MoeEpLayer:
         order, one rounding to `dtype`.  expert_out has the row layout of `d.expand_x`."""
         q = _QUANT[expert_out_quant]
         bs, h = d.bs, self.hidden
+        # the library reads raw bytes: a tensor of another element type would be reinterpreted, not converted
+        want = {ep.Q_NONE: (dtype,), ep.Q_TOKEN_INT8: (torch.int8, torch.uint8),
+                ep.Q_FP8_BLOCK128: (torch.float8_e4m3fn, torch.uint8)}[q]
+        if expert_out.dtype not in want:
+            raise ValueError(f"expert_out is {expert_out.dtype}, expected one of {want} for this payload")
+        if expert_out.shape[-1] != h:
+            raise ValueError(f"expert_out rows have {expert_out.shape[-1]} columns, expected {h}")
         expert_out = expert_out.contiguous()
+        if q != ep.Q_NONE:
+            if expert_out_scales is None or expert_out_scales.dtype != torch.float32:
+                raise ValueError("a quantised expert_out needs float32 expert_out_scales")
+            expert_out_scales = expert_out_scales.contiguous()
+        if shared_expert_x is not None:
+            if shared_expert_x.dtype != dtype or tuple(shared_expert_x.shape) != (bs, h):
+                raise ValueError("shared_expert_x must be [bs, hidden] of the output type")
+            shared_expert_x = shared_expert_x.contiguous()
         if weights is not None:
             weights = weights.to(torch.float32).contiguous()
         y = torch.empty((bs, h), dtype=dtype, device=self.device)
@@ -175,9 +190,12 @@ class PlanDrivenLayer:
         mp = self._mp
         self._dst = dst.contiguous()
         raw = torch.where(self._dst >= 0, self._dst, -self._dst - 1).to(torch.int64)
-        # reverse routes: receive row -> rank * nvs + route (rank 0 here), -1 where no route lands
+        # reverse routes: receive row -> rank * nvs + route (rank 0 here), -1 where no route lands.  A row outside
+        # [0, nvs) is left out here (an index past the end would abort the device context); the library reports it
+        # through the plan's status word when the plan is used
+        ok = raw < self.nvs
         self._dst_local = torch.full((self.nvs,), -1, dtype=torch.int32, device=self.device)
-        self._dst_local[raw] = torch.arange(self.s * self.k, dtype=torch.int32, device=self.device)
+        self._dst_local[raw[ok]] = torch.arange(self.s * self.k, dtype=torch.int32, device=self.device)[ok]
         self._plan = mp.plan(self.s * self.k, 1, self.k, 1, self.nvs, self.k, self._dst, self._groups, self._loffs,
                              self._counts, self.status)
         self._built = False

@@ -195,6 +195,21 @@ def moonep_home_plan(topk_experts, experts, token_padding=1, prefetch_slots=1, s
     return {"dst": dst.to(torch.int32).contiguous(), "cu_seqlens": cu.to(torch.int32), "nvs": int(nvs)}
 
 
+def moonep_dst_local(dst, nvs):
+    """Reverse routes of a world for Combine: int32 [R, nvs], entry [rank][row] = source rank * nvs + route index of
+    the route that lands on that row, -1 where none does (reference: the dstLocal input of
+    src/moonep/combine/kernels/tilexr_moonep_combine_kernel.cpp:117-177).  `dst` int32 [R, S*K] as moonep_home_plan
+    returns it; raises ValueError for a route word outside the world."""
+    R, n = dst.shape
+    raw = torch.where(dst >= 0, dst, -dst - 1).to(torch.int64)
+    if int(raw.max()) >= R * nvs:
+        raise ValueError("a route word names a row outside the world")
+    out = torch.full((R * nvs,), -1, dtype=torch.int32)
+    src = torch.arange(R, dtype=torch.int64).unsqueeze(1) * nvs + torch.arange(n, dtype=torch.int64).unsqueeze(0)
+    out[raw.reshape(-1)] = src.reshape(-1).to(torch.int32)
+    return out.reshape(R, nvs)
+
+
 def moonep_algorithmic_bytes(s: int, k: int, h: int, with_weights: bool = True):
     """Bytes one rank's dispatch and combine must move when every route names its own row:
        dispatch = S*H*2 (read tokens once) + S*K*4 (route words) + S*K*H*2 (write rows) [+ S*K*8 weights in and out]
