@@ -185,6 +185,26 @@ int TileXRMoeEpCombineMemoryEx(void *expertOut, int32_t *assistInfoForCombine, i
     TileXRCommPtr comm, int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
     const TileXREpCombineExOptions *options, void *yOut, TileXR::TileXRDataType dtype, aclrtStream stream);
 
+// TileXRMoeEpDispatchMemory for callers that cannot allocate device memory at call time.  No counterpart in the
+// reference.  It is for code under HIP graph capture, serving loops that have handed all device memory to a pool of
+// their own, and harnesses that forbid hipMalloc: this call makes no hipMalloc / hipFree and calls no allocating
+// library routine.  Arguments, outputs, order of rows and return codes are those of TileXRMoeEpDispatchMemory; the
+// caller still passes every input and output.  What differs is where the kernels' scratch (per-route ranks, per-chunk
+// histograms, per-expert offsets) lives: in one static array of 2 MiB that every GPU the library runs on holds until
+// the process ends, instead of a buffer the communicator allocates and grows.
+//   * limits: rankSize 1; bs * topK routes and moeExpertNum experts whose count scratch fits the array (131 072 routes
+//     over 2048 experts do; about 8.3 bytes per route + 264 bytes per expert and 1024-route chunk).  Larger calls
+//     return TILEXR_ERROR_NOT_SUPPORT (-6) with a line on stderr that names the sizes, before a magic is drawn.
+//   * all calls on one GPU share that GPU's array, whatever their communicator or stream: calls that overlap in time
+//     on one GPU race on it.  Calls that follow one another on a stream, or are otherwise ordered, are fine; the array
+//     keeps the previous call's contents and the call clears what it needs cleared itself.
+//   * the array's device address is resolved when a communicator is created on the device (TileXRCommInitRankLocal);
+//     -1 (TILEXR_ERROR_NOT_INITIALIZED) if that failed.
+int TileXRMoeEpDispatchMemoryNoAlloc(void *x, int32_t *expertIds, TileXRCommPtr comm,
+    int64_t bs, int64_t h, int64_t topK, int64_t moeExpertNum,
+    void *expandXOut, int64_t *expertTokenNumsOut, int32_t *sendCountsOut,
+    int32_t *assistInfoForCombineOut, TileXR::TileXRDataType dtype, aclrtStream stream);
+
 // Measurement aid without a reference counterpart: while a pair of hipEvent_t is set for a kernel, every call on
 // `comm` that launches that kernel records `startEvent` immediately before and `stopEvent` immediately after it, on
 // the stream of the call.  Pass null events to clear.  Kernel ids: 0 count, 1 place, 2 scatter, 3 invert, 4 reduce.

@@ -14,6 +14,7 @@
 #include "ep_host.h"
 #include "ep_launch.h"
 #include "ep_run_common.h"
+#include "ep_static_scratch.h"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -66,10 +67,27 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
         }
     }
     const CountScratchLayout plan = PlanCountScratch(n, numKeys, experts, expertHist);
-    if (!comm->dispatchScratch.Reserve(static_cast<size_t>(plan.totalBytes), true)) {
-        return TileXR::TILEXR_ERROR_INTERNAL;
+    void *scratchBase = nullptr;
+    if (p.noAlloc) {
+        // this call may not allocate: the per-GPU static array or nothing
+        void *staticScratch = comm->world->staticScratchReady ? StaticScratchOnDevice(comm->world->device) : nullptr;
+        if (staticScratch == nullptr) {
+            return TileXR::TILEXR_ERROR_NOT_INITIALIZED;
+        }
+        if (plan.totalBytes > static_cast<int64_t>(kStaticScratchBytes)) {
+            return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // DispatchMemory has said why
+        }
+        scratchBase = staticScratch;
+        // the array keeps what the previous call left: the count kernel's ticket has to start at zero
+        if (ClearScratchWord(scratchBase, stream) != hipSuccess) {
+            return TileXR::TILEXR_ERROR_MKIRT;
+        }
+    } else {
+        if (!comm->dispatchScratch.Reserve(static_cast<size_t>(plan.totalBytes), true)) {
+            return TileXR::TILEXR_ERROR_INTERNAL;
+        }
+        scratchBase = comm->dispatchScratch.ptr;
     }
-    void *scratchBase = comm->dispatchScratch.ptr;
     const CountScratch scratch = CarveCountScratch(scratchBase, plan, expertHist);
     int32_t *rowOf = p.rowIndexMapOut != nullptr ? p.rowIndexMapOut :
         reinterpret_cast<int32_t *>(static_cast<char *>(scratchBase) + plan.rowOfOff);
@@ -329,6 +347,19 @@ int DispatchMemory(const EpDispatchParams &p)
     if (ret != kOk) {
         return ret;
     }
+    if (p.noAlloc) {
+        // worlds of several logical ranks stage rows in allocated buffers; and the static scratch has a fixed size
+        if (args->rankSize != 1 || !WithinKernelLimits(p.bs, p.h, p.topK, p.moeExpertNum)) {
+            return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+        }
+        const CountScratchLayout plan = PlanCountScratch(p.bs * p.topK, p.moeExpertNum, p.moeExpertNum, false);
+        if (plan.totalBytes > static_cast<int64_t>(kStaticScratchBytes)) {
+            std::fprintf(stderr, "tilexr-ep: %lld routes over %lld experts need %lld bytes of scratch, the entry point that "
+                "allocates nothing holds %lld\n", static_cast<long long>(p.bs * p.topK), static_cast<long long>(p.moeExpertNum),
+                static_cast<long long>(plan.totalBytes), static_cast<long long>(kStaticScratchBytes));
+            return TileXR::TILEXR_ERROR_NOT_SUPPORT;
+        }
+    }
     int64_t magic = 0;
     ret = TileXRCommNextMagic(p.comm, &magic);
     if (ret != kOk) {
@@ -556,6 +587,31 @@ int TileXRMoeEpDispatchMemory(void *x, int32_t *expertIds, TileXRCommPtr comm, i
     return TileXRMoeEpDispatchMemoryV2(x, expertIds, nullptr, nullptr, TILEXR_EP_ACTIVE_MASK_NONE, nullptr, comm, bs, h,
         topK, moeExpertNum, 0, 0, 1, 0, 0, 0, 0, 0, 0, kEpExpertTokenNumsTypeCount, expandXOut, nullptr,
         assistInfoForCombineOut, expertTokenNumsOut, sendCountsOut, nullptr, nullptr, dtype, dtype, stream);
+}
+
+int TileXRMoeEpDispatchMemoryNoAlloc(void *x, int32_t *expertIds, TileXRCommPtr comm, int64_t bs, int64_t h,
+    int64_t topK, int64_t moeExpertNum, void *expandXOut, int64_t *expertTokenNumsOut, int32_t *sendCountsOut,
+    int32_t *assistInfoForCombineOut, TileXR::TileXRDataType dtype, aclrtStream stream)
+{
+    EpDispatchParams p {};
+    p.x = x;
+    p.expertIds = expertIds;
+    p.comm = comm;
+    p.bs = bs;
+    p.h = h;
+    p.topK = topK;
+    p.moeExpertNum = moeExpertNum;
+    p.tpWorldSize = 1;
+    p.expertTokenNumsType = kEpExpertTokenNumsTypeCount;
+    p.expandXOut = expandXOut;
+    p.assistInfoForCombineOut = assistInfoForCombineOut;
+    p.expertTokenNumsOut = expertTokenNumsOut;
+    p.epRecvCountsOut = sendCountsOut;
+    p.dtype = dtype;
+    p.expandXOutDtype = dtype;
+    p.stream = stream;
+    p.noAlloc = true;
+    return DispatchMemory(p);
 }
 
 int TileXRMoeEpDispatchMemoryEx(void *x, int32_t *expertIds, TileXRCommPtr comm, int64_t bs, int64_t h,

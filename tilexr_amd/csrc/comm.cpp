@@ -9,6 +9,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include "ep_context.h"
+#include "ep_static_scratch.h"
 #include "moonep_host.h"
 #include "tilexr_api.h"
 #include "tilexr_types.h"
@@ -61,6 +62,8 @@ EpWorld *CreateWorld(int rankSize)
             hipStreamSynchronize(nullptr) == hipSuccess) {
             world->flagArea = static_cast<uint8_t *>(area);
             world->deviceReady = true;
+            // the per-GPU scratch of the entry point that allocates nothing: its address on this device
+            world->staticScratchReady = ResolveStaticScratch(device) == hipSuccess;
             int cus = 0;
             if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, device) == hipSuccess) {
                 world->numComputeUnits = cus;

@@ -84,6 +84,7 @@ struct EpWorld {
     int device = -1;
     int live = 0;
     bool deviceReady = false;
+    bool staticScratchReady = false;   // the static per-GPU scratch has an address on `device`
     int numComputeUnits = 0;
     std::vector<EpComm *> comms;
     uint8_t *flagArea = nullptr;

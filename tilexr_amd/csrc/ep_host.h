@@ -80,6 +80,8 @@ struct EpDispatchParams {
     int64_t *epochOut = nullptr;
     void *metaReadyEvent = nullptr;
     bool extended = false;
+    // TileXRMoeEpDispatchMemoryNoAlloc: the kernels' scratch is the per-GPU static array, nothing is allocated
+    bool noAlloc = false;
 };
 
 struct EpCombineParams {

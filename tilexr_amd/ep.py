@@ -22,7 +22,7 @@ Q_NONE, Q_STATIC_INT8, Q_TOKEN_INT8, Q_COMM_E5M2, Q_MXFP8, Q_FP8_BLOCK128 = 0, 1
 EXPORTS = (
     "TileXRMoeEpDispatch", "TileXRMoeEpDispatchV2", "TileXRMoeEpDispatchMemory", "TileXRMoeEpDispatchMemoryV2",
     "TileXRMoeEpCombine", "TileXRMoeEpCombineV2", "TileXRMoeEpCombineMemory", "TileXRMoeEpCombineMemoryV2",
-    "TileXRMoeEpDispatchMemoryEx", "TileXRMoeEpCombineMemoryEx", "TileXREpVersion", "TileXREpSetKernelTimingEvents",
+    "TileXRMoeEpDispatchMemoryEx", "TileXRMoeEpCombineMemoryEx", "TileXRMoeEpDispatchMemoryNoAlloc", "TileXREpVersion", "TileXREpSetKernelTimingEvents",
     "TileXREpLastKernelName", "TileXREpMemoryProbe",
     "TileXRCommInitRankLocal", "TileXRCommDestroy", "TileXRGetCommArgsHost", "TileXRGetCommArgsDev",
     "TileXRCommNextMagic",
@@ -83,6 +83,7 @@ def lib():
         simple_dispatch = [vp, vp, vp, i64, i64, i64, i64, vp, vp, vp, vp, i32, vp]
         _lib.TileXRMoeEpDispatch.argtypes = simple_dispatch
         _lib.TileXRMoeEpDispatchMemory.argtypes = simple_dispatch
+        _lib.TileXRMoeEpDispatchMemoryNoAlloc.argtypes = simple_dispatch
         simple_combine = [vp, vp, vp, vp, i64, i64, i64, i64, vp, i32, vp]
         _lib.TileXRMoeEpCombine.argtypes = simple_combine
         _lib.TileXRMoeEpCombineMemory.argtypes = simple_combine
@@ -166,6 +167,14 @@ def dispatch_memory(x, expert_ids, comm, bs, h, top_k, experts, expand_x, token_
     return lib().TileXRMoeEpDispatchMemory(_ptr(x), _ptr(expert_ids), _h(comm), bs, h, top_k, experts,
                                            _ptr(expand_x), _ptr(token_nums), _ptr(send_counts), _ptr(assist), dtype,
                                            _stream(stream))
+
+
+def dispatch_memory_no_alloc(x, expert_ids, comm, bs, h, top_k, experts, expand_x, token_nums, send_counts, assist,
+                             dtype, stream):
+    """TileXRMoeEpDispatchMemory with the kernels' scratch in the library's static per-GPU array: allocates nothing."""
+    return lib().TileXRMoeEpDispatchMemoryNoAlloc(_ptr(x), _ptr(expert_ids), _h(comm), bs, h, top_k, experts,
+                                                  _ptr(expand_x), _ptr(token_nums), _ptr(send_counts), _ptr(assist),
+                                                  dtype, _stream(stream))
 
 
 def dispatch_v2(x, expert_ids, comm, bs, h, top_k, experts, expand_x, assist, token_nums, recv_counts, dtype, stream,
