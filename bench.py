@@ -82,6 +82,14 @@ def parse():
     p.add_argument("--no-overlap-leg", action="store_true",
                    help="skip the extra, separately timed runs of the schedules that are not the timed one (reported "
                         "under config.other_schedules)")
+    p.add_argument("--no-stage-leg", action="store_true",
+                   help="skip the extra leg with a slow expert-stage stand-in between dispatch and combine (reported under "
+                        "config.expert_stage)")
+    p.add_argument("--stage-workgroups", type=int, default=64,
+                   help="expert-stage leg: workgroups of the producer (it must leave room for the waiting combine)")
+    p.add_argument("--stage-tile-rows", type=int, default=16, help="expert-stage leg: rows per readiness tile")
+    p.add_argument("--stage-tile-ns", type=int, default=40000,
+                   help="expert-stage leg: time the producer spends on a tile at least, in nanoseconds")
     p.add_argument("--moon-cached-row-bytes", type=int, default=None,
                    help="M1: value for TileXRMoonEpSetCachedRowBytes (0 = always the scatter kernel that tolerates "
                         "token rows that come from HBM)")
@@ -612,6 +620,77 @@ def main():
                           "steps": other_steps, "us_per_layer": round(other_us, 2),
                           "GBps": round((dispatch_bytes + combine_bytes) / (other_us * 1e-6) / 1e9, 1)})
 
+    # What the flags are for: an expert stage between dispatch and combine that is slower than memory and publishes
+    # tiles as it finishes them.  A stand-in producer of the library (a few workgroups copy expandX to expertOut tile by
+    # tile at a set pace) runs (a) followed by an ordinary combine on the same stream, (b) beside a combine on a second
+    # stream that waits on the producer's flags and reduces every token as soon as its tiles are there.  Not part of
+    # `value`.
+    expert_stage = None
+    if not args.no_stage_leg:
+        expert_out = torch.empty_like(expand_x)
+        stage_tile_rows = args.stage_tile_rows
+        stage_flags = torch.zeros(((rows_max + stage_tile_rows - 1) // stage_tile_rows,), dtype=torch.int64, device=dev)
+        stage_done, combine_done = ep.HipEvent(), ep.HipEvent()
+        st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts, ep.DT_BF16,
+                                      stream, quant_mode=quant, expert_capacity=w.capacity, dynamic_scales=scales,
+                                      row_index_map=row_map)
+        ep.check(st, "dispatch")
+        torch.cuda.synchronize()
+        epoch_counter = [1 << 20]
+
+        def producer():
+            epoch_counter[0] += 1
+            ep.check(ep.tile_producer_probe(expand_x, expert_out, kept_rows, row_bytes, stage_flags, stage_tile_rows,
+                                            epoch_counter[0], args.stage_workgroups, args.stage_tile_ns, stream), "producer")
+            return epoch_counter[0]
+
+        def stage_alone():
+            producer()
+
+        def stage_then_combine():
+            producer()
+            ep.check(ep.combine_memory_ex(expert_out, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
+                                          expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
+                                          row_index_map=row_map), "combine")
+
+        def stage_beside_combine():
+            # the producer is enqueued first; the next producer must not overwrite rows this combine still reads
+            epoch = producer()
+            ep.check(ep.combine_memory_ex(expert_out, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, side,
+                                          expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
+                                          row_index_map=row_map, tile_flags=stage_flags, tile_rows=stage_tile_rows,
+                                          flag_epoch=epoch, device_status=status), "combine")
+            combine_done.record(side)
+            combine_done.wait_on(stream)
+
+        def timed(fn, n):
+            for _ in range(3):
+                fn()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            for _ in range(n):
+                fn()
+            torch.cuda.synchronize()
+            return (time.perf_counter() - t1) / n * 1e6
+
+        n_stage = max(10, args.steps // 4)
+        alone_us = timed(stage_alone, n_stage)
+        serial_us = timed(stage_then_combine, n_stage)
+        y_serial = y.clone()
+        beside_us = timed(stage_beside_combine, n_stage)
+        if status.item() != 0:
+            print("a tile-flag wait expired during the expert-stage leg", file=sys.stderr)
+            sys.exit(1)
+        if not torch.equal(y.view(torch.int16), y_serial.view(torch.int16)):
+            print("combine beside the producer differs from combine after it", file=sys.stderr)
+            sys.exit(1)
+        expert_stage = {"producer": f"{args.stage_workgroups} workgroups copy expandX to expertOut tile by tile, at least "
+                                    f"{args.stage_tile_ns} ns per tile, publish each tile (release at agent scope + flag word)",
+                        "tile_rows": stage_tile_rows, "steps": n_stage, "producer_alone_us": round(alone_us, 2),
+                        "combine_after_producer_us": round(serial_us, 2), "combine_beside_producer_us": round(beside_us, 2),
+                        "saved_us": round(serial_us - beside_us, 2), "outputs_identical": True}
+        del expert_out, y_serial
+
     # the serial schedule once more with the token rows of every step in a different tensor, enough of them that none
     # is still in the 256 MiB memory-side cache when its turn comes again: what a caller sees whose x was produced long
     # before the dispatch.  Not part of `value`.
@@ -702,7 +781,7 @@ def main():
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": dict(workloads.describe(w, ids), schedule=SCHEDULES[schedule],
                        tile_rows=args.tile_rows if uses_flags else None, schedule_calibration_us=calibration,
-                       other_schedules=other, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+                       other_schedules=other, expert_stage=expert_stage, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
         "roofline": roofline, "kernels": kernels, "ceilings": ceilings,
     }

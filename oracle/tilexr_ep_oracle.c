@@ -694,6 +694,9 @@ void orc_mem_combine_rank(const orc_case *c, int32_t rank, int64_t max_rows, con
         if (rows < 0) {
             rows = 0;
         }
+        if (rows > max_rows) {
+            rows = max_rows;      /* the kernel trusts the count (:256-266); a count beyond the buffer stops at its end here */
+        }
         for (int64_t row = 0; row < rows; ++row) {
             const int32_t *tuple = assist + ((int64_t)er * max_rows + row) * 4;
             if (tuple[0] != rank || tuple[1] < 0 || (int64_t)tuple[1] >= c->bs || tuple[2] < 0 ||

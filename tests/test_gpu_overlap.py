@@ -214,3 +214,66 @@ def test_combine_follows_an_expert_stage_that_publishes_tiles_in_random_order():
             wy = O.mem_combine(case, 0, want["expand_x"].view(np.uint16)[None], want["assist"][None],
                                want["send_counts"][None], expert_scales=w)
             assert np.array_equal(bits16(y), wy), f"epoch {epoch}"
+
+
+@pytest.mark.parametrize("shape,tile_rows,workgroups,tile_ns", [((1024, 7168, 8, 64), 64, 48, 20000),
+                                                                ((2048, 2048, 6, 32), 100, 16, 5000),
+                                                                ((512, 1024, 4, 16), 8, 200, 0)])
+def test_combine_beside_a_slow_producer_that_publishes_tiles_as_it_goes(shape, tile_rows, workgroups, tile_ns):
+    """An expert-stage stand-in of the library (a HIP kernel: a few workgroups copy the dispatched rows into the expert
+    output tile by tile at a set pace, ordinary stores, one release at agent scope per tile, then the tile's word) runs
+    on one stream; combine runs beside it on another, waits per token for the tiles it needs and reads them from memory.
+    The expert output starts as garbage and is garbage again before every round, so a row that is read early, or from a
+    stale cache line, changes the result.  Three rounds on the same buffers with growing epochs."""
+    bs, h, K, E = shape
+    rng = np.random.default_rng(sum(shape) + tile_rows)
+    n = bs * K
+    tiles = (n + tile_rows - 1) // tile_rows
+    ids, w = routing(rng, bs, K, E)
+    x = torch.from_numpy(rng.standard_normal((bs, h)).astype(np.float32)).to(torch.bfloat16)
+    xb = bits16(x)
+    case = O.Case(1, bs, h, K, E, token_nums_type=1)
+    want = O.mem_dispatch(case, 0, xb[None], ids[None])
+    wy = O.mem_combine(case, 0, want["expand_x"].view(np.uint16)[None], want["assist"][None],
+                       want["send_counts"][None], expert_scales=w)
+    with Session() as s:
+        side = torch.cuda.Stream()
+        d_x, d_ids, d_w = x.to(DEV), to_dev(ids), to_dev(w)
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        st, _ = ep.dispatch_memory_ex(d_x, d_ids, s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, ep.DT_BF16, s.stream, row_index_map=out["row_map"])
+        assert st == 0
+        s.sync()
+        rows = int(counts[-1].item())
+        assert rows == n
+        expert_out = torch.empty((n, h * 2), dtype=torch.uint8, device=DEV)
+        flags = torch.zeros((tiles,), dtype=torch.int64, device=DEV)
+        status = torch.zeros((1,), dtype=torch.int32, device=DEV)
+        y = torch.empty((bs, h), dtype=torch.bfloat16, device=DEV)
+        for epoch in (11, 12, 4_000_000_000):
+            expert_out.fill_(0x7f)                 # bf16 0x7f7f = 3.4e38: an early read cannot go unnoticed
+            y.fill_(-1.0)
+            torch.cuda.synchronize()
+            print(f"slow producer: shape {shape} tile_rows {tile_rows} epoch {epoch}", flush=True)
+            # producer first: a waiting kernel enqueued ahead of it on a shared hardware queue would keep it out
+            assert ep.tile_producer_probe(out["expand_x"], expert_out, rows, h * 2, flags, tile_rows, epoch, workgroups,
+                                          tile_ns, s.stream) == 0
+            st = ep.combine_memory_ex(expert_out, out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, side,
+                                      expert_scales=d_w, row_index_map=out["row_map"], tile_flags=flags,
+                                      tile_rows=tile_rows, flag_epoch=epoch, wait_timeout_us=10_000_000,
+                                      device_status=status)
+            assert st == 0
+            s.sync()
+            side.synchronize()
+            assert status.item() == 0
+            assert np.array_equal(expert_out.cpu().numpy(), want["expand_x"])
+            assert np.array_equal(bits16(y), wy), f"epoch {epoch}"
+            f = flags.cpu().numpy().astype(np.uint64)
+            rows_in_tile = np.minimum(tile_rows, n - np.arange(tiles) * tile_rows)
+            assert np.array_equal(f, (np.uint64(epoch) << np.uint64(32)) | rows_in_tile.astype(np.uint64))
+    # argument checks of the stand-in
+    with Session() as s:
+        assert ep.tile_producer_probe(expert_out, expert_out, 0, 64, flags, 8, 1, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.tile_producer_probe(expert_out, expert_out, 8, 24, flags, 8, 1, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.tile_producer_probe(expert_out, expert_out, 8, 64, flags, 8, 0, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL

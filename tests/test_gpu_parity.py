@@ -510,3 +510,104 @@ def test_quantised_combine_input_on_every_code(dtype, quant):
         want = O.mem_combine(O.Case(1, bs, h, K, E, dtype=dtype), 0, payload[None], out["assist"].cpu().numpy()[None],
                              counts.cpu().numpy()[None], expert_scales=w, in_quant=quant, in_scales=scales)
         assert np.array_equal(bits16(y), want)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# corrupted assist tuples, counts and row maps: skipped, never followed
+# (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:256-266, 340-342; tilexr_ep_combine_kernel.cpp:94-97)
+# ---------------------------------------------------------------------------------------------------------------
+def _guarded(bs, h, dtype, fill):
+    """y as the middle of a larger buffer whose edges must stay as they are."""
+    tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+    whole = torch.full((bs + 64, h), fill, dtype=tdt, device=DEV)
+    return whole, whole[32:32 + bs]
+
+
+@pytest.mark.parametrize("shape", [(64, 64, 4, 16), (300, 1024, 8, 64), (2100, 256, 8, 256), (40, 7168, 8, 256)])
+@pytest.mark.parametrize("route", ["memory", "mvp"])
+def test_combine_skips_corrupted_tuples(shape, route):
+    from test_oracle_routes import corrupt_tuples
+    bs, h, K, E = shape
+    dtype = ep.DT_BF16 if route == "memory" else ep.DT_FP16
+    rng = np.random.default_rng(sum(shape) + len(route))
+    ids = ids_for(rng, bs, K, E, invalid=0.05)
+    _, xb = x_for(rng, bs, h, dtype, scale=3.0)
+    case = O.Case(1, bs, h, K, E, dtype=dtype)
+    d = (O.mem_dispatch if route == "memory" else O.mvp_dispatch)(case, 0, xb[None], ids[None])
+    rows = d["rows"]
+    counts_key = "send_counts" if route == "memory" else "recv_counts"
+    eo = d["expand_x"].view(np.uint16).copy()
+    for r in range(rows):
+        eo[r] = np.roll(eo[r], r % 5)
+    assist = d["assist"].copy()
+    corrupt_tuples(rng, assist[None], [rows], bs, K, 1, max(6, rows // 10))
+    if route == "memory":
+        # a duplicate: a later row that claims the slot of an intact earlier one (the later row wins)
+        intact = [r for r in range(rows) if np.array_equal(assist[r], d["assist"][r])]
+        assist[intact[-1], :3] = assist[intact[0], :3]
+    w = (0.25 + rng.random((bs, K))).astype(np.float32)
+    for count_case in ("as dispatched", "past the buffer", "negative"):
+        counts = d[counts_key].copy()
+        if count_case == "past the buffer":
+            counts[-1] = bs * K + 12345 if route == "memory" else bs * K + 1       # MVP: outside [0, bs*K] reads as 0
+        elif count_case == "negative":
+            counts[-1] = -7
+        with Session() as s:
+            whole, y = _guarded(bs, h, dtype, 9.0)
+            d_eo = torch.full((bs * K, h), 0x7f7f, dtype=torch.int16, device=DEV)      # rows past `rows` hold 3.4e38
+            d_eo[:eo.shape[0]] = torch.from_numpy(eo.view(np.int16)).to(DEV)
+            d_assist = torch.full((bs * K, 4), -77, dtype=torch.int32, device=DEV)
+            d_assist[:assist.shape[0]] = torch.from_numpy(assist).to(DEV)
+            torch.cuda.synchronize()
+            print(f"corrupted tuples: {route} {shape} counts {count_case}", flush=True)
+            if route == "memory":
+                st = ep.combine_memory_v2(d_eo, d_assist, to_dev(counts), s.comm, bs, h, K, E, y, dtype, s.stream,
+                                          expert_scales=to_dev(w))
+            else:
+                st = ep.combine_v2(d_eo, d_assist, to_dev(counts), s.comm, bs, h, K, E, y, dtype, s.stream)
+            assert st == 0
+            s.sync()
+            host_eo = d_eo.cpu().numpy().view(np.uint16)[None]
+            host_assist = d_assist.cpu().numpy()[None]
+            if route == "memory":
+                want = O.mem_combine(case, 0, host_eo, host_assist, counts[None], expert_scales=w)
+            else:
+                want = O.mvp_combine(case, 0, host_eo, host_assist, counts[None])
+            assert np.array_equal(bits16(y), want), count_case
+            edges = torch.cat([whole[:32], whole[32 + bs:]])
+            assert torch.all(edges == 9.0)                  # nothing was stored outside y
+
+
+def test_combine_ignores_row_map_entries_outside_the_buffer():
+    """The row map dispatch hands to combine is trusted input, but an entry at or beyond bs * topK (or below -1) must
+    read as "no row": the kernels never touch memory outside the rows the caller's buffer holds."""
+    bs, h, K, E = 200, 1024, 4, 32
+    rng = np.random.default_rng(5)
+    ids = ids_for(rng, bs, K, E)
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+    case = O.Case(1, bs, h, K, E, dtype=O.DT_BF16)
+    d = O.mem_dispatch(case, 0, xb[None], ids[None])
+    w = (0.25 + rng.random((bs, K))).astype(np.float32)
+    with Session() as s:
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, ep.DT_BF16, s.stream, row_index_map=out["row_map"])
+        assert st == 0
+        s.sync()
+        row_map = out["row_map"].cpu().numpy().copy()
+        assist = d["assist"].copy()
+        for j, (t, k) in enumerate([(0, 0), (5, 3), (77, 1), (199, 3), (100, 2)]):
+            row = row_map[t, k]
+            row_map[t, k] = [bs * K, 0x7fffffff, -5, bs * K + 7, -2147483648][j]
+            assist[row, 1] = -1                     # the oracle learns of the same loss through the tuple
+        whole, y = _guarded(bs, h, ep.DT_BF16, 9.0)
+        torch.cuda.synchronize()
+        st = ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream,
+                                  expert_scales=to_dev(w), row_index_map=to_dev(row_map))
+        assert st == 0
+        s.sync()
+        want = O.mem_combine(case, 0, d["expand_x"].view(np.uint16)[None], assist[None], d["send_counts"][None],
+                             expert_scales=w)
+        assert np.array_equal(bits16(y), want)
+        assert torch.all(torch.cat([whole[:32], whole[32 + bs:]]) == 9.0)

@@ -685,3 +685,109 @@ def test_tensor_parallel_groups_match_demo_golden(orc, shape, masked):
             o = orc.mvp_dispatch(case, g + lane, x, ids, mask)
             sets.append(sorted(map(tuple, o["assist"][:o["rows"]].tolist())))
         assert all(s == sets[0] for s in sets)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# corrupted assist tuples and counts: skipped, never followed
+# (src/ep/kernels/tilexr_ep_combine_memory_kernel.h:256-266, 340-342; tilexr_ep_combine_kernel.cpp:28-52, 94-97)
+# ---------------------------------------------------------------------------------------------------------------
+def corrupt_tuples(rng, assist, rows, bs, K, rank_size, how_many):
+    """Plants the mistakes the kernels must survive into `how_many` random rows of each rank's table; returns the
+    rows that were touched.  A later test with the same seed reproduces the same table."""
+    bad = {}
+    for er in range(assist.shape[0]):
+        picks = rng.choice(rows[er], size=min(how_many, rows[er]), replace=False)
+        for j, row in enumerate(picks):
+            kind = j % 6
+            if kind == 0:
+                assist[er, row, 1] = -1
+            elif kind == 1:
+                assist[er, row, 1] = bs
+            elif kind == 2:
+                assist[er, row, 2] = K
+            elif kind == 3:
+                assist[er, row, 2] = -3
+            elif kind == 4:
+                assist[er, row, 0] = rank_size + 5            # a rank that does not exist
+            else:
+                assist[er, row, 1] = 0x7fffffff
+        bad[er] = set(int(r) for r in picks)
+    return bad
+
+
+def np_bf16(f):
+    return torch.from_numpy(np.ascontiguousarray(f, np.float32)).to(torch.bfloat16).view(torch.int16).numpy().view(np.uint16)
+
+
+def np_memory_combine_walk(rank, bs, h, K, expert_out, assist, send_counts, w):
+    """Plain walk over the rows, written without reference to the oracle's code: rows [0, min(count, buffer)) of every
+    expert rank; a row whose tuple names this rank, a token in [0, bs) and a slot in [0, K) fills that slot (a later
+    row replaces an earlier one); y[t] = bf16(sum over k in order of fp32(w * row))."""
+    R, max_rows = assist.shape[0], assist.shape[1]
+    slot = {}
+    for er in range(R):
+        rows = min(max(int(send_counts[er][-1]), 0), max_rows)
+        for row in range(rows):
+            s, t, k, _ = (int(v) for v in assist[er, row])
+            if s != rank or not 0 <= t < bs or not 0 <= k < K:
+                continue
+            slot[(t, k)] = (er, row)
+    y = np.zeros((bs, h), np.float32)
+    for t in range(bs):
+        acc = np.zeros(h, np.float32)
+        for k in range(K):
+            if (t, k) in slot:
+                er, row = slot[(t, k)]
+                r = (expert_out[er, row].astype(np.uint32) << 16).view(np.float32)
+                acc = (acc + (r * np.float32(w[t, k])).astype(np.float32)).astype(np.float32)
+        y[t] = acc
+    return np_bf16(y)
+
+
+def test_memory_combine_skips_corrupted_tuples_like_a_plain_walk(orc):
+    rng = np.random.default_rng(71)
+    R, bs, h, K, E = 2, 24, 32, 4, 8
+    ids = rand_ids(rng, R, bs, K, E, 0.05)
+    x = np_bf16(rng.standard_normal((R, bs, h)) * 3)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_BF16)
+    expert_out, assist, counts = _dispatch_all(orc, case, x, ids, memory=True)
+    rows = [int(counts[er][-1]) for er in range(R)]
+    w = (0.5 + rng.random((R, bs, K))).astype(np.float32)
+    clean = [orc.mem_combine(case, r, expert_out, assist, counts, expert_scales=w[r]) for r in range(R)]
+    bad = corrupt_tuples(rng, assist, rows, bs, K, R, 12)
+    # one duplicate as well: a second row that claims the slot of an intact one (the later row wins)
+    er, victim = 0, next(r for r in range(rows[0]) if r not in bad[0])
+    thief = next(r for r in range(victim + 1, rows[0]) if r not in bad[0])
+    assist[er, thief, :3] = assist[er, victim, :3]
+    # and a count that runs past the buffer: the walk stops at the buffer's end
+    counts = counts.copy()
+    counts[1][-1] = assist.shape[1] + 1000
+    for rank in range(R):
+        y = orc.mem_combine(case, rank, expert_out, assist, counts, expert_scales=w[rank])
+        assert np.array_equal(y, np_memory_combine_walk(rank, bs, h, K, expert_out, assist, counts, w[rank]))
+        assert not np.array_equal(y, clean[rank])        # the planted rows really mattered
+
+
+def test_mvp_combine_skips_corrupted_tuples_like_a_plain_walk(orc):
+    rng = np.random.default_rng(73)
+    R, bs, h, K, E = 2, 16, 16, 3, 6
+    ids = rand_ids(rng, R, bs, K, E)
+    xf = (rng.standard_normal((R, bs, h)) * 5).astype(np.float16)
+    case = O.Case(R, bs, h, K, E, dtype=O.DT_FP16)
+    expert_out, assist, counts = _dispatch_all(orc, case, xf.view(np.uint16), ids, memory=False)
+    rows = [int(counts[er].sum()) for er in range(R)]
+    corrupt_tuples(rng, assist, rows, bs, K, R, 9)
+    counts = counts.copy()
+    counts[1][0] = -4                      # a count outside [0, bs * K] reads as 0: rank 0 gets nothing from rank 1,
+    for rank in range(R):                  # and rank 1's own rows start at row 0 of that table
+        y = orc.mvp_combine(case, rank, expert_out, assist, counts)
+        want = np.zeros((bs, h), np.float16)
+        for er in range(R):
+            c = [int(v) if 0 <= int(v) <= bs * K else 0 for v in counts[er]]
+            start = sum(c[:rank])
+            for row in range(start, start + c[rank]):
+                _, t, k, _ = (int(v) for v in assist[er, row])
+                if not 0 <= t < bs or not 0 <= k < K:
+                    continue               # the rank field is overwritten on the way (combine_kernel.cpp:28-52)
+                want[t] = (want[t].astype(np.float32) + expert_out[er, row].view(np.float16).astype(np.float32)).astype(np.float16)
+        assert np.array_equal(y, want.view(np.uint16))

@@ -250,6 +250,7 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     red.bs = p.bs;
     red.h = p.h;
     red.topK = p.topK;
+    red.maxRows = n;
     red.y = p.yOut;
     red.tileFlags = p.tileFlags;
     red.tileRows = std::min<int64_t>(p.tileRows, std::max<int64_t>(n, 1));

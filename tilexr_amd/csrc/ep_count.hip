@@ -407,7 +407,19 @@ __global__ __launch_bounds__(kThreads) void ep_invert_kernel(InvertArgs a)
     if ((a.countsArePrefix && srcRank != a.rank) || token < 0 || token >= a.bs || k < 0 || k >= a.topK) {
         return;
     }
-    a.inverse[static_cast<int64_t>(token) * a.topK + k] = (a.epoch << 32) | static_cast<uint32_t>(row);
+    // Two rows that name the same (token, k) -- only a corrupted table has them -- leave the higher row, whatever the
+    // order the threads run in (the reference's sequential walk lets the later row win as well).  A word of another
+    // epoch is stale and always replaced.
+    unsigned long long *slot = reinterpret_cast<unsigned long long *>(&a.inverse[static_cast<int64_t>(token) * a.topK + k]);
+    const unsigned long long mine = (a.epoch << 32) | static_cast<uint32_t>(row);
+    unsigned long long seen = *slot;
+    while ((seen >> 32) != a.epoch || seen < mine) {
+        const unsigned long long prev = atomicCAS(slot, seen, mine);
+        if (prev == seen) {
+            break;
+        }
+        seen = prev;
+    }
 }
 
 int KeyBits(int64_t numKeys)

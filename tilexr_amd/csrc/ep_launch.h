@@ -156,6 +156,7 @@ struct ReduceLaunch {
     int64_t bs;
     int64_t h;
     int64_t topK;
+    int64_t maxRows;                 // rows expertOut holds: map entries at or beyond it count as "no row"; 0 = unchecked
     int64_t sharedSlots;             // slots per token beyond topK (shared experts): summed after the routed ones
                                      // with weight 1; the row map / inverse then has topK + sharedSlots entries
                                      // per token while expertScales keeps topK

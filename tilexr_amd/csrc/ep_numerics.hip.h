@@ -44,6 +44,13 @@ __device__ __forceinline__ uint32_t FloatToBf16Rne(float v)
     return FloatPairToBf16Rne(v, 0.0f) & 0xffffu;
 }
 
+// An fp32 value rounded to bf16 (same rounding), returned as fp32: the pair convert with 0.0 in the low half leaves the
+// rounded value's own fp32 bit pattern, so one instruction does the rounding and no unpacking follows.
+__device__ __forceinline__ float FloatRoundedToBf16(float v)
+{
+    return __uint_as_float(FloatPairToBf16Rne(0.0f, v));
+}
+
 // IEEE round-to-nearest-even; overflow becomes infinity.
 __device__ __forceinline__ uint32_t FloatToHalfRne(float v)
 {
@@ -176,6 +183,19 @@ __device__ __forceinline__ uint32_t Fp8E4m3EncodePairSat(float lo, float hi)
 __device__ __forceinline__ bool Fp8E4m3WordHasNan(uint32_t word)
 {
     return (((word & 0x7f7f7f7fu) + 0x01010101u) & 0x80808080u) != 0u;
+}
+
+// Four e4m3 codes -> four fp32 through the hardware convert alone: the values of Fp8Decode<false> for every code but
+// the NaN code 0x7f, whose NaN comes back with the other sign.  For callers that notice a NaN in their result and then
+// redo the work with Fp8E4m3DecodeWord.
+__device__ __forceinline__ void Fp8E4m3DecodeWordFast(uint32_t word, float *out)
+{
+    const f32x2 lo = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), false);
+    const f32x2 hi = __builtin_amdgcn_cvt_pk_f32_fp8(static_cast<int>(word), true);
+    out[0] = lo[0];
+    out[1] = lo[1];
+    out[2] = hi[0];
+    out[3] = hi[1];
 }
 
 // Four e4m3 codes -> four fp32, same values as Fp8Decode<false> (NaN codes take the software path).

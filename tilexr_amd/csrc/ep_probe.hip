@@ -10,6 +10,10 @@
 //   gather    the same mix with the reduce's addresses: every output row of 14 KiB combines eight rows of src that lie
 //             at unrelated positions
 //
+//   tile producer   a stand-in for an expert stage between dispatch and combine: a few workgroups copy rows tile by tile,
+//             spend a set time per tile, and publish every tile's readiness word the way any producer outside this
+//             library has to: rows complete, release at agent scope, then the word
+//
 // No reference counterpart; nothing on the dispatch / combine path calls these.
 #include <hip/hip_runtime.h>
 
@@ -123,8 +127,70 @@ __global__ __launch_bounds__(kWave) void ep_probe_gather_rows_kernel(const u32x4
     __builtin_nontemporal_store(acc, dst + static_cast<int64_t>(t) * kProbeRowVecs + at);
 }
 
+// Tiles t = blockIdx.x, blockIdx.x + gridDim.x, ... in turn.  Ordinary loads and stores (the rows may sit dirty in this
+// XCD's L2), then per tile: every wave waits for its stores, the barrier collects the waves, one lane writes the L2 back
+// with a release fence at agent scope and stores the word.  One such fence per tile of tens of rows is cheap; one per row
+// is not (the scatter kernels therefore write rows through instead).
+__global__ __launch_bounds__(kThreads) void ep_probe_tile_producer_kernel(const char *src, char *dst, int rows,
+    int64_t rowBytes, uint64_t *tileFlags, int tileRows, uint64_t epoch, int64_t minTileTicks)
+{
+    const int tiles = (rows + tileRows - 1) / tileRows;
+    const int64_t vecsPerRow = rowBytes / 16;
+    for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const uint64_t begin = wall_clock64();
+        const int first = tile * tileRows;
+        const int count = min(tileRows, rows - first);
+        const u32x4 *in = reinterpret_cast<const u32x4 *>(src + static_cast<int64_t>(first) * rowBytes);
+        u32x4 *out = reinterpret_cast<u32x4 *>(dst + static_cast<int64_t>(first) * rowBytes);
+        const int64_t vecs = vecsPerRow * count;
+        for (int64_t at = threadIdx.x; at < vecs; at += 4 * kThreads) {
+            u32x4 v[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t idx = at + static_cast<int64_t>(i) * kThreads;
+                v[i] = idx < vecs ? in[idx] : u32x4{0u, 0u, 0u, 0u};
+            }
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const int64_t idx = at + static_cast<int64_t>(i) * kThreads;
+                if (idx < vecs) {
+                    out[idx] = v[i];
+                }
+            }
+        }
+        // the time an expert stage would spend computing the tile
+        while (static_cast<int64_t>(wall_clock64() - begin) < minTileTicks) {
+            __builtin_amdgcn_s_sleep(32);
+        }
+        WaitOwnStores();
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            __hip_atomic_store(&tileFlags[tile], (epoch << 32) | static_cast<uint32_t>(count), __ATOMIC_RELAXED,
+                __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+}
+
 } // namespace
 } // namespace TileXREp
+
+extern "C" int TileXREpTileProducerProbe(const void *src, void *dst, int64_t rows, int64_t rowBytes, uint64_t *tileFlags,
+    int64_t tileRows, int64_t epoch, int64_t workgroups, int64_t minTileNs, aclrtStream stream)
+{
+    using namespace TileXREp;
+    if (src == nullptr || dst == nullptr || tileFlags == nullptr || stream == nullptr || !Aligned16(src) || !Aligned16(dst) ||
+        rows <= 0 || rows > 0x7fffffff || rowBytes <= 0 || rowBytes % 16 != 0 || tileRows <= 0 || tileRows > 0x7fffffff ||
+        epoch <= 0 || epoch > 0xffffffffll || workgroups <= 0 || workgroups > 65535 || minTileNs < 0 ||
+        minTileNs > 1000000000ll) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    const int64_t ticks = minTileNs / 10;       // wall_clock64() counts at 100 MHz
+    hipLaunchKernelGGL(ep_probe_tile_producer_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(kThreads), 0,
+        static_cast<hipStream_t>(stream), static_cast<const char *>(src), static_cast<char *>(dst), static_cast<int>(rows),
+        rowBytes, tileFlags, static_cast<int>(tileRows), static_cast<uint64_t>(epoch), ticks);
+    return hipGetLastError() == hipSuccess ? TileXR::TILEXR_SUCCESS : TileXR::TILEXR_ERROR_MKIRT;
+}
 
 extern "C" int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int64_t bytes, aclrtStream stream)
 {

@@ -17,6 +17,8 @@
 //                 type first (no reference counterpart)
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
 #include "ep_numerics.hip.h"
@@ -40,6 +42,7 @@ struct ReduceArgs {
     int bs;
     int h;
     int topK;
+    int maxRows;                     // rows expertOut holds
     int slots;                       // rows summed per token: topK routed ones, then the shared-expert slots
     void *y;
     int colSlices;                   // slices a row is cut into (vec kernel, wide rows), else 1
@@ -50,13 +53,18 @@ struct ReduceArgs {
     int32_t *deviceStatus;
 };
 
+// Row of a (token, slot), -1 for none.  A row at or beyond `maxRows` (only a corrupted map has one) counts as none: the
+// kernels never read outside the rows the caller's buffer holds.
 __device__ __forceinline__ int LookupRow(const ReduceArgs &a, int64_t slot)
 {
+    int row;
     if (a.rowIndexMap != nullptr) {
-        return a.rowIndexMap[slot];
+        row = a.rowIndexMap[slot];
+    } else {
+        const uint64_t e = a.inverseTagged[slot];
+        row = (e >> 32) == a.epoch ? static_cast<int>(e & 0xffffffffu) : -1;
     }
-    const uint64_t e = a.inverseTagged[slot];
-    return (e >> 32) == a.epoch ? static_cast<int>(e & 0xffffffffu) : -1;
+    return static_cast<unsigned>(row) < static_cast<unsigned>(a.maxRows) ? row : -1;
 }
 
 // Bounded wait until the tile holding `row` has been published for this epoch (its word carries the epoch).  The poll itself is a relaxed
@@ -145,10 +153,24 @@ __device__ __forceinline__ float ScaleLoad(const float *p)
     return *p;
 }
 
-// Fills s_row / s_w for one token; waits for tile flags when asked to.  A wait that expires sets the launch's status
-// word and leaves kRowExpired in the slot: the token then gets a row of zeros (AnyExpired), never the sum of the rows
-// that happened to be ready.
+// One look at the tile holding `row`: published for this epoch or not.
+__device__ __forceinline__ bool TilePublished(const ReduceArgs &a, int row)
+{
+    const uint64_t w = __hip_atomic_load(&a.tileFlags[row / a.tileRows], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return TileWordReady(w, a.flagEpoch);
+}
+
+// Fills s_row / s_w for one token and deals with tile flags.  BLOCK: every slot waits (bounded) for its tile.  Otherwise
+// `mode` says what a slot does about its tile:
+//   kRouteCheck    look once; a tile that is not there yet leaves kRowPending in the slot and the call returns true
+//                  ("come back later")
+//   kRouteTrusted  nothing: the caller has just seen every tile of this token published
+//   kRouteGiveUp   look once; a tile that is not there turns the slot into an expired one
+// An expired wait sets the launch's status word and leaves kRowExpired in the slot: the token then gets a row of zeros
+// (AnyExpired), never the sum of the rows that happened to be ready.
 constexpr int kRowExpired = -2;
+constexpr int kRowPending = -3;
+enum RouteMode : int { kRouteCheck = 0, kRouteTrusted = 1, kRouteGiveUp = 2 };
 
 __device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
 {
@@ -159,18 +181,25 @@ __device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
     return expired;
 }
 
-template <bool FENCE>
-__device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
-    float *weights)
+template <bool FENCE, bool BLOCK>
+__device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
+    float *weights, int mode)
 {
+    bool pending = false;
     for (int k = lane; k < a.slots; k += lanes) {
         const int64_t slot = static_cast<int64_t>(tokOk ? token : 0) * a.slots + k;
         int row = tokOk ? LookupRow(a, slot) : -1;
-        if (row >= 0 && a.tileFlags != nullptr && !WaitTile(a, row)) {
-            if (a.deviceStatus != nullptr) {
-                atomicExch(a.deviceStatus, 1);
+        if (row >= 0 && a.tileFlags != nullptr && (BLOCK || mode != kRouteTrusted)) {
+            const bool there = BLOCK ? WaitTile(a, row) : TilePublished(a, row);
+            if (!there && !BLOCK && mode == kRouteCheck) {
+                row = kRowPending;
+                pending = true;
+            } else if (!there) {
+                if (a.deviceStatus != nullptr) {
+                    atomicExch(a.deviceStatus, 1);
+                }
+                row = kRowExpired;
             }
-            row = kRowExpired;
         }
         rows[k] = row;
         // shared-expert slots follow the routed ones and carry no gate weight
@@ -182,6 +211,113 @@ __device__ __forceinline__ void LoadRoutes(const ReduceArgs &a, int token, bool 
         // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
         // workgroup after the barrier that follows) are at least as new as the flag values seen above
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    return pending;
+}
+
+// Runs unit(group) for this workgroup's groups: blockIdx.x, blockIdx.x + gridDim.x, ...  `load(group, mode)` fills the
+// workgroup's route tables for a group and returns (per lane) whether a tile it needs is not published yet;
+// `tokenAt(group, t)` names the t-th of a group's `tokensPerGroup` tokens (-1 = none).
+//
+// Without readiness flags that is a plain loop.  With them (WAITS) a workgroup never sits on one group while others it
+// owes are ready: a token needs the tiles of all its rows, which a producer that works tile by tile finishes at
+// unrelated times, so tokens become ready in no particular order.  The workgroup takes its groups 32 at a time.  A
+// first pass reduces every group whose tiles are there already (all of them when the producer ran earlier on the same
+// stream).  For what is left it then goes in rounds: all lanes together look once at every tile the pending groups need
+// (one round trip for the lot), the groups that have become complete are reduced, and a round without any is followed
+// by a sleep that grows to about 14 us.  When nothing it owes has become ready for the wait bound, or another workgroup
+// has reported an expired wait, the rest is given up: those tokens get rows of zeros and the launch's status word is set.
+template <bool WAITS, typename TokenAt, typename Load, typename Unit>
+__device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, int tokensPerGroup, TokenAt tokenAt,
+    Load load, Unit unit)
+{
+    if constexpr (!WAITS) {
+        for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+            __syncthreads();        // the previous iteration's readers are done with the route tables
+            load(group, kRouteTrusted);
+            __syncthreads();
+            unit(group);
+        }
+    } else {
+        __shared__ uint32_t s_notReady;
+        const int first = static_cast<int>(blockIdx.x);
+        const int stride = static_cast<int>(gridDim.x);
+        const int mine = groups > first ? (groups - 1 - first) / stride + 1 : 0;
+        const int perGroup = tokensPerGroup * a.slots;
+        for (int base = 0; base < mine; base += 32) {
+            const int inWindow = mine - base < 32 ? mine - base : 32;
+            uint32_t pending = inWindow == 32 ? 0xffffffffu : ((1u << inWindow) - 1u);
+            for (uint32_t m = pending; m != 0u; m &= m - 1u) {
+                const int i = __builtin_ctz(m);
+                const int group = first + (base + i) * stride;
+                __syncthreads();
+                const bool waiting = load(group, kRouteCheck);
+                if (__syncthreads_or(waiting ? 1 : 0) != 0) {
+                    continue;                       // uniform: every lane gets the same answer
+                }
+                unit(group);
+                pending &= ~(1u << i);
+            }
+            uint64_t idleSince = wall_clock64();
+            int backoff = 0;
+            while (pending != 0u) {
+                if (threadIdx.x == 0) {
+                    s_notReady = 0u;
+                }
+                __syncthreads();
+                for (int idx = threadIdx.x; idx < inWindow * perGroup; idx += blockDim.x) {
+                    const int i = idx / perGroup;
+                    if (((pending >> i) & 1u) == 0u) {
+                        continue;
+                    }
+                    const int token = tokenAt(first + (base + i) * stride, (idx % perGroup) / a.slots);
+                    if (token < 0) {
+                        continue;
+                    }
+                    const int row = LookupRow(a, static_cast<int64_t>(token) * a.slots + idx % a.slots);
+                    if (row >= 0 && !TilePublished(a, row)) {
+                        atomicOr(&s_notReady, 1u << i);
+                    }
+                }
+                __syncthreads();
+                const uint32_t ready = pending & ~s_notReady;
+                if (ready == 0u) {
+                    bool stop = false;
+                    if (threadIdx.x == 0) {
+                        stop = static_cast<int64_t>(wall_clock64() - idleSince) > a.waitTimeoutTicks ||
+                            (a.deviceStatus != nullptr &&
+                             __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0);
+                    }
+                    if (__syncthreads_or(stop ? 1 : 0) != 0) {
+                        for (uint32_t m = pending; m != 0u; m &= m - 1u) {
+                            const int group = first + (base + __builtin_ctz(m)) * stride;
+                            __syncthreads();
+                            load(group, kRouteGiveUp);
+                            __syncthreads();
+                            unit(group);
+                        }
+                        pending = 0u;
+                        break;
+                    }
+                    for (int r = 0; r < (1 << backoff); ++r) {
+                        __builtin_amdgcn_s_sleep(127);      // 127 x 64 clocks, about 3.5 us
+                    }
+                    backoff += backoff < 2 ? 1 : 0;
+                    continue;
+                }
+                for (uint32_t m = ready; m != 0u; m &= m - 1u) {
+                    const int i = __builtin_ctz(m);
+                    const int group = first + (base + i) * stride;
+                    __syncthreads();
+                    load(group, kRouteTrusted);
+                    __syncthreads();
+                    unit(group);
+                    pending &= ~(1u << i);
+                }
+                idleSince = wall_clock64();
+                backoff = 0;
+            }
+        }
     }
 }
 
@@ -196,7 +332,10 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 
     const int tg = threadIdx.x / G;
     const int lane = threadIdx.x % G;
-    constexpr int KB = V <= 2 ? 4 : (V <= 4 ? 2 : 1);      // rows in flight per lane
+    // Rows in flight per lane.  A whole workgroup per token is the geometry of launches that may wait on flags: at most two
+    // such workgroups run per compute unit, so a wave may use half a SIMD's registers and keeps four rows in flight
+    // whatever the row width; the other geometries run many more waves and trade rows in flight for occupancy.
+    constexpr int KB = G == kThreads ? 4 : (V <= 2 ? 4 : (V <= 4 ? 2 : 1));
     const int vecs = a.h / 8;
     // a unit is one token, or -- for wide rows -- one slice of G * V vectors of a token
     const int units = a.bs * a.colSlices;
@@ -204,14 +343,19 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
     const int unitsPerGroup = static_cast<int>(blockDim.x) / G;
     const int groups = (units + unitsPerGroup - 1) / unitsPerGroup;
 
-    for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+    auto tokenAt = [&](int group, int t) {
+        const int unit = group * unitsPerGroup + t;
+        return unit < units ? unit / a.colSlices : -1;
+    };
+    auto load = [&](int group, int mode) {
+        const int unit = group * unitsPerGroup + tg;
+        return LoadRoutes<false, false>(a, unit / a.colSlices, unit < units, lane, G, s_row[tg], s_w[tg], mode);
+    };
+    auto reduceUnit = [&](int group) {
         const int unit = group * unitsPerGroup + tg;
         const bool tokOk = unit < units;
         const int token = unit / a.colSlices;
         const int colBase = (unit % a.colSlices) * (G * V);
-        __syncthreads();        // the previous iteration's readers are done with s_row / s_w
-        LoadRoutes<false>(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
-        __syncthreads();
         if (KIND == kReducePerAdd) {
             if (lane == 0) {
                 SortRows(s_row[tg], a.slots, a.orderKeys);
@@ -321,7 +465,8 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                 }
             }
         }
-    }
+    };
+    ForEachGroup<FL>(a, groups, unitsPerGroup, tokenAt, load, reduceUnit);
 }
 
 // Quantised expert output: int8 rows with one fp32 scale per row, or fp8 e4m3 rows with one fp32 scale per 128
@@ -342,87 +487,115 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
     const int groups = (a.bs + kTokens - 1) / kTokens;
     const int b128 = (a.h + 127) / 128;
 
-    for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+    auto tokenAt = [&](int group, int t) {
+        const int token = group * kTokens + t;
+        return token < a.bs ? token : -1;
+    };
+    auto load = [&](int group, int mode) {
+        const int token = group * kTokens + tg;
+        return LoadRoutes<false, false>(a, token, token < a.bs, lane, G, s_row[tg], s_w[tg], mode);
+    };
+    auto reduceUnit = [&](int group) {
         const int token = group * kTokens + tg;
         const bool tokOk = token < a.bs;
-        __syncthreads();
-        LoadRoutes<false>(a, token, tokOk, lane, G, s_row[tg], s_w[tg]);
-        __syncthreads();
         const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !(FL && AnyExpired(s_row[tg], a.slots));
 
         float acc[V][16];
+        // The K loop.  fp8 rows are decoded by the hardware convert alone, which differs from the reference decode in
+        // one respect only (the sign of the NaN it returns for code 0x7f); a NaN code always surfaces as a NaN in the
+        // sum, so a wave that finds a NaN among its sums runs the loop once more with the exact decode.  That keeps a
+        // test of every word (four instructions and a branch per four values) out of the loop that everything else
+        // shares.
+        auto accumulate = [&](auto exactDecode) {
+            constexpr bool kExactDecode = decltype(exactDecode)::value;
 #pragma unroll
-        for (int j = 0; j < V; ++j) {
+            for (int j = 0; j < V; ++j) {
 #pragma unroll
-            for (int e = 0; e < 16; ++e) {
-                acc[j][e] = 0.0f;
-            }
-        }
-        for (int k0 = 0; k0 < a.slots; k0 += KB) {
-            u32x4 q[KB][V];
-            float sc[KB][V];
-            int rowOfK[KB];
-#pragma unroll
-            for (int u = 0; u < KB; ++u) {
-                const int k = k0 + u;
-                const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
-                rowOfK[u] = row;
-                // Bounds are the buffer resources' business: an absent row gets resources of zero bytes, so its loads, like
-                // those of the lanes past the end of a row, return zeros without a branch (and without the register
-                // clears a branch would need).
-                const int64_t rowAt = row < 0 ? 0 : row;
-                const char *base = static_cast<const char *>(a.expertOut) + rowAt * a.rowBytes;
-                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, row < 0 ? 0 : vecs * 16);
-                const bool perRow = INQ == TILEXR_EP_QUANT_TOKEN_INT8;
-                const float *scaleBase = a.inScales + (perRow ? rowAt : rowAt * b128);
-                const __amdgpu_buffer_rsrc_t scaleRsrc = RowResource(scaleBase, row < 0 ? 0 : (perRow ? 4 : b128 * 4));
-#pragma unroll
-                for (int j = 0; j < V; ++j) {
-                    const int idx = j * G + lane;
-                    q[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 16, 0, FL ? kAuxAgentScope : kAuxNonTemporal);
-                    sc[u][j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scaleRsrc, perRow ? 0 : (idx >> 3) * 4, 0,
-                        FL ? kAuxAgentScope : 0));
+                for (int e = 0; e < 16; ++e) {
+                    acc[j][e] = 0.0f;
                 }
             }
+            for (int k0 = 0; k0 < a.slots; k0 += KB) {
+                u32x4 q[KB][V];
+                float sc[KB][V];
+                int rowOfK[KB];
 #pragma unroll
-            for (int u = 0; u < KB; ++u) {
-                if (rowOfK[u] < 0) {
-                    continue;                       // uniform across the lanes of a token
+                for (int u = 0; u < KB; ++u) {
+                    const int k = k0 + u;
+                    const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
+                    rowOfK[u] = row;
+                    // Bounds are the buffer resources' business: an absent row gets resources of zero bytes, so its loads, like
+                    // those of the lanes past the end of a row, return zeros without a branch (and without the register
+                    // clears a branch would need).
+                    const int64_t rowAt = row < 0 ? 0 : row;
+                    const char *base = static_cast<const char *>(a.expertOut) + rowAt * a.rowBytes;
+                    const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, row < 0 ? 0 : vecs * 16);
+                    const bool perRow = INQ == TILEXR_EP_QUANT_TOKEN_INT8;
+                    const float *scaleBase = a.inScales + (perRow ? rowAt : rowAt * b128);
+                    const __amdgpu_buffer_rsrc_t scaleRsrc = RowResource(scaleBase, row < 0 ? 0 : (perRow ? 4 : b128 * 4));
+#pragma unroll
+                    for (int j = 0; j < V; ++j) {
+                        const int idx = j * G + lane;
+                        q[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 16, 0, FL ? kAuxAgentScope : kAuxNonTemporal);
+                        sc[u][j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(scaleRsrc, perRow ? 0 : (idx >> 3) * 4, 0,
+                            FL ? kAuxAgentScope : 0));
+                    }
                 }
-                const float w = s_w[tg][k0 + u];
 #pragma unroll
-                for (int j = 0; j < V; ++j) {
+                for (int u = 0; u < KB; ++u) {
+                    if (rowOfK[u] < 0) {
+                        continue;                       // uniform across the lanes of a token
+                    }
+                    const float w = s_w[tg][k0 + u];
 #pragma unroll
-                    for (int d = 0; d < 4; ++d) {
-                        const uint32_t word = q[u][j][d];
-                        float f[4];
-                        if (INQ == TILEXR_EP_QUANT_TOKEN_INT8) {
+                    for (int j = 0; j < V; ++j) {
 #pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                f[e] = static_cast<float>(static_cast<int>(static_cast<int8_t>((word >> (8 * e)) & 0xffu)));
-                            }
-                        } else {
-                            Fp8E4m3DecodeWord(word, f);
-                        }
+                        for (int d = 0; d < 4; ++d) {
+                            const uint32_t word = q[u][j][d];
+                            float f[4];
+                            if (INQ == TILEXR_EP_QUANT_TOKEN_INT8) {
 #pragma unroll
-                        for (int e = 0; e < 4; e += 2) {
-                            const float d0 = __fmul_rn(f[e], sc[u][j]);
-                            const float d1 = __fmul_rn(f[e + 1], sc[u][j]);
-                            float r0;
-                            float r1;
-                            if (BF16) {
-                                const uint32_t packed = FloatPairToBf16Rne(d0, d1);
-                                r0 = __uint_as_float(packed << 16);
-                                r1 = __uint_as_float(packed & 0xffff0000u);
+                                for (int e = 0; e < 4; ++e) {
+                                    f[e] = static_cast<float>(static_cast<int>(static_cast<int8_t>((word >> (8 * e)) & 0xffu)));
+                                }
+                            } else if (kExactDecode) {
+                                Fp8E4m3DecodeWord(word, f);
                             } else {
-                                r0 = __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d0))));
-                                r1 = __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d1))));
+                                Fp8E4m3DecodeWordFast(word, f);
                             }
-                            acc[j][4 * d + e] = __fadd_rn(acc[j][4 * d + e], __fmul_rn(r0, w));
-                            acc[j][4 * d + e + 1] = __fadd_rn(acc[j][4 * d + e + 1], __fmul_rn(r1, w));
+#pragma unroll
+                            for (int e = 0; e < 4; e += 2) {
+                                const float d0 = __fmul_rn(f[e], sc[u][j]);
+                                const float d1 = __fmul_rn(f[e + 1], sc[u][j]);
+                                float r0;
+                                float r1;
+                                if (BF16) {
+                                    r0 = FloatRoundedToBf16(d0);
+                                    r1 = FloatRoundedToBf16(d1);
+                                } else {
+                                    r0 = __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d0))));
+                                    r1 = __half2float(__ushort_as_half(static_cast<unsigned short>(FloatToHalfRneSat(d1))));
+                                }
+                                acc[j][4 * d + e] = __fadd_rn(acc[j][4 * d + e], __fmul_rn(r0, w));
+                                acc[j][4 * d + e + 1] = __fadd_rn(acc[j][4 * d + e + 1], __fmul_rn(r1, w));
+                            }
                         }
                     }
                 }
+            }
+        };
+        accumulate(std::false_type {});
+        if (INQ == TILEXR_EP_QUANT_FP8_BLOCK128) {
+            bool sawNan = false;
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    sawNan |= acc[j][e] != acc[j][e];
+                }
+            }
+            if (__any(sawNan ? 1 : 0)) {
+                accumulate(std::true_type {});
             }
         }
         if (a.sharedExpertX != nullptr && active) {
@@ -464,7 +637,8 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_quant_kernel(ReduceArgs a)
                 }
             }
         }
-    }
+    };
+    ForEachGroup<FL>(a, groups, kTokens, tokenAt, load, reduceUnit);
 }
 
 // Element-granular reduce for any h / alignment.  One workgroup per token; a thread owns whole 32-column blocks so
@@ -478,7 +652,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
     const int b128 = (a.h + 127) / 128;
     for (int token = blockIdx.x; token < a.bs; token += gridDim.x) {
         __syncthreads();
-        LoadRoutes<true>(a, token, true, tid, kThreads, s_row, s_w);
+        LoadRoutes<true, true>(a, token, true, tid, kThreads, s_row, s_w, kRouteCheck);
         __syncthreads();
         if (kind == kReducePerAdd) {
             if (tid == 0) {
@@ -659,6 +833,7 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     a.h = static_cast<int>(l.h);
     a.topK = static_cast<int>(l.topK);
     a.slots = static_cast<int>(l.topK + l.sharedSlots);
+    a.maxRows = l.maxRows > 0 ? static_cast<int>(l.maxRows) : 0x7fffffff;
     a.y = l.y;
     a.tileFlags = l.tileFlags;
     a.tileRows = static_cast<int>(l.tileRows);

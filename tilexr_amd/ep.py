@@ -23,7 +23,7 @@ EXPORTS = (
     "TileXRMoeEpDispatch", "TileXRMoeEpDispatchV2", "TileXRMoeEpDispatchMemory", "TileXRMoeEpDispatchMemoryV2",
     "TileXRMoeEpCombine", "TileXRMoeEpCombineV2", "TileXRMoeEpCombineMemory", "TileXRMoeEpCombineMemoryV2",
     "TileXRMoeEpDispatchMemoryEx", "TileXRMoeEpCombineMemoryEx", "TileXRMoeEpDispatchMemoryNoAlloc", "TileXREpVersion", "TileXREpSetKernelTimingEvents",
-    "TileXREpLastKernelName", "TileXREpMemoryProbe",
+    "TileXREpLastKernelName", "TileXREpMemoryProbe", "TileXREpTileProducerProbe",
     "TileXRCommInitRankLocal", "TileXRCommDestroy", "TileXRGetCommArgsHost", "TileXRGetCommArgsDev",
     "TileXRCommNextMagic",
 )
@@ -294,6 +294,16 @@ def memory_probe(pattern, src, dst, nbytes, stream):
     fn = lib().TileXREpMemoryProbe
     fn.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     return fn(pattern, _ptr(src), _ptr(dst), int(nbytes), _stream(stream))
+
+
+def tile_producer_probe(src, dst, rows, row_bytes, tile_flags, tile_rows, epoch, workgroups, min_tile_ns, stream):
+    """A stand-in for an expert stage: copies rows src -> dst tile by tile at a set pace and publishes each tile's
+    readiness word (see tilexr_ep.h)."""
+    fn = lib().TileXREpTileProducerProbe
+    fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
+                   C.c_void_p]
+    return fn(_ptr(src), _ptr(dst), int(rows), int(row_bytes), _ptr(tile_flags), int(tile_rows), int(epoch),
+              int(workgroups), int(min_tile_ns), _stream(stream))
 
 
 def last_kernel_name(comm, kernel):
