@@ -82,6 +82,9 @@ def parse():
     p.add_argument("--no-overlap-leg", action="store_true",
                    help="skip the extra, separately timed runs of the schedules that are not the timed one (reported "
                         "under config.other_schedules)")
+    p.add_argument("--no-graph-leg", action="store_true",
+                   help="decode-sized workloads: skip the extra leg that replays a captured HIP graph of 16 layers "
+                        "(reported under config.graph_replay)")
     p.add_argument("--no-stage-leg", action="store_true",
                    help="skip the extra leg with a slow expert-stage stand-in between dispatch and combine (reported under "
                         "config.expert_stage)")
@@ -508,6 +511,11 @@ def main():
     steps_by_schedule = {"flags-serial": step_flags_serial, "flags-overlapped": step_overlapped, "plain": step_plain}
     schedule = "flags-overlapped" if args.overlap else args.schedule
     calibration = None
+    # decode-sized calls (at most 2048 routes) take the library's single-launch dispatch, which publishes no flags: two
+    # launches per layer instead of four is what counts there
+    small = bs * K <= 2048
+    if schedule == "auto" and small:
+        schedule = "plain"
     if schedule == "auto":
         # the faster of the two schedules that publish and consume flags, by a short calibration outside the timed region
         torch.cuda.synchronize()
@@ -580,21 +588,25 @@ def main():
         del ref, kept_w
 
     # split of one step into its two calls, run back to back on one stream (outside the timed region), with the timed
-    # schedule's flag settings
-    d_ev[0].record(stream)
-    st, epoch = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts, ep.DT_BF16,
-                                      stream, quant_mode=quant, expert_capacity=w.capacity, dynamic_scales=scales,
-                                      row_index_map=row_map, tile_flags=flags if uses_flags else None,
-                                      tile_rows=args.tile_rows if uses_flags else 0)
-    d_ev[1].record(stream)
-    ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
-                         expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w, row_index_map=row_map,
-                         tile_flags=flags if uses_flags else None, tile_rows=args.tile_rows if uses_flags else 0,
-                         flag_epoch=epoch, device_status=status if uses_flags else None)
-    d_ev[2].record(stream)
+    # schedule's flag settings: median of 20 event-bracketed layers (a single layer after an idle queue reads high)
+    splits = []
+    for _ in range(20):
+        d_ev = [ep.HipEvent(timing=True) for _ in range(3)]
+        d_ev[0].record(stream)
+        st, epoch = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts, ep.DT_BF16,
+                                          stream, quant_mode=quant, expert_capacity=w.capacity, dynamic_scales=scales,
+                                          row_index_map=row_map, tile_flags=flags if uses_flags else None,
+                                          tile_rows=args.tile_rows if uses_flags else 0)
+        d_ev[1].record(stream)
+        ep.combine_memory_ex(expand_x, assist, send_counts, comm, bs, h, K, E, y, ep.DT_BF16, stream,
+                             expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w, row_index_map=row_map,
+                             tile_flags=flags if uses_flags else None, tile_rows=args.tile_rows if uses_flags else 0,
+                             flag_epoch=epoch, device_status=status if uses_flags else None)
+        d_ev[2].record(stream)
+        splits.append(d_ev)
     torch.cuda.synchronize()
-    dispatch_us = d_ev[0].elapsed_ms(d_ev[1]) * 1e3
-    combine_us = d_ev[1].elapsed_ms(d_ev[2]) * 1e3
+    dispatch_us = sorted(e[0].elapsed_ms(e[1]) * 1e3 for e in splits)[len(splits) // 2]
+    combine_us = sorted(e[1].elapsed_ms(e[2]) * 1e3 for e in splits)[len(splits) // 2]
 
     # the schedules that were not timed, each on its own after the main region so that all three are on record; they
     # are not part of `value`
@@ -619,6 +631,35 @@ def main():
             other.append({"schedule": SCHEDULES[name], "tile_rows": args.tile_rows if name != "plain" else None,
                           "steps": other_steps, "us_per_layer": round(other_us, 2),
                           "GBps": round((dispatch_bytes + combine_bytes) / (other_us * 1e-6) / 1e9, 1)})
+
+    # decode-sized workloads: 16 layers captured once in a HIP graph and replayed, against the same layers launched one
+    # call at a time.  Not part of `value`.
+    graph_replay = None
+    if small and not args.no_graph_leg:
+        layers = 16
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for _ in range(layers):
+                step_plain()
+        torch.cuda.synchronize()
+        for _ in range(5):
+            graph.replay()
+        torch.cuda.synchronize()
+        replays = max(10, args.steps // 4)
+        t1 = time.perf_counter()
+        for _ in range(replays):
+            graph.replay()
+        torch.cuda.synchronize()
+        replay_us = (time.perf_counter() - t1) / replays / layers * 1e6
+        t1 = time.perf_counter()
+        for _ in range(replays * layers):
+            step_plain()
+        torch.cuda.synchronize()
+        eager_us = (time.perf_counter() - t1) / (replays * layers) * 1e6
+        graph_replay = {"layers_per_graph": layers, "replays": replays, "us_per_layer": round(replay_us, 2),
+                        "eager_us_per_layer": round(eager_us, 2)}
+        del graph
 
     # What the flags are for: an expert stage between dispatch and combine that is slower than memory and publishes
     # tiles as it finishes them.  A stand-in producer of the library (a few workgroups copy expandX to expertOut tile by
@@ -781,7 +822,7 @@ def main():
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
         "config": dict(workloads.describe(w, ids), schedule=SCHEDULES[schedule],
                        tile_rows=args.tile_rows if uses_flags else None, schedule_calibration_us=calibration,
-                       other_schedules=other, expert_stage=expert_stage, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
+                       other_schedules=other, expert_stage=expert_stage, graph_replay=graph_replay, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),
         "roofline": roofline, "kernels": kernels, "ceilings": ceilings,
     }

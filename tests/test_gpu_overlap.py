@@ -277,3 +277,101 @@ def test_combine_beside_a_slow_producer_that_publishes_tiles_as_it_goes(shape, t
         assert ep.tile_producer_probe(expert_out, expert_out, 0, 64, flags, 8, 1, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
         assert ep.tile_producer_probe(expert_out, expert_out, 8, 24, flags, 8, 1, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
         assert ep.tile_producer_probe(expert_out, expert_out, 8, 64, flags, 8, 0, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
+
+
+def test_flag_protocol_on_randomised_rounds():
+    """A bounded randomised run of the whole flag protocol on buffers that are reused from round to round: random shapes,
+    tile sizes, payload formats and schedules (combine after dispatch on one stream, beside it on a second stream, or
+    beside an expert-stage stand-in that rewrites the rows).  Every round is compared bit for bit with the CPU oracle
+    and must report no expired wait; the run ends at the first round that fails, after 48 rounds or after 60 seconds,
+    whichever comes first.  Seeded: the same rounds every time."""
+    import time
+    rng = np.random.default_rng(20240607)
+    max_rows, max_h = 4096 * 8, 7168
+    with Session() as s:
+        side = torch.cuda.Stream()
+        pool_rows = torch.empty((max_rows * max_h * 2,), dtype=torch.uint8, device=DEV)
+        pool_stage = torch.empty((max_rows * max_h * 2,), dtype=torch.uint8, device=DEV)
+        pool_scales = torch.empty((max_rows * (max_h // 128),), dtype=torch.float32, device=DEV)
+        pool_y = torch.empty((4096 * max_h,), dtype=torch.bfloat16, device=DEV)
+        flags = torch.zeros((max_rows,), dtype=torch.int64, device=DEV)          # one array for every tile size
+        stage_flags = torch.zeros((max_rows,), dtype=torch.int64, device=DEV)
+        status = torch.zeros((1,), dtype=torch.int32, device=DEV)
+        meta_ready, consumed = ep.HipEvent(), ep.HipEvent()
+        started = time.monotonic()
+        rounds = 0
+        for round_ in range(48):
+            if time.monotonic() - started > 60.0:
+                break
+            bs = int(rng.choice([64, 200, 777, 1024, 2048, 4096]))
+            h = int(rng.choice([256, 1024, 2048, 4096, 7168]))
+            K = int(rng.choice([2, 4, 8]))
+            E = int(rng.choice([16, 64, 256]))
+            tile_rows = int(rng.choice([1, 8, 16, 64, 100, 1024]))
+            quant = str(rng.choice(["none", "none", "int8", "fp8_block128"]))
+            schedule = str(rng.choice(["one_stream", "two_streams", "expert_stage"]))
+            if quant != "none" and schedule == "expert_stage":
+                schedule = "two_streams"
+            qmode = {"none": ep.Q_NONE, "int8": ep.Q_TOKEN_INT8, "fp8_block128": ep.Q_FP8_BLOCK128}[quant]
+            oq = {"none": O.Q_NONE, "int8": O.Q_TOKEN_INT8, "fp8_block128": O.Q_FP8_BLOCK128}[quant]
+            n = bs * K
+            row_bytes = h * 2 if qmode == ep.Q_NONE else h
+            ids, w = routing(rng, bs, K, E)
+            x = torch.from_numpy((rng.standard_normal((bs, h)) * (1 + round_ % 5)).astype(np.float32)).to(torch.bfloat16)
+            xb = bits16(x)
+            d_x, d_ids, d_w = x.to(DEV), to_dev(ids), to_dev(w)
+            expand_x = pool_rows[:n * row_bytes].view(n, row_bytes)
+            expert_out = pool_stage[:n * row_bytes].view(n, row_bytes)
+            scales = None
+            if qmode == ep.Q_TOKEN_INT8:
+                scales = pool_scales[:n].view(n, 1)
+            elif qmode == ep.Q_FP8_BLOCK128:
+                scales = pool_scales[:n * ((h + 127) // 128)].view(n, (h + 127) // 128)
+            y = pool_y[:bs * h].view(bs, h)
+            assist = torch.empty((n, 4), dtype=torch.int32, device=DEV)
+            token_nums = torch.empty((E,), dtype=torch.int64, device=DEV)
+            counts = torch.empty((E,), dtype=torch.int32, device=DEV)
+            row_map = torch.empty((bs, K), dtype=torch.int32, device=DEV)
+            torch.cuda.synchronize()
+            print(f"flag rounds: {round_} bs={bs} h={h} K={K} E={E} tile_rows={tile_rows} {quant} {schedule}", flush=True)
+            two = schedule == "two_streams"
+            st, epoch = ep.dispatch_memory_ex(d_x, d_ids, s.comm, bs, h, K, E, expand_x, assist, token_nums, counts,
+                                              ep.DT_BF16, s.stream, quant_mode=qmode, dynamic_scales=scales,
+                                              row_index_map=row_map, tile_flags=flags, tile_rows=tile_rows,
+                                              meta_ready_event=meta_ready.value if two else None)
+            assert st == 0
+            rows_in, use_flags, use_epoch, consumer = expand_x, flags, epoch, s.stream
+            if two:
+                meta_ready.wait_on(side)
+                consumer = side
+            elif schedule == "expert_stage":
+                # the stand-in follows the dispatch on its stream and republishes the rows under an epoch of its own;
+                # combine runs beside it on the second stream (the row map is complete: dispatch was enqueued first and
+                # the stand-in's stream order puts every flag of it after the dispatch)
+                s.sync()
+                assert ep.tile_producer_probe(expand_x, expert_out, n, row_bytes, stage_flags, tile_rows, 1000 + round_,
+                                              int(rng.choice([8, 64, 200])), int(rng.choice([0, 3000])), s.stream) == 0
+                rows_in, use_flags, use_epoch, consumer = expert_out, stage_flags, 1000 + round_, side
+            st = ep.combine_memory_ex(rows_in, assist, counts, s.comm, bs, h, K, E, y, ep.DT_BF16, consumer,
+                                      expert_out_quant_mode=qmode, expert_out_scales=scales, expert_scales=d_w,
+                                      row_index_map=row_map, tile_flags=use_flags, tile_rows=tile_rows,
+                                      flag_epoch=use_epoch, wait_timeout_us=5_000_000, device_status=status)
+            assert st == 0
+            if consumer is side:
+                consumed.record(side)
+                consumed.wait_on(s.stream)
+            s.sync()
+            side.synchronize()
+            assert status.item() == 0, f"round {round_}: a flag wait expired"
+            case = O.Case(1, bs, h, K, E, dtype=O.DT_BF16, quant_mode=oq, token_nums_type=1)
+            want = O.mem_dispatch(case, 0, xb[None], ids[None])
+            assert np.array_equal(expand_x.cpu().numpy(), want["expand_x"]), f"round {round_}: rows"
+            eo = want["expand_x"][None] if oq else want["expand_x"].view(np.uint16)[None]
+            wy = O.mem_combine(O.Case(1, bs, h, K, E, dtype=O.DT_BF16), 0, eo, want["assist"][None],
+                               want["send_counts"][None], expert_scales=w, in_quant=oq,
+                               in_scales=want["dyn_scales"] if oq else None)
+            assert np.array_equal(bits16(y), wy), f"round {round_}: y"
+            rounds += 1
+        assert rounds >= 8
+        meta_ready.destroy()
+        consumed.destroy()
