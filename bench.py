@@ -108,7 +108,7 @@ def parse():
     return p.parse_args()
 
 
-def measured_ceilings(ep, torch, stream, dev, reps=10):
+def measured_ceilings(ep, torch, stream, dev, reps=10, narrow=None):
     """What this device's memory system delivers for plain access patterns, measured in this run with the library's
     own probe kernels (HIP events around `reps` launches each): pure read, pure write, copy, and the read : write
     mixes of the scatter (1 : 8) and the reduce (8 : 1).  GB/s of all bytes moved, reads plus writes.  The mixed
@@ -143,6 +143,25 @@ def measured_ceilings(ep, torch, stream, dev, reps=10):
             us = a.elapsed_ms(b) * 1e3 / reps
             rate = round(moved[name] / (us * 1e-6) / 1e9, 1)
             out[name + "_GBps"] = max(rate, out.get(name + "_GBps", 0.0))
+        del src, dst
+    if narrow is not None:
+        # the quantised reduce's mix with its addresses: rows of 2048 (4096) one-byte payloads, eight (six) per output
+        # row of twice the width, at unrelated positions; the source sized like the workload's rows
+        name, pattern, row_bytes, k = narrow
+        # as many rows as the probe's row arithmetic allows (fewer than 2^17), so that the source exceeds the memory-side cache
+        nbytes = min(600 << 20, ((1 << 17) - 1) * row_bytes) // (row_bytes * k) * (row_bytes * k)
+        src = torch.zeros((nbytes,), dtype=torch.uint8, device=dev)
+        dst = torch.zeros((nbytes * 2 // k,), dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+        for _ in range(3):
+            ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+        a, b = ep.HipEvent(timing=True), ep.HipEvent(timing=True)
+        a.record(stream)
+        for _ in range(reps):
+            ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+        b.record(stream)
+        stream.synchronize()
+        out[name + "_GBps"] = round((nbytes + nbytes * 2 // k) / (a.elapsed_ms(b) * 1e-3 / reps) / 1e9, 1)
         del src, dst
     return out
 
@@ -807,12 +826,15 @@ def main():
 
     ceilings = None
     if not args.no_ceilings:
-        ceilings = measured_ceilings(ep, torch, stream, dev)
+        narrow = {("int8", 4096, 6): ("gather_rows_4k_6r_GBps"[:-5], ep.PROBE_GATHER_ROWS_4K_X6, 4096, 6),
+                  ("fp8_block128", 2048, 8): ("gather_rows_2k_8r_GBps"[:-5], ep.PROBE_GATHER_ROWS_2K_X8, 2048, 8)}.get((w.quant, h, K))
+        ceilings = measured_ceilings(ep, torch, stream, dev, narrow=narrow)
         if roofline is not None:
             mix = ceilings["fan_out_1r8w_GBps"] if dom == "scatter" else ceilings["fan_in_8r1w_GBps"]
             roofline["frac_of_measured_mix"] = round(roofline["achieved"] / mix, 4)
             if dom == "reduce":
-                roofline["frac_of_measured_row_gather"] = round(roofline["achieved"] / ceilings["gather_rows_8r1w_GBps"], 4)
+                gather = ceilings[narrow[0] + "_GBps"] if narrow is not None else ceilings["gather_rows_8r1w_GBps"]
+                roofline["frac_of_measured_row_gather"] = round(roofline["achieved"] / gather, 4)
 
     result = {
         "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",

@@ -211,6 +211,25 @@ int TileXRMoeEpDispatchMemoryNoAlloc(void *x, int32_t *expertIds, TileXRCommPtr 
 // Ids 2 and 4 also cover the scatter and reduce kernels of the plan-driven stages (tilexr_moonep.h).
 int TileXREpSetKernelTimingEvents(TileXRCommPtr comm, int kernel, void *startEvent, void *stopEvent);
 
+// Debug aids without a reference counterpart as an API (the reference's kernels leave breadcrumbs of the same kind:
+// RunPosRecord, src/ep/kernels/tilexr_ep_dispatch_memory_kernel.h:1319-1328).  Stamps cover every kernel a call on
+// `comm` launches; the poison fill applies to the dispatches of a one-rank communicator.  Null options switch both off.
+struct TileXREpDebugOptions {
+    uint64_t *phaseStamps;        // optional device ring of phaseStampCapacity records of four uint64 each:
+                                  //   {magic of the call, kernel id (as TileXREpSetKernelTimingEvents), edge: 0 written
+                                  //   by a one-thread kernel enqueued ahead of that kernel / 1 behind it, device clock
+                                  //   (100 MHz ticks)}.  Records are written in call order, record i at index
+                                  //   i % phaseStampCapacity; after a wait that expired, or a run that never came back,
+                                  //   the ring says which phase was reached and how long each took on the device
+    int64_t phaseStampCapacity;   // > 0 exactly when phaseStamps is set, at most 2^24
+    int64_t poisonUnwrittenRows;  // non-zero: a dispatch first fills every row it may write (bs * topK of them, or
+                                  //   moeExpertNum * expertCapacity when that is less), their assist tuples and their
+                                  //   scales with 0x7f bytes (bf16 3.4e38, int8 127, the e4m3 NaN code, int32
+                                  //   2139062143), so that a row which was counted but never written cannot pass for
+                                  //   data.  Costs a full pass over the output buffers
+};
+int TileXREpSetDebugOptions(TileXRCommPtr comm, const TileXREpDebugOptions *options);
+
 // Measurement aid without a reference counterpart: name of the kernel template the last call on `comm` launched
 // for a kernel id (the data kernels have several templates, chosen by row width, alignment and payload type), so
 // that a harness can match its event timings with a profiler's per-kernel rows.  Null before the first launch.
@@ -230,6 +249,10 @@ const char *TileXREpVersion(void);
 //   FAN_IN   reads `bytes` of src as eight regions, writes bytes / 8 of dst  (the reduce's 8 : 1 mix)
 //   GATHER_ROWS  the same mix with the reduce's addresses: src is rows of 14336 bytes, every output row combines
 //            eight source rows at unrelated positions; `bytes` a multiple of 8 * 14336; writes bytes / 8 of dst
+//   GATHER_ROWS_2K_X8 / GATHER_ROWS_4K_X6  the quantised reduce's mix and addresses: src is rows of 2048 (4096) one-byte
+//            payloads, every output row of twice that many bytes combines eight (six) source rows at unrelated
+//            positions; `bytes` a multiple of 8 * 2048 (6 * 4096), fewer than 2^17 rows; writes bytes / 4 (bytes / 3)
+//            of dst
 // Asynchronous on `stream`; returns 0, -3 for bad arguments, -2 when the launch fails.
 enum TileXREpProbePattern {
     TILEXR_EP_PROBE_READ = 0,
@@ -237,7 +260,9 @@ enum TileXREpProbePattern {
     TILEXR_EP_PROBE_COPY = 2,
     TILEXR_EP_PROBE_FAN_OUT = 3,
     TILEXR_EP_PROBE_FAN_IN = 4,
-    TILEXR_EP_PROBE_GATHER_ROWS = 5
+    TILEXR_EP_PROBE_GATHER_ROWS = 5,
+    TILEXR_EP_PROBE_GATHER_ROWS_2K_X8 = 6,
+    TILEXR_EP_PROBE_GATHER_ROWS_4K_X6 = 7
 };
 int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int64_t bytes, aclrtStream stream);
 

@@ -164,7 +164,8 @@ def test_memory_probe_patterns_move_what_they_say():
     assert torch.equal(dst[:n].view(-1, 4), torch.tensor([1, 2, 3, 4], dtype=torch.int32, device=dev).expand(n // 4, 4))
     assert bool((dst[n:] == -1).all())
     # argument rules
-    assert ep.memory_probe(7, src, dst, nbytes, stream) == -3
+    assert ep.memory_probe(8, src, dst, nbytes, stream) == -3
+    assert ep.memory_probe(-1, src, dst, nbytes, stream) == -3
     assert ep.memory_probe(ep.PROBE_COPY, src, dst, nbytes + 4, stream) == -3
     assert ep.memory_probe(ep.PROBE_COPY, None, dst, nbytes, stream) == -3
 
@@ -192,3 +193,33 @@ def test_memory_probe_row_gather_reads_rows_whole():
         assert torch.equal(dst[t], want), f"row {t}"
     assert bool((dst[rows // 8] == -1).all())
     assert ep.memory_probe(ep.PROBE_GATHER_ROWS, src, dst, rows * 14336 + 128, stream) == -3
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("pattern,row_bytes,k", [("PROBE_GATHER_ROWS_2K_X8", 2048, 8), ("PROBE_GATHER_ROWS_4K_X6", 4096, 6)])
+def test_memory_probe_narrow_row_gathers(pattern, row_bytes, k):
+    """The yardsticks of the quantised reduce: every output row, twice as wide as a source row, interleaves 16-byte
+    pieces of the xor of k source rows with pieces of the same xor without its last row."""
+    import torch
+    from tilexr_amd import ep
+
+    dev = "cuda:0"
+    groups = 11
+    rows, row_ints = groups * k, row_bytes // 4
+    stream = torch.cuda.Stream()
+    g = torch.Generator().manual_seed(6)
+    src = torch.randint(-2**31, 2**31 - 1, (rows, row_ints), generator=g, dtype=torch.int64).to(torch.int32).to(dev)
+    dst = torch.full((groups + 1, 2 * row_ints), -1, dtype=torch.int32, device=dev)
+    torch.cuda.synchronize()
+    assert ep.memory_probe(getattr(ep, pattern), src, dst, rows * row_bytes, stream) == 0
+    stream.synchronize()
+    strides = [1, 7919, 10007, 12289, 15013, 17389, 20011, 22291]
+    for t in range(groups):
+        picked = [src[(t * strides[j] + j * 977) % rows] for j in range(k)]
+        all_k = picked[0].clone()
+        for r in picked[1:]:
+            all_k ^= r
+        want = torch.stack([all_k.view(-1, 4), (all_k ^ picked[-1]).view(-1, 4)], dim=1).reshape(-1)
+        assert torch.equal(dst[t], want), f"row {t}"
+    assert bool((dst[groups] == -1).all())
+    assert ep.memory_probe(getattr(ep, pattern), src, dst, rows * row_bytes + row_bytes, stream) == -3

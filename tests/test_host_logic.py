@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for header in ("tilexr_ep.h", "tilexr_api.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         declared |= set(re.findall(r"^(?:int|const char \*)\s*\*?(TileXR\w+)\(", text, flags=re.M))
-    assert len(declared) == 21, sorted(declared)
+    assert len(declared) == 22, sorted(declared)
     assert declared == set(ep.EXPORTS)
     for name in declared:
         assert getattr(lib, name) is not None

@@ -41,6 +41,25 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     const bool expertHist = !memoryRoute;
 
     std::lock_guard<std::mutex> lock(comm->mu);
+    comm->debug.magic = magic;
+    if (comm->debug.poison) {
+        // every row this dispatch may write, its tuple and its scales: a row that is counted but never written shows
+        const int64_t rows = p.expertCapacity > 0 ? std::min<int64_t>(n, experts * p.expertCapacity) : n;
+        const int64_t rowBytes = p.quantMode == TILEXR_EP_QUANT_NONE ? p.h * 2 : p.h;
+        int64_t scaleBytes = 0;
+        if (p.quantMode == TILEXR_EP_QUANT_TOKEN_INT8) {
+            scaleBytes = 4;
+        } else if (p.quantMode == TILEXR_EP_QUANT_MXFP8) {
+            scaleBytes = ((p.h + 31) / 32 + 1) / 2 * 2;
+        } else if (p.quantMode == TILEXR_EP_QUANT_FP8_BLOCK128) {
+            scaleBytes = (p.h + 127) / 128 * 4;
+        }
+        if (LaunchDebugPoison(p.expandXOut, rows * rowBytes, stream) != hipSuccess ||
+            LaunchDebugPoison(p.assistInfoForCombineOut, rows * 16, stream) != hipSuccess ||
+            LaunchDebugPoison(p.dynamicScalesOut, rows * scaleBytes, stream) != hipSuccess) {
+            return TileXR::TILEXR_ERROR_MKIRT;
+        }
+    }
     if (memoryRoute && p.quantMode == TILEXR_EP_QUANT_NONE && p.xActiveMask == nullptr && p.tileFlagsOut == nullptr &&
         p.metaReadyEvent == nullptr) {
         // decode-sized calls: one launch instead of count + scatter
@@ -206,6 +225,7 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     hipStream_t stream = static_cast<hipStream_t>(p.stream);
     const int64_t n = p.bs * p.topK;
     std::lock_guard<std::mutex> lock(comm->mu);
+    comm->debug.magic = magic;
 
     const uint64_t epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
     uint64_t *inverse = nullptr;
@@ -470,6 +490,26 @@ int TileXREpSetKernelTimingEvents(TileXRCommPtr comm, int kernel, void *startEve
     std::lock_guard<std::mutex> lock(c->mu);
     c->timing[kernel][0] = static_cast<hipEvent_t>(startEvent);
     c->timing[kernel][1] = static_cast<hipEvent_t>(stopEvent);
+    return TileXR::TILEXR_SUCCESS;
+}
+
+int TileXREpSetDebugOptions(TileXRCommPtr comm, const TileXREpDebugOptions *options)
+{
+    EpComm *c = LookupComm(comm);
+    if (c == nullptr) {
+        return TileXR::TILEXR_ERROR_NOT_INITIALIZED;
+    }
+    if (options != nullptr && ((options->phaseStamps != nullptr) != (options->phaseStampCapacity > 0) ||
+                               options->phaseStampCapacity < 0 || options->phaseStampCapacity > (int64_t{1} << 24))) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    std::lock_guard<std::mutex> lock(c->mu);
+    c->debug = DebugState {};
+    if (options != nullptr) {
+        c->debug.phaseStamps = options->phaseStamps;
+        c->debug.capacity = options->phaseStampCapacity;
+        c->debug.poison = options->poisonUnwrittenRows != 0;
+    }
     return TileXR::TILEXR_SUCCESS;
 }
 

@@ -20,6 +20,7 @@
 #include <hip/hip_runtime_api.h>
 
 #include "comm_args.h"
+#include "ep_debug.h"
 #include "ep_host.h"
 
 namespace TileXRMoon {
@@ -121,6 +122,7 @@ struct EpComm {
     const void *lastFlagWords = nullptr;
     uint64_t lastFlagEpoch = 0;
     hipStream_t lastFlagStream = nullptr;
+    DebugState debug;                 // TileXREpSetDebugOptions
     hipEvent_t timing[5][2] = {};     // optional (start, stop) pairs around each kernel, see tilexr_ep.h
     const char *lastKernel[5] = {};   // name of the kernel template last launched for each kernel id
     std::mutex mu;

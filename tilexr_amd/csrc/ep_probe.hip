@@ -127,6 +127,33 @@ __global__ __launch_bounds__(kWave) void ep_probe_gather_rows_kernel(const u32x4
     __builtin_nontemporal_store(acc, dst + static_cast<int64_t>(t) * kProbeRowVecs + at);
 }
 
+// The quantised reduce's mix with its addresses: src is rows of ROW_BYTES one-byte payloads, output row t (two bytes per
+// column) is combined from K rows at unrelated positions.  One wave per 1 KiB slice of the input rows: K 16-byte loads
+// and two 16-byte stores per lane.
+template <int ROW_BYTES, int K>
+__global__ __launch_bounds__(kWave) void ep_probe_gather_narrow_kernel(const u32x4 *src, u32x4 *dst, int64_t rows)
+{
+    constexpr int kRowVecs = ROW_BYTES / 16;
+    constexpr int kSlices = kRowVecs / kWave;
+    const uint32_t t = blockIdx.x / kSlices;
+    const int at = (blockIdx.x % kSlices) * kWave + threadIdx.x;
+    const uint32_t strides[8] = {1u, 7919u, 10007u, 12289u, 15013u, 17389u, 20011u, 22291u};
+    u32x4 v[K];
+#pragma unroll
+    for (int k = 0; k < K; ++k) {
+        const uint32_t row = (t * strides[k] + static_cast<uint32_t>(k) * 977u) % static_cast<uint32_t>(rows);
+        v[k] = __builtin_nontemporal_load(src + static_cast<int64_t>(row) * kRowVecs + at);
+    }
+    u32x4 acc = v[0];
+#pragma unroll
+    for (int k = 1; k < K; ++k) {
+        acc ^= v[k];
+    }
+    u32x4 *out = dst + (static_cast<int64_t>(t) * kRowVecs + at) * 2;
+    __builtin_nontemporal_store(acc, out);
+    __builtin_nontemporal_store(acc ^ v[K - 1], out + 1);
+}
+
 // Tiles t = blockIdx.x, blockIdx.x + gridDim.x, ... in turn.  Ordinary loads and stores (the rows may sit dirty in this
 // XCD's L2), then per tile: every wave waits for its stores, the barrier collects the waves, one lane writes the L2 back
 // with a release fence at agent scope and stores the word.  One such fence per tile of tens of rows is cheap; one per row
@@ -200,7 +227,13 @@ extern "C" int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int6
     if (pattern == TILEXR_EP_PROBE_GATHER_ROWS && (bytes % (8 * kProbeRowBytes) != 0 || bytes / kProbeRowBytes >= (1 << 17))) {
         return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
     }
-    if (pattern < TILEXR_EP_PROBE_READ || pattern > TILEXR_EP_PROBE_GATHER_ROWS || bytes < 128 || bytes % 128 != 0 ||
+    if (pattern == TILEXR_EP_PROBE_GATHER_ROWS_2K_X8 && (bytes % (8 * 2048) != 0 || bytes / 2048 >= (1 << 17))) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    if (pattern == TILEXR_EP_PROBE_GATHER_ROWS_4K_X6 && (bytes % (6 * 4096) != 0 || bytes / 4096 >= (1 << 17))) {
+        return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
+    }
+    if (pattern < TILEXR_EP_PROBE_READ || pattern > TILEXR_EP_PROBE_GATHER_ROWS_4K_X6 || bytes < 128 || bytes % 128 != 0 ||
         bytes > (int64_t{1} << 40) || (needSrc && (src == nullptr || !Aligned16(src))) ||
         (needDst && (dst == nullptr || !Aligned16(dst)))) {
         return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
@@ -227,6 +260,16 @@ extern "C" int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int6
         case TILEXR_EP_PROBE_FAN_IN:
             hipLaunchKernelGGL(ep_probe_fan_in_kernel, blocks(vecs / 8, kWave), dim3(kWave), 0, s, in, out, vecs / 8);
             break;
+        case TILEXR_EP_PROBE_GATHER_ROWS_2K_X8: {
+            const int64_t rows = bytes / 2048;
+            hipLaunchKernelGGL((ep_probe_gather_narrow_kernel<2048, 8>), blocks(vecs / 8, kWave), dim3(kWave), 0, s, in, out, rows);
+            break;
+        }
+        case TILEXR_EP_PROBE_GATHER_ROWS_4K_X6: {
+            const int64_t rows = bytes / 4096;
+            hipLaunchKernelGGL((ep_probe_gather_narrow_kernel<4096, 6>), blocks(vecs / 6, kWave), dim3(kWave), 0, s, in, out, rows);
+            break;
+        }
         default: {
             const int64_t rows = bytes / kProbeRowBytes;
             hipLaunchKernelGGL(ep_probe_gather_rows_kernel, blocks(vecs / 8, kWave), dim3(kWave), 0, s, in, out, rows);

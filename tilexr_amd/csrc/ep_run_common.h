@@ -29,12 +29,26 @@ int Timed(EpComm *comm, int kernel, hipStream_t stream, const char *what, Launch
 {
     hipEvent_t start = comm->timing[kernel][0];
     hipEvent_t stop = comm->timing[kernel][1];
+    DebugState &dbg = comm->debug;
+    auto stamp = [&](int edge) {
+        if (dbg.phaseStamps == nullptr || dbg.capacity <= 0) {
+            return true;
+        }
+        uint64_t *record = dbg.phaseStamps + (dbg.next++ % dbg.capacity) * kDebugStampWords;
+        return LaunchDebugStamp(record, static_cast<uint64_t>(dbg.magic), kernel, edge, stream) == hipSuccess;
+    };
+    if (!stamp(0)) {
+        return TileXR::TILEXR_ERROR_MKIRT;
+    }
     if (start != nullptr && hipEventRecord(start, stream) != hipSuccess) {
         return TileXR::TILEXR_ERROR_INTERNAL;
     }
     const int ret = LaunchStatus(launch(), what);
     if (ret == TileXR::TILEXR_SUCCESS && stop != nullptr && hipEventRecord(stop, stream) != hipSuccess) {
         return TileXR::TILEXR_ERROR_INTERNAL;
+    }
+    if (ret == TileXR::TILEXR_SUCCESS && !stamp(1)) {
+        return TileXR::TILEXR_ERROR_MKIRT;
     }
     return ret;
 }

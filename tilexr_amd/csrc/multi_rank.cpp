@@ -192,6 +192,7 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     shape.memoryRoute = memoryRoute;
 
     std::lock_guard<std::mutex> lock(world->mu);
+    comm->debug.magic = magic;
     for (int s = 0; s < R; ++s) {
         if (world->comms[static_cast<size_t>(s)] == nullptr) {
             return TileXR::TILEXR_ERROR_NOT_INITIALIZED;     // the world is not complete yet
@@ -390,6 +391,7 @@ int RunCombineMulti(EpComm *comm, const EpCombineParams &p, bool memoryRoute, in
     shape.memoryRoute = memoryRoute;
 
     std::lock_guard<std::mutex> lock(world->mu);
+    comm->debug.magic = magic;
     for (int s = 0; s < R; ++s) {
         if (world->comms[static_cast<size_t>(s)] == nullptr) {
             return TileXR::TILEXR_ERROR_NOT_INITIALIZED;

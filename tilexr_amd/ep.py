@@ -23,7 +23,7 @@ EXPORTS = (
     "TileXRMoeEpDispatch", "TileXRMoeEpDispatchV2", "TileXRMoeEpDispatchMemory", "TileXRMoeEpDispatchMemoryV2",
     "TileXRMoeEpCombine", "TileXRMoeEpCombineV2", "TileXRMoeEpCombineMemory", "TileXRMoeEpCombineMemoryV2",
     "TileXRMoeEpDispatchMemoryEx", "TileXRMoeEpCombineMemoryEx", "TileXRMoeEpDispatchMemoryNoAlloc", "TileXREpVersion", "TileXREpSetKernelTimingEvents",
-    "TileXREpLastKernelName", "TileXREpMemoryProbe", "TileXREpTileProducerProbe",
+    "TileXREpLastKernelName", "TileXREpMemoryProbe", "TileXREpTileProducerProbe", "TileXREpSetDebugOptions",
     "TileXRCommInitRankLocal", "TileXRCommDestroy", "TileXRGetCommArgsHost", "TileXRGetCommArgsDev",
     "TileXRCommNextMagic",
 )
@@ -286,7 +286,8 @@ def set_kernel_timing_events(comm, kernel, start=None, stop=None):
                                                stop.handle if stop else None)
 
 
-PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_FAN_OUT, PROBE_FAN_IN, PROBE_GATHER_ROWS = range(6)
+PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_FAN_OUT, PROBE_FAN_IN, PROBE_GATHER_ROWS, PROBE_GATHER_ROWS_2K_X8, \
+    PROBE_GATHER_ROWS_4K_X6 = range(8)
 
 
 def memory_probe(pattern, src, dst, nbytes, stream):
@@ -304,6 +305,22 @@ def tile_producer_probe(src, dst, rows, row_bytes, tile_flags, tile_rows, epoch,
                    C.c_void_p]
     return fn(_ptr(src), _ptr(dst), int(rows), int(row_bytes), _ptr(tile_flags), int(tile_rows), int(epoch),
               int(workgroups), int(min_tile_ns), _stream(stream))
+
+
+class DebugOptions(C.Structure):
+    _fields_ = [("phaseStamps", C.c_void_p), ("phaseStampCapacity", C.c_int64), ("poisonUnwrittenRows", C.c_int64)]
+
+
+def set_debug_options(comm, phase_stamps=None, poison=False):
+    """phase_stamps: int64 / uint64 device tensor [capacity, 4] or None; poison: fill the rows a dispatch may write with
+    0x7f bytes first.  Both off: clears the options."""
+    fn = lib().TileXREpSetDebugOptions
+    fn.argtypes = [C.c_void_p, C.POINTER(DebugOptions)]
+    if phase_stamps is None and not poison:
+        return fn(_h(comm), None)
+    opt = DebugOptions(None if phase_stamps is None else phase_stamps.data_ptr(),
+                       0 if phase_stamps is None else phase_stamps.shape[0], 1 if poison else 0)
+    return fn(_h(comm), C.byref(opt))
 
 
 def last_kernel_name(comm, kernel):
