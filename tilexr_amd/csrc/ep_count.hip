@@ -5,6 +5,8 @@
 //   place   destination row of every route, assist tuples, inverse map
 //   invert  (combine side) row -> (token, k) inverse rebuilt from assist tuples
 // All integer work; the reference behaviour each kernel restates is cited at the kernel.
+#include <type_traits>
+
 #include <hip/hip_runtime.h>
 
 #include "ep_block_scan.hip.h"
@@ -250,21 +252,52 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     int *kept = s_cnt;                 // reuse: [numKeys]
     for (int key = tid; key < a.numKeys; key += kThreads) {
         int run = a.numChunks == 1 ? s_tot[key] : 0;
-        // the loads of a batch are independent: one round trip per 32 chunks
+        // the loads of a batch are independent: one round trip per 32 chunks.  Whole batches run without a test per
+        // load: this workgroup is alone on the launch's critical path and runs code nobody has fetched before it, so
+        // the instructions it needs count as much as the memory round trips
+        // (hence also buffer accesses: the chunk's offset is a scalar, one instruction per load)
         constexpr int kBatch = 32;
-        for (int c0 = 0; c0 < a.numChunks && a.numChunks > 1; c0 += kBatch) {
-            int v[kBatch];
+        int32_t *col = a.s.chunkHist + key;
+        const int rowBytes = a.numKeys * 4;
+        int c0 = 0;
+        if (a.numChunks > 1 && static_cast<int64_t>(a.numChunks) * rowBytes < (int64_t{1} << 31)) {
+            // chunks past the last one lie outside the buffer: their loads return zero, their stores are dropped
+            const __amdgpu_buffer_rsrc_t hist = RowResource(a.s.chunkHist, a.numChunks * rowBytes);
+            auto batches = [&](auto width) {
+                constexpr int kWidth = decltype(width)::value;
+                for (; c0 < a.numChunks; c0 += kWidth) {
+                    int v[kWidth];
 #pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
+                    for (int u = 0; u < kWidth; ++u) {
+                        v[u] = __builtin_amdgcn_raw_buffer_load_b32(hist, (c0 + u) * rowBytes + key * 4, 0, kAuxAgentScopeKept);
+                    }
+#pragma unroll
+                    for (int u = 0; u < kWidth; ++u) {
+                        __builtin_amdgcn_raw_buffer_store_b32(run, hist, (c0 + u) * rowBytes + key * 4, 0, 0);
+                        run += v[u];
+                    }
+                }
+            };
+            if (a.numChunks <= kBatch) {
+                batches(std::integral_constant<int, kBatch>{});
+            } else {
+                batches(std::integral_constant<int, 2 * kBatch>{});
+            }
+        }
+#pragma unroll 1
+        for (; c0 < a.numChunks && a.numChunks > 1; c0 += 4) {
+            int v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
                 const int c = c0 + u;
-                v[u] = c < a.numChunks ? __hip_atomic_load(&a.s.chunkHist[static_cast<int64_t>(c) * a.numKeys + key],
-                    __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+                v[u] = c < a.numChunks ? __hip_atomic_load(col + static_cast<int64_t>(c) * a.numKeys, __ATOMIC_RELAXED,
+                    __HIP_MEMORY_SCOPE_AGENT) : 0;
             }
 #pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
+            for (int u = 0; u < 4; ++u) {
                 const int c = c0 + u;
                 if (c < a.numChunks) {
-                    a.s.chunkHist[static_cast<int64_t>(c) * a.numKeys + key] = run;
+                    col[static_cast<int64_t>(c) * a.numKeys] = run;
                     run += v[u];
                 }
             }

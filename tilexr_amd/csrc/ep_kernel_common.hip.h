@@ -47,6 +47,9 @@ __device__ __forceinline__ void LdsBarrier()
 // workgroups of a token share (measured: 132 us instead of 93 us for the scatter).
 constexpr int kAuxAgentScope = 16 | 2;      // sc1 nt
 constexpr int kAuxNonTemporal = 2;          // nt
+constexpr int kAuxAgentScopeKept = 16;      // sc1 alone: for small tables a later kernel reads again (with nt on the
+                                            // loads of the count kernel's histograms the scatter that resolves rows from
+                                            // the same table afterwards ran 10 us slower: 92 instead of 82 us)
 constexpr unsigned kRawBufferWord3 = 0x00020000u;
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t RowResource(const void *row, int bytes)

@@ -58,10 +58,11 @@ inline PlaceArgs MakePlaceArgs(const RoutePlaceLaunch &l)
 // Resolves route i (< a.n), writes its assist tuple and rowOf entry, returns the row or -1.
 __device__ __forceinline__ int PlaceRoute(const PlaceArgs &a, int i)
 {
+    // both loads at once: the id is there for every route, whether it is live or not
     const int lr = a.localRank[i];
+    const int e = a.ids[i];
     int row = -1;
     if (lr >= 0) {
-        const int e = a.ids[i];
         const int key = a.keyDiv == 1 ? e : e / a.keyDiv;
         const int within = a.chunkBase[static_cast<int64_t>(i >> a.chunkShift) * a.numKeys + key] + lr;
         if (a.capacity <= 0 || within < a.capacity) {
