@@ -175,7 +175,10 @@ struct TileXREpCombineExOptions {
     int32_t *deviceStatusOut;     // device int32, required with tileFlags (-3 without it): set to 1 when a flag
                                   //      wait expired; the waits that follow in that launch give up at once.  A
                                   //      token with an expired wait gets a row of zeros in yOut, never a partial sum.
-                                  //      The caller clears the word before the call
+                                  //      The caller clears the word before the call.  A combine on the stream of
+                                  //      the very dispatch that published these flags (same array, same epoch)
+                                  //      never waits, its producer being done before it starts: a word that is
+                                  //      not there then counts as expired at once
 };
 
 // Memory-route combine (same result as TileXRMoeEpCombineMemoryV2) with quantised expert output, a ready-made

@@ -162,6 +162,58 @@ def test_flag_wait_expires_instead_of_hanging():
         assert st == ep.ERR_PARA_CHECK_FAIL
 
 
+@pytest.mark.parametrize("quant", ["none", "int8"])
+def test_missing_word_after_a_same_stream_dispatch_gives_zero_tokens_at_once(quant):
+    """Combine on the stream of the dispatch that published the flags does not wait (the producer is done before it
+    starts); a word that is not there then (here: wiped between the two calls) can never come, so the tokens that need
+    that tile get rows of zeros and the status word is set, without the wait bound being sat out, and every other token
+    still equals the oracle."""
+    bs, h, K, E, tile_rows = 512, 1024, 4, 32, 32
+    rng = np.random.default_rng(21)
+    ids, w = routing(rng, bs, K, E)
+    x = torch.from_numpy(rng.standard_normal((bs, h)).astype(np.float32)).to(torch.bfloat16)
+    q = ep.Q_TOKEN_INT8 if quant == "int8" else ep.Q_NONE
+    oq = O.Q_TOKEN_INT8 if quant == "int8" else O.Q_NONE
+    case = O.Case(1, bs, h, K, E, dtype=O.DT_BF16, quant_mode=oq, token_nums_type=1)
+    want = O.mem_dispatch(case, 0, bits16(x)[None], ids[None])
+    eo = want["expand_x"][None] if oq else want["expand_x"].view(np.uint16)[None]
+    want_y = O.mem_combine(O.Case(1, bs, h, K, E, dtype=O.DT_BF16), 0, eo, want["assist"][None],
+                           want["send_counts"][None], expert_scales=w, in_quant=oq,
+                           in_scales=want["dyn_scales"] if oq else None)
+    n = bs * K
+    wiped = [3, 17]
+    with Session() as s:
+        d_x, d_ids, d_w = x.to(DEV), to_dev(ids), to_dev(w)
+        out = alloc_dispatch_outputs(bs, h, K, E, quant=q)
+        counts = torch.zeros((E,), dtype=torch.int32, device=DEV)
+        flags = torch.zeros((n // tile_rows,), dtype=torch.int64, device=DEV)
+        status = torch.zeros((1,), dtype=torch.int32, device=DEV)
+        y = torch.full((bs, h), 3.0, dtype=torch.bfloat16, device=DEV)
+        st, epoch = ep.dispatch_memory_ex(d_x, d_ids, s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                          out["token_nums"], counts, ep.DT_BF16, s.stream, quant_mode=q,
+                                          dynamic_scales=out.get("scales"), row_index_map=out["row_map"],
+                                          tile_flags=flags, tile_rows=tile_rows)
+        assert st == 0
+        flags[wiped] = 0                                   # on the session's stream, between the two calls
+        start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        st = ep.combine_memory_ex(out["expand_x"], out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, s.stream,
+                                  expert_out_quant_mode=q, expert_out_scales=out.get("scales"), expert_scales=d_w,
+                                  row_index_map=out["row_map"], tile_flags=flags, tile_rows=tile_rows, flag_epoch=epoch,
+                                  wait_timeout_us=30_000_000, device_status=status)
+        stop.record()
+        assert st == 0
+        s.sync()
+        assert status.item() == 1
+        assert start.elapsed_time(stop) < 1000.0           # milliseconds: nowhere near the 30 s bound
+        row_map = out["row_map"].cpu().numpy()
+        hit = np.isin(row_map // tile_rows, wiped).any(axis=1) & (row_map >= 0).any(axis=1)
+        assert 0 < hit.sum() < bs
+        got = bits16(y)
+        assert np.all(got[hit] == 0)
+        assert np.array_equal(got[~hit], want_y[~hit])
+
+
 def test_combine_follows_an_expert_stage_that_publishes_tiles_in_random_order():
     """The producer here is not the dispatch but an "expert stage" written with torch ops on a second stream: it
     rewrites the rows tile by tile in a random order and stores a tile's readiness word after the tile's rows (a
