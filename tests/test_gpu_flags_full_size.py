@@ -152,6 +152,15 @@ def test_wide_quantised_rows_with_tile_flags(two_streams):
                   expect_reduce="ep_reduce_quant_kernel")
 
 
+@pytest.mark.parametrize("two_streams", [False, True], ids=["one_stream", "two_streams"])
+def test_rows_wider_than_one_publishing_workgroup(two_streams):
+    """Rows of 1536 vectors: the publishing per-route scatter cuts them into two workgroups of 512 lanes, each of which
+    reports its part of the row, so a row counts twice towards its tile (the headline rows fit one such workgroup)."""
+    wide = workloads.Workload("bf16@12288", 1, 1024, 12288, 4, 32, x_dist="normal", routing="zipf", zipf_s=1.0, seed=77)
+    run_and_check(layers_of(wide), 100, two_streams, expect_scatter="ep_scatter_route_kernel",
+                  expect_reduce="ep_reduce_vec_kernel")
+
+
 def test_two_communicators_share_one_flag_array():
     """Flag epochs come from one counter for the whole process: two communicators that are handed the same flag array
     one after the other can never tag it with the same value, so words left by the first read as not ready to a

@@ -196,6 +196,7 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     scatter.out = p.expandXOut;
     scatter.scalesOut = p.dynamicScalesOut;
     scatter.tileFlags = p.tileFlagsOut;
+    scatter.consumerBeside = p.metaReadyEvent != nullptr;
     // a tile never holds more rows than the dispatch can produce: larger values name the same single tile
     scatter.tileRows = std::min<int64_t>(p.tileRows, std::max<int64_t>(n, 1));
     scatter.epoch = flagEpoch;

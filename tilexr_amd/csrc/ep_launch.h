@@ -114,6 +114,8 @@ struct ScatterLaunch {
     int64_t tileRows;
     uint64_t epoch;
     const int32_t *totalRowsPtr; // device word: rows kept by this dispatch (size of the last tile)
+    bool consumerBeside;         // a consumer of the flags is expected to run beside this launch (the caller asked for a
+                                 // metadata-ready event): keep the workgroups small enough to fit next to its waiting ones
     const char **kernelNameOut;  // optional: receives the name of the kernel template that was launched
     hipStream_t stream;
 };

@@ -2,7 +2,8 @@
 //
 // HBM-bound byte movement, no MFMA.  Three kernels share the work:
 //   ep_scatter_route_kernel    plain copies of wide rows in batches of 1024 tokens and more: one workgroup per
-//                              (token, k, slice of 512 vectors), two 16-byte loads and two 16-byte stores per lane
+//                              (token, k, slice of 512 vectors; 1024 when readiness flags are published), two 16-byte
+//                              loads and two 16-byte stores per lane
 //   ep_scatter_vec_kernel      everything else that is 16-byte aligned (quantised payloads, narrow rows, small
 //                              batches): G lanes cooperate on one token (a wave for narrow rows, the whole workgroup
 //                              for wide ones); a lane keeps V 16-byte vectors of the row in registers, so every load of
@@ -485,7 +486,20 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
                 if (l.kernelNameOut != nullptr) {
                     *l.kernelNameOut = "ep_scatter_route_kernel";
                 }
-                if (WriteThrough(a)) {
+                if (WriteThrough(a) && a.colSlices > 1 && !l.consumerBeside) {
+                    // A publishing workgroup stays until its stores have landed and then counts its part of the row
+                    // towards the tile: worth doing once per row rather than once per half row, so rows wider than 512
+                    // vectors get workgroups of 512 lanes (4096 x 7168 x top-8: 82.2 instead of 84.7 us; without
+                    // flags the narrower workgroups are the faster ones, 81.9 against 82.5 us).  Not when a consumer
+                    // is expected beside this launch: its waiting workgroups leave room for the narrower ones only
+                    // (dispatch + combine on two streams: 272 us with the wide ones, 244 us with the narrow ones).
+                    constexpr int kWide = 2 * kThreads;
+                    ScatterArgs wide = a;
+                    wide.colSlices = (a.h / 8 + kRouteVecs * kWide - 1) / (kRouteVecs * kWide);
+                    const dim3 wideBlocks(static_cast<unsigned>(static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK * wide.colSlices));
+                    hipLaunchKernelGGL((ep_scatter_route_kernel<kWide, kRouteVecs, true>), wideBlocks, dim3(kWide), 0,
+                        l.stream, wide);
+                } else if (WriteThrough(a)) {
                     hipLaunchKernelGGL((ep_scatter_route_kernel<kThreads, kRouteVecs, true>), blocks, dim3(kThreads), 0,
                         l.stream, a);
                 } else {
