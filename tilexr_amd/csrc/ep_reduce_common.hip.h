@@ -1,0 +1,376 @@
+// Shared by the translation units of the reduce: launch arguments, the row map, tile readiness flags on the consumer
+// side and the loop that hands a workgroup its tokens.  (The kernels are spread over several files so that they compile
+// side by side; the code of one kernel is in one place.)
+#ifndef TILEXR_AMD_EP_REDUCE_COMMON_HIP_H
+#define TILEXR_AMD_EP_REDUCE_COMMON_HIP_H
+
+#include <hip/hip_runtime.h>
+
+#include <type_traits>
+
+#include "ep_kernel_common.hip.h"
+#include "ep_launch.h"
+#include "ep_numerics.hip.h"
+#include "ep_tile_publish.h"
+#include "tilexr_ep.h"
+
+namespace TileXREp {
+
+struct ReduceArgs {
+    const void *expertOut;
+    int64_t rowBytes;
+    const uint64_t *inverseTagged;
+    uint64_t epoch;
+    const int32_t *rowIndexMap;
+    const uint64_t *orderKeys;
+    const float *expertScales;
+    const uint8_t *tokenMask;
+    const void *sharedExpertX;
+    const float *inScales;
+    int bs;
+    int h;
+    int topK;
+    int maxRows;                     // rows expertOut holds
+    int slots;                       // rows summed per token: topK routed ones, then the shared-expert slots
+    void *y;
+    int colSlices;                   // slices a row is cut into (vec kernel, wide rows), else 1
+    const uint64_t *tileFlags;
+    int tileRows;
+    uint64_t flagEpoch;
+    int64_t waitTimeoutTicks;
+    int32_t *deviceStatus;
+    int flagsSettled;                // the producer of the flags finished before this launch began (same stream)
+};
+
+// Launchers of the register-resident kernels, one translation unit per (element type, with / without readiness flags).
+// g, v: lanes per token (or per slice of a token's row) and 16-byte vectors per lane; a combination that a unit does
+// not hold is a programming error and launches nothing.
+void LaunchReduceVecBf16(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceVecBf16Flags(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceVecFp16(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceVecFp16Flags(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceQuantBf16(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceQuantBf16Flags(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceQuantFp16(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceQuantFp16Flags(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+
+namespace {
+
+// Row of a (token, slot), -1 for none.  A row at or beyond `maxRows` (only a corrupted map has one) counts as none: the
+// kernels never read outside the rows the caller's buffer holds.
+__device__ __forceinline__ int LookupRow(const ReduceArgs &a, int64_t slot)
+{
+    int row;
+    if (a.rowIndexMap != nullptr) {
+        row = a.rowIndexMap[slot];
+    } else {
+        const uint64_t e = a.inverseTagged[slot];
+        row = (e >> 32) == a.epoch ? static_cast<int>(e & 0xffffffffu) : -1;
+    }
+    return static_cast<unsigned>(row) < static_cast<unsigned>(a.maxRows) ? row : -1;
+}
+
+// Bounded wait until the tile holding `row` has been published for this epoch (its word carries the epoch).  The poll itself is a relaxed
+// device-scope load (no cache maintenance per iteration -- an acquire in the loop would invalidate this XCD's L2 on
+// every spin and starve the producer).  What the caller reads afterwards must not come from a stale L2 line: the
+// register-resident kernels read published rows with agent-scope loads, which are served from memory; the
+// element-granular kernel issues one acquire fence after all its waits have succeeded.
+__device__ inline bool WaitTile(const ReduceArgs &a, int row)
+{
+    const int tile = row / a.tileRows;
+    const uint64_t start = wall_clock64();
+    // every poll is a round trip to memory (agent scope): the gap between polls doubles up to about 3 us
+    int backoff = 0;
+    while (true) {
+        const uint64_t w = __hip_atomic_load(&a.tileFlags[tile], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (TileWordReady(w, a.flagEpoch)) {
+            return true;
+        }
+        if (static_cast<int64_t>(wall_clock64() - start) > a.waitTimeoutTicks) {
+            return false;
+        }
+        // once one wait of the launch has expired the producer is taken to be gone: later waits give up at once,
+        // so a launch whose flags never arrive ends after about one timeout, not one per tile
+        if (a.deviceStatus != nullptr &&
+            __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0) {
+            return false;
+        }
+        switch (backoff) {                  // s_sleep takes an immediate: 64 clocks per unit
+            case 0: __builtin_amdgcn_s_sleep(8); break;
+            case 1: __builtin_amdgcn_s_sleep(16); break;
+            case 2: __builtin_amdgcn_s_sleep(32); break;
+            case 3: __builtin_amdgcn_s_sleep(64); break;
+            default: __builtin_amdgcn_s_sleep(127); break;
+        }
+        backoff += backoff < 4 ? 1 : 0;
+    }
+}
+
+// Insertion sort of row indices, absent rows (-1) last.  The order is the row index itself, or -- when rows come
+// from several expert ranks -- the (expert rank, row) key recorded for each slot.  K is small.
+__device__ inline void SortRows(int *rows, int k, const uint64_t *orderKeys)
+{
+    if (orderKeys != nullptr) {
+        for (int i = 1; i < k; ++i) {
+            const int v = rows[i];
+            const uint64_t kv = v < 0 ? ~0ull : orderKeys[v];
+            int j = i - 1;
+            while (j >= 0 && (rows[j] < 0 ? ~0ull : orderKeys[rows[j]]) > kv) {
+                rows[j + 1] = rows[j];
+                --j;
+            }
+            rows[j + 1] = v;
+        }
+        return;
+    }
+    for (int i = 1; i < k; ++i) {
+        const int v = rows[i];
+        const unsigned kv = static_cast<unsigned>(v);      // -1 becomes the largest key
+        int j = i - 1;
+        while (j >= 0 && static_cast<unsigned>(rows[j]) > kv) {
+            rows[j + 1] = rows[j];
+            --j;
+        }
+        rows[j + 1] = v;
+    }
+}
+
+// Row loads of the register-resident kernels.  FL = false: non-temporal loads.  FL = true (rows published through
+// readiness flags, possibly a moment ago by a workgroup on another XCD): agent-scope loads, served from memory, so
+// that no acquire fence (an invalidate of this XCD's whole L2) is needed per token.
+template <bool FL>
+__device__ __forceinline__ u32x4 RowLoad(const char *rowBase, __amdgpu_buffer_rsrc_t rsrc, int byteOffset)
+{
+    if (FL) {
+        return __builtin_amdgcn_raw_buffer_load_b128(rsrc, byteOffset, 0, kAuxAgentScope);
+    }
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(rowBase + byteOffset));
+}
+
+template <bool FL>
+__device__ __forceinline__ float ScaleLoad(const float *p)
+{
+    if (FL) {
+        return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return *p;
+}
+
+// One look at the tile holding `row`: published for this epoch or not.
+__device__ __forceinline__ bool TilePublished(const ReduceArgs &a, int row)
+{
+    const uint64_t w = __hip_atomic_load(&a.tileFlags[row / a.tileRows], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return TileWordReady(w, a.flagEpoch);
+}
+
+// Fills s_row / s_w for one token and deals with tile flags.  BLOCK: every slot waits (bounded) for its tile.  Otherwise
+// `mode` says what a slot does about its tile:
+//   kRouteCheck    look once; a tile that is not there yet leaves kRowPending in the slot and the call returns true
+//                  ("come back later")
+//   kRouteTrusted  nothing: the caller has just seen every tile of this token published
+//   kRouteGiveUp   look once; a tile that is not there turns the slot into an expired one
+//   kRouteSettled  the producer finished before this launch began, so nothing is waited for and no read can come too
+//                  early: the slot gets its row at once and the call returns whether the tile's word says otherwise,
+//                  a value the caller needs only after the rows have been read (the word travels beside the rows
+//                  instead of ahead of them: one dependent round trip less)
+// An expired wait sets the launch's status word and leaves kRowExpired in the slot: the token then gets a row of zeros
+// (AnyExpired), never the sum of the rows that happened to be ready.
+constexpr int kRowExpired = -2;
+constexpr int kRowPending = -3;
+enum RouteMode : int { kRouteCheck = 0, kRouteTrusted = 1, kRouteGiveUp = 2, kRouteSettled = 3 };
+
+__device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
+{
+    bool expired = false;
+    for (int k = 0; k < slots; ++k) {
+        expired |= rows[k] == kRowExpired;
+    }
+    return expired;
+}
+
+template <bool FENCE, bool BLOCK>
+__device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
+    float *weights, int mode)
+{
+    bool pending = false;
+    for (int k = lane; k < a.slots; k += lanes) {
+        const int64_t slot = static_cast<int64_t>(tokOk ? token : 0) * a.slots + k;
+        int row = tokOk ? LookupRow(a, slot) : -1;
+        const bool settled = !BLOCK && mode == kRouteSettled;
+        if (!settled && row >= 0 && a.tileFlags != nullptr && (BLOCK || mode != kRouteTrusted)) {
+            const bool there = BLOCK ? WaitTile(a, row) : TilePublished(a, row);
+            if (!there && !BLOCK && mode == kRouteCheck) {
+                row = kRowPending;
+                pending = true;
+            } else if (!there) {
+                if (a.deviceStatus != nullptr) {
+                    atomicExch(a.deviceStatus, 1);
+                }
+                row = kRowExpired;
+            }
+        }
+        rows[k] = row;
+        // shared-expert slots follow the routed ones and carry no gate weight
+        // (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:650-657)
+        weights[k] = (tokOk && a.expertScales != nullptr && k < a.topK) ?
+            a.expertScales[static_cast<int64_t>(token) * a.topK + k] : 1.0f;
+        if (settled && row >= 0 && a.tileFlags != nullptr) {
+            // the last load of all: the memory counter runs in order, so nothing that is needed before the rows may
+            // come after it
+            // (an ordinary load: the words are final, this XCD's L2 may keep them)
+            pending |= !TileWordReady(a.tileFlags[row / a.tileRows], a.flagEpoch);
+        }
+    }
+    if (FENCE && a.tileFlags != nullptr && lane < a.slots) {
+        // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
+        // workgroup after the barrier that follows) are at least as new as the flag values seen above
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    return pending;
+}
+
+// Runs unit(group, beforeStores) for this workgroup's groups: blockIdx.x, blockIdx.x + gridDim.x, ...  beforeStores is
+// a callable the unit invokes once, after its last load has been used and before its first store.  `load(group, mode)`
+// fills the workgroup's route tables for a group and returns (per lane) whether a tile it needs is not published yet;
+// `tokenAt(group, t)` names the t-th of a group's `tokensPerGroup` tokens (-1 = none).
+//
+// Without readiness flags that is a plain loop.  With them (WAITS) a workgroup never sits on one group while others it
+// owes are ready: a token needs the tiles of all its rows, which a producer that works tile by tile finishes at
+// unrelated times, so tokens become ready in no particular order.  The workgroup takes its groups 32 at a time.  A
+// first pass reduces every group whose tiles are there already (all of them when the producer ran earlier on the same
+// stream).  For what is left it then goes in rounds: all lanes together look once at every tile the pending groups need
+// (one round trip for the lot), the groups that have become complete are reduced, and a round without any is followed
+// by a sleep that grows to about 14 us.  When nothing it owes has become ready for the wait bound, or another workgroup
+// has reported an expired wait, the rest is given up: those tokens get rows of zeros and the launch's status word is set.
+template <bool WAITS, typename TokenAt, typename Load, typename Unit>
+__device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, int tokensPerGroup, TokenAt tokenAt,
+    Load load, Unit unit)
+{
+    if constexpr (!WAITS) {
+        for (int group = blockIdx.x; group < groups; group += gridDim.x) {
+            __syncthreads();        // the previous iteration's readers are done with the route tables
+            load(group, kRouteTrusted);
+            __syncthreads();
+            unit(group, [] {});
+        }
+    } else {
+        if (a.flagsSettled != 0) {
+            // No barrier of the kind that waits for memory after the rows have been stored: a workgroup that has to see
+            // its stores complete before it may leave stays a store round trip longer (2048-byte fp8 rows: 53 instead of
+            // 43 us).  The verdict on the tile words goes through LDS, two slots taken in turn so that the reset of one
+            // is a whole iteration away from its last readers.
+            __shared__ int s_missing[2];
+            int turn = 0;
+            for (int group = blockIdx.x; group < groups; group += gridDim.x, turn ^= 1) {
+                if (threadIdx.x == 0) {
+                    s_missing[turn] = 0;
+                }
+                __syncthreads();
+                const bool missing = load(group, kRouteSettled);
+                LdsBarrier();                       // the tile words are still on their way: nothing waits for them here
+                // the verdict is handed over between the last use of the rows and the first store: whoever asks for the
+                // tile word there finds it long since arrived (it was requested ahead of the rows), and the barrier
+                // below does not wait for the stores
+                unit(group, [&] {
+                    if (missing) {
+                        s_missing[turn] = 1;
+                    }
+                });
+                LdsBarrier();
+                if (s_missing[turn] != 0) {
+                    // a word that is not there now never will be: the token gets a row of zeros and the status is set
+                    __syncthreads();
+                    load(group, kRouteGiveUp);
+                    __syncthreads();
+                    unit(group, [] {});
+                }
+            }
+            return;
+        }
+        __shared__ uint32_t s_notReady;
+        const int first = static_cast<int>(blockIdx.x);
+        const int stride = static_cast<int>(gridDim.x);
+        const int mine = groups > first ? (groups - 1 - first) / stride + 1 : 0;
+        const int perGroup = tokensPerGroup * a.slots;
+        for (int base = 0; base < mine; base += 32) {
+            const int inWindow = mine - base < 32 ? mine - base : 32;
+            uint32_t pending = inWindow == 32 ? 0xffffffffu : ((1u << inWindow) - 1u);
+            for (uint32_t m = pending; m != 0u; m &= m - 1u) {
+                const int i = __builtin_ctz(m);
+                const int group = first + (base + i) * stride;
+                __syncthreads();
+                const bool waiting = load(group, kRouteCheck);
+                if (__syncthreads_or(waiting ? 1 : 0) != 0) {
+                    continue;                       // uniform: every lane gets the same answer
+                }
+                unit(group, [] {});
+                pending &= ~(1u << i);
+            }
+            uint64_t idleSince = wall_clock64();
+            int backoff = 0;
+            while (pending != 0u) {
+                if (threadIdx.x == 0) {
+                    s_notReady = 0u;
+                }
+                __syncthreads();
+                for (int idx = threadIdx.x; idx < inWindow * perGroup; idx += blockDim.x) {
+                    const int i = idx / perGroup;
+                    if (((pending >> i) & 1u) == 0u) {
+                        continue;
+                    }
+                    const int token = tokenAt(first + (base + i) * stride, (idx % perGroup) / a.slots);
+                    if (token < 0) {
+                        continue;
+                    }
+                    const int row = LookupRow(a, static_cast<int64_t>(token) * a.slots + idx % a.slots);
+                    if (row >= 0 && !TilePublished(a, row)) {
+                        atomicOr(&s_notReady, 1u << i);
+                    }
+                }
+                __syncthreads();
+                const uint32_t ready = pending & ~s_notReady;
+                if (ready == 0u) {
+                    bool stop = false;
+                    if (threadIdx.x == 0) {
+                        stop = static_cast<int64_t>(wall_clock64() - idleSince) > a.waitTimeoutTicks ||
+                            (a.deviceStatus != nullptr &&
+                             __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0);
+                    }
+                    if (__syncthreads_or(stop ? 1 : 0) != 0) {
+                        for (uint32_t m = pending; m != 0u; m &= m - 1u) {
+                            const int group = first + (base + __builtin_ctz(m)) * stride;
+                            __syncthreads();
+                            load(group, kRouteGiveUp);
+                            __syncthreads();
+                            unit(group, [] {});
+                        }
+                        pending = 0u;
+                        break;
+                    }
+                    for (int r = 0; r < (1 << backoff); ++r) {
+                        __builtin_amdgcn_s_sleep(127);      // 127 x 64 clocks, about 3.5 us
+                    }
+                    backoff += backoff < 2 ? 1 : 0;
+                    continue;
+                }
+                for (uint32_t m = ready; m != 0u; m &= m - 1u) {
+                    const int i = __builtin_ctz(m);
+                    const int group = first + (base + i) * stride;
+                    __syncthreads();
+                    load(group, kRouteTrusted);
+                    __syncthreads();
+                    unit(group, [] {});
+                    pending &= ~(1u << i);
+                }
+                idleSince = wall_clock64();
+                backoff = 0;
+            }
+        }
+    }
+}
+
+
+} // namespace
+} // namespace TileXREp
+
+#endif // TILEXR_AMD_EP_REDUCE_COMMON_HIP_H

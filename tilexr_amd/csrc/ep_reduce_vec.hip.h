@@ -1,0 +1,240 @@
+// reduce: y[token] = sum over the token's rows, gathered through the inverse map (gfx950, wave64).
+//
+// HBM-bound: topK row reads per output row, < 0.5 FLOP per byte, no MFMA.  G lanes cooperate on one token and keep
+// V x 8 fp32 accumulators in registers; for each route in k order a lane issues all V of its 128-bit non-temporal
+// loads of that row before touching the accumulators, so 64-128 bytes per lane are in flight while the previous
+// row is being summed.  Measured on MI355X this moves 4096 x 7168 bf16 x top-8 (529 MB) at about 6 TB/s.
+//
+//   KIND fp32     sum = 0; for k = 0..K-1: sum = sum + (w_k * row_k) in fp32 (separate multiply and add), then the
+//                 shared-expert row, then one round-to-nearest-even (saturating for fp16) to the output type;
+//                 an inactive token (mask) gives zeros
+//                 (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:505-553, 555-571, 573-601, 632-662)
+//   KIND per-add  rows in ascending row index; y = T(float(y) + float(row)) after every add
+//                 (reference: src/ep/kernels/tilexr_ep_combine_kernel.cpp:15-26, 54-101)
+//   COMMQ 3/4     every row first takes the MXFP8 e5m2 / e4m3 round trip and is accumulated as
+//                 ((fp8 * 2^(s-127)) * w) (reference: src/ep/kernels/tilexr_ep_mxfp8_quant.h:286-352)
+//   INQ 2/5       rows hold int8 / fp8 payloads that are dequantised with their scales and rounded to the element
+//                 type first (no reference counterpart)
+//
+// This file holds the register-resident kernel for 16-bit rows and is compiled once per (element type, with / without
+// readiness flags): the including file sets TILEXR_REDUCE_BF16, TILEXR_REDUCE_FLAGS and TILEXR_REDUCE_ENTRY.
+#if !defined(TILEXR_REDUCE_BF16) || !defined(TILEXR_REDUCE_FLAGS) || !defined(TILEXR_REDUCE_ENTRY)
+#error "include from ep_reduce_vec_*.hip"
+#endif
+
+#include "ep_reduce_common.hip.h"
+
+namespace TileXREp {
+namespace {
+
+template <int G, int V, int KIND, bool BF16, int COMMQ, bool FL>
+__global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
+{
+    constexpr int kTokens = kThreads / G;
+    constexpr bool kMx = COMMQ != 0;
+    constexpr bool kCommE5m2 = COMMQ == TILEXR_EP_QUANT_COMM_MXFP8_E5M2;
+    __shared__ int s_row[kTokens][kMaxTopK];
+    __shared__ float s_w[kTokens][kMaxTopK];
+
+    const int tg = threadIdx.x / G;
+    const int lane = threadIdx.x % G;
+    // Rows in flight per lane.  A whole workgroup per token is the geometry of launches that may wait on flags: at most two
+    // such workgroups run per compute unit, so a wave may use half a SIMD's registers and keeps four rows in flight
+    // whatever the row width; the other geometries run many more waves and trade rows in flight for occupancy.
+    constexpr int KB = G == kThreads ? 4 : (V <= 2 ? 4 : (V <= 4 ? 2 : 1));
+    const int vecs = a.h / 8;
+    // a unit is one token, or -- for wide rows -- one slice of G * V vectors of a token
+    const int units = a.bs * a.colSlices;
+    // the launch may use fewer waves per workgroup than kThreads / kWave (single-wave workgroups for sliced rows)
+    const int unitsPerGroup = static_cast<int>(blockDim.x) / G;
+    const int groups = (units + unitsPerGroup - 1) / unitsPerGroup;
+
+    auto tokenAt = [&](int group, int t) {
+        const int unit = group * unitsPerGroup + t;
+        return unit < units ? unit / a.colSlices : -1;
+    };
+    auto load = [&](int group, int mode) {
+        const int unit = group * unitsPerGroup + tg;
+        return LoadRoutes<false, false>(a, unit / a.colSlices, unit < units, lane, G, s_row[tg], s_w[tg], mode);
+    };
+    auto reduceUnit = [&](int group, auto beforeStores) {
+        const int unit = group * unitsPerGroup + tg;
+        const bool tokOk = unit < units;
+        const int token = unit / a.colSlices;
+        const int colBase = (unit % a.colSlices) * (G * V);
+        if (KIND == kReducePerAdd) {
+            if (lane == 0) {
+                SortRows(s_row[tg], a.slots, a.orderKeys);
+            }
+            __syncthreads();
+        }
+        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !(FL && AnyExpired(s_row[tg], a.slots));
+
+        float acc[V][8];
+#pragma unroll
+        for (int j = 0; j < V; ++j) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                acc[j][e] = 0.0f;
+            }
+        }
+        // control flow below is uniform across the lanes that share a token (the MXFP8 round trip shuffles)
+        for (int k0 = 0; k0 < a.slots; k0 += KB) {
+            u32x4 v16[KB][V];
+            int rowOfK[KB];
+#pragma unroll
+            for (int u = 0; u < KB; ++u) {
+                const int k = k0 + u;
+                // the lanes of a wave share one token, so the row is wave-uniform
+                const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
+                rowOfK[u] = row;
+                const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
+                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    const int idx = colBase + j * G + lane;
+                    v16[u][j] = (row >= 0 && idx < vecs) ? RowLoad<FL>(base, rsrc, idx * 16) : u32x4{0u, 0u, 0u, 0u};
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < KB; ++u) {
+                if (rowOfK[u] < 0) {
+                    continue;
+                }
+                const float w = s_w[tg][k0 + u];
+#pragma unroll
+                for (int j = 0; j < V; ++j) {
+                    float f[8];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        f[2 * q] = Decode16<BF16>(v16[u][j][q] & 0xffffu);
+                        f[2 * q + 1] = Decode16<BF16>(v16[u][j][q] >> 16);
+                    }
+                    if (kMx) {
+                        float amax = 0.0f;
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            amax = fmaxf(amax, fabsf(f[e]));
+                        }
+                        amax = fmaxf(amax, __shfl_xor(amax, 1));
+                        amax = fmaxf(amax, __shfl_xor(amax, 2));
+                        const int se = MxSharedExponent<kCommE5m2>(amax);
+                        const float up = Exp2Int(se);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            const float back = Fp8Decode<kCommE5m2>(Fp8Encode<kCommE5m2>(ldexpf(f[e], -se)));
+                            f[e] = __fmul_rn(back, up);
+                        }
+                    }
+                    if (KIND == kReducePerAdd) {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            acc[j][e] = RoundTo16<BF16>(__fadd_rn(acc[j][e], f[e]));
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            acc[j][e] = __fadd_rn(acc[j][e], __fmul_rn(f[e], w));
+                        }
+                    }
+                }
+            }
+        }
+        if (a.sharedExpertX != nullptr && active) {
+            const u32x4 *sx = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.sharedExpertX) +
+                static_cast<int64_t>(token) * a.h * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = colBase + j * G + lane;
+                if (idx < vecs) {
+                    const u32x4 v = sx[idx];
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        acc[j][2 * q] = __fadd_rn(acc[j][2 * q], Decode16<BF16>(v[q] & 0xffffu));
+                        acc[j][2 * q + 1] = __fadd_rn(acc[j][2 * q + 1], Decode16<BF16>(v[q] >> 16));
+                    }
+                }
+            }
+        }
+        beforeStores();
+        if (tokOk) {
+            u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.y) + static_cast<int64_t>(token) * a.h * 2);
+#pragma unroll
+            for (int j = 0; j < V; ++j) {
+                const int idx = colBase + j * G + lane;
+                if (idx < vecs) {
+                    u32x4 o;
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        o[q] = active ? EncodePair16Sat<BF16>(acc[j][2 * q], acc[j][2 * q + 1]) : 0u;
+                    }
+                    __builtin_nontemporal_store(o, dst + idx);
+                }
+            }
+        }
+    };
+    ForEachGroup<FL>(a, groups, unitsPerGroup, tokenAt, load, reduceUnit);
+}
+
+
+template <int G, int V, int KIND, bool BF16, int COMMQ, bool FL>
+void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
+{
+    if constexpr (G == kThreads) {
+        // whole-workgroup tokens are only used for rows published through readiness flags
+        static_assert(FL, "one workgroup per token is the geometry of launches that wait on flags");
+        int grid = a.bs;
+        if (gridLimit > 0 && grid > gridLimit) {
+            grid = gridLimit;
+        }
+        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, true>), dim3(grid), dim3(kThreads), 0, stream, a);
+    } else {
+        // sliced rows: one wave per workgroup, so that no wave waits at a barrier for another slice's rows
+        const int threads = a.colSlices > 1 ? G : kThreads;
+        const int perGroup = threads / G;
+        const int64_t units = static_cast<int64_t>(a.bs) * a.colSlices;
+        int grid = static_cast<int>((units + perGroup - 1) / perGroup);
+        if (gridLimit > 0 && grid > gridLimit * (kThreads / threads)) {
+            grid = gridLimit * (kThreads / threads);
+        }
+        hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, FL>), dim3(grid), dim3(threads), 0, stream, a);
+    }
+}
+
+template <int G, int V, bool BF16, bool FL>
+void LaunchByMode(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
+{
+    if (l.reduceKind == kReducePerAdd) {
+        LaunchVec<G, V, kReducePerAdd, BF16, 0, FL>(a, gridLimit, l.stream);
+    } else if (l.commQuant == TILEXR_EP_QUANT_COMM_MXFP8_E5M2) {
+        LaunchVec<G, V, kReduceFp32, BF16, TILEXR_EP_QUANT_COMM_MXFP8_E5M2, FL>(a, gridLimit, l.stream);
+    } else if (l.commQuant == TILEXR_EP_QUANT_MXFP8) {
+        LaunchVec<G, V, kReduceFp32, BF16, TILEXR_EP_QUANT_MXFP8, FL>(a, gridLimit, l.stream);
+    } else {
+        LaunchVec<G, V, kReduceFp32, BF16, 0, FL>(a, gridLimit, l.stream);
+    }
+}
+
+} // namespace
+
+void TILEXR_REDUCE_ENTRY(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
+{
+    constexpr bool kBf16 = TILEXR_REDUCE_BF16;
+    constexpr bool kFlags = TILEXR_REDUCE_FLAGS;
+    if (g == kWave && v == 2) {
+        LaunchByMode<kWave, 2, kBf16, kFlags>(l, a, gridLimit);
+    } else if (g == kWave && v == 4) {
+        LaunchByMode<kWave, 4, kBf16, kFlags>(l, a, gridLimit);
+    }
+    if constexpr (kFlags) {
+        if (g == kThreads && v == 2) {
+            LaunchByMode<kThreads, 2, kBf16, true>(l, a, gridLimit);
+        } else if (g == kThreads && v == 4) {
+            LaunchByMode<kThreads, 4, kBf16, true>(l, a, gridLimit);
+        } else if (g == kThreads && v == 8) {
+            LaunchByMode<kThreads, 8, kBf16, true>(l, a, gridLimit);
+        }
+    }
+}
+
+} // namespace TileXREp
