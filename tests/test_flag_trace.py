@@ -204,7 +204,7 @@ def test_trace_covers_the_two_level_counters():
     (INJECT_REPORT_BEFORE_WRITE, RANDOM, {PUBLISH_BEFORE_LANDED}, None),
     (INJECT_CONSUMER_ENQUEUED_FIRST, RANDOM, {DEADLOCK}, False),
     (INJECT_OLD_EPOCH_CONSUMER, SERIAL, {FLAG_STALE_EPOCH}, None),          # polls meet the newer words
-    (INJECT_OLD_EPOCH_CONSUMER, CONSUMER_EAGER, {FLAG_NO_PRODUCER}, None),  # round 1 waits for an epoch nobody stores
+    (INJECT_OLD_EPOCH_CONSUMER, CONSUMER_EAGER, {FLAG_NO_PRODUCER}, None),  # the first dispatch + combine pair waits for an epoch nobody stores
 ])
 def test_each_planted_mistake_is_reported(inject, scheduler, expect, wrong_tokens):
     events, findings, wrong = run(100, 128, 8, 2, scheduler=scheduler, inject=inject, budget=60, rounds=2, seed=5)

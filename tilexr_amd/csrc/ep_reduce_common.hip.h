@@ -256,9 +256,9 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
     } else {
         if (a.flagsSettled != 0) {
             // No barrier of the kind that waits for memory after the rows have been stored: a workgroup that has to see
-            // its stores complete before it may leave stays a store round trip longer (2048-byte fp8 rows: 53 instead of
-            // 43 us).  The verdict on the tile words goes through LDS, two slots taken in turn so that the reset of one
-            // is a whole iteration away from its last readers.
+            // its stores complete before it may leave stays a store round trip longer (2048-byte fp8 rows: 53 us with
+            // such a barrier, 50 without).  What the tile words said goes through LDS, two slots taken in turn so that
+            // the reset of one is a whole iteration away from its last readers.
             __shared__ int s_missing[2];
             int turn = 0;
             for (int group = blockIdx.x; group < groups; group += gridDim.x, turn ^= 1) {
@@ -268,7 +268,7 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
                 __syncthreads();
                 const bool missing = load(group, kRouteSettled);
                 LdsBarrier();                       // the tile words are still on their way: nothing waits for them here
-                // the verdict is handed over between the last use of the rows and the first store: whoever asks for the
+                // what they said is handed over between the last use of the rows and the first store: whoever asks for the
                 // tile word there finds it long since arrived (it was requested ahead of the rows), and the barrier
                 // below does not wait for the stores
                 unit(group, [&] {
