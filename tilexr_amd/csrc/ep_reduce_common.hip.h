@@ -295,20 +295,30 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
         for (int base = 0; base < mine; base += 32) {
             const int inWindow = mine - base < 32 ? mine - base : 32;
             uint32_t pending = inWindow == 32 ? 0xffffffffu : ((1u << inWindow) - 1u);
-            for (uint32_t m = pending; m != 0u; m &= m - 1u) {
-                const int i = __builtin_ctz(m);
-                const int group = first + (base + i) * stride;
-                __syncthreads();
-                const bool waiting = load(group, kRouteCheck);
-                if (__syncthreads_or(waiting ? 1 : 0) != 0) {
-                    continue;                       // uniform: every lane gets the same answer
-                }
-                unit(group, [] {});
-                pending &= ~(1u << i);
-            }
+            // One loop body does the work of all three stages, so that the code of `unit` exists once: `todo` holds
+            // the groups to try now, `mode` says how (first pass: look once; after a scan: trusted; giving up).
+            uint32_t todo = pending;
+            int mode = kRouteCheck;
             uint64_t idleSince = wall_clock64();
             int backoff = 0;
             while (pending != 0u) {
+                for (; todo != 0u; todo &= todo - 1u) {
+                    const int i = __builtin_ctz(todo);
+                    const int group = first + (base + i) * stride;
+                    __syncthreads();
+                    const bool waiting = load(group, mode);
+                    if (__syncthreads_or((mode == kRouteCheck && waiting) ? 1 : 0) != 0) {
+                        continue;                       // uniform: every lane gets the same answer
+                    }
+                    unit(group, [] {});
+                    pending &= ~(1u << i);
+                    idleSince = wall_clock64();
+                    backoff = 0;
+                }
+                if (pending == 0u || mode == kRouteGiveUp) {
+                    break;
+                }
+                // all lanes together look once at every tile the pending groups need
                 if (threadIdx.x == 0) {
                     s_notReady = 0u;
                 }
@@ -328,42 +338,26 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
                     }
                 }
                 __syncthreads();
-                const uint32_t ready = pending & ~s_notReady;
-                if (ready == 0u) {
-                    bool stop = false;
-                    if (threadIdx.x == 0) {
-                        stop = static_cast<int64_t>(wall_clock64() - idleSince) > a.waitTimeoutTicks ||
-                            (a.deviceStatus != nullptr &&
-                             __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0);
-                    }
-                    if (__syncthreads_or(stop ? 1 : 0) != 0) {
-                        for (uint32_t m = pending; m != 0u; m &= m - 1u) {
-                            const int group = first + (base + __builtin_ctz(m)) * stride;
-                            __syncthreads();
-                            load(group, kRouteGiveUp);
-                            __syncthreads();
-                            unit(group, [] {});
-                        }
-                        pending = 0u;
-                        break;
-                    }
-                    for (int r = 0; r < (1 << backoff); ++r) {
-                        __builtin_amdgcn_s_sleep(127);      // 127 x 64 clocks, about 3.5 us
-                    }
-                    backoff += backoff < 2 ? 1 : 0;
+                todo = pending & ~s_notReady;
+                mode = kRouteTrusted;
+                if (todo != 0u) {
                     continue;
                 }
-                for (uint32_t m = ready; m != 0u; m &= m - 1u) {
-                    const int i = __builtin_ctz(m);
-                    const int group = first + (base + i) * stride;
-                    __syncthreads();
-                    load(group, kRouteTrusted);
-                    __syncthreads();
-                    unit(group, [] {});
-                    pending &= ~(1u << i);
+                bool stop = false;
+                if (threadIdx.x == 0) {
+                    stop = static_cast<int64_t>(wall_clock64() - idleSince) > a.waitTimeoutTicks ||
+                        (a.deviceStatus != nullptr &&
+                         __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0);
                 }
-                idleSince = wall_clock64();
-                backoff = 0;
+                if (__syncthreads_or(stop ? 1 : 0) != 0) {
+                    todo = pending;                     // the rest is given up: rows of zeros, status word set
+                    mode = kRouteGiveUp;
+                    continue;
+                }
+                for (int r = 0; r < (1 << backoff); ++r) {
+                    __builtin_amdgcn_s_sleep(127);      // 127 x 64 clocks, about 3.5 us
+                }
+                backoff += backoff < 2 ? 1 : 0;
             }
         }
     }
