@@ -1,0 +1,29 @@
+"""The library from a plain C++ program: tests/cxx/demo.cpp is written like the reference's own demo
+(tests/ep/demo/tilexr_ep_dispatch_demo.cpp: allocate with the runtime, dispatch, identity expert, combine, compare with
+a host model), includes nothing but include/*.h and the HIP runtime, and links libtilexr-ep.so.  No Python object and no
+torch tensor is involved in the run; this test only starts the program and reads its verdict.
+"""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+DEMO = os.path.join(ROOT, "tests", "cxx", "bin", "demo")
+
+
+@pytest.mark.parametrize("bs,h,top_k,experts", [
+    (128, 7168, 8, 256),        # decode-sized: the single-launch dispatch
+    (1536, 7168, 8, 256),       # count + per-route scatter, sliced reduce
+    (777, 1000, 3, 10),         # odd sizes: element-granular kernels (rows of 2000 bytes are not 16-byte multiples)
+    (4096, 2048, 4, 64),        # narrow rows: a wave per token
+])
+def test_cxx_demo(bs, h, top_k, experts):
+    if not os.path.exists(DEMO):
+        pytest.fail(f"{DEMO} is missing: build it with `make -C tilexr_amd/csrc` (or __graft_entry__.build())")
+    print(f"cxx demo bs={bs} h={h} top_k={top_k} experts={experts}", flush=True)
+    run = subprocess.run([DEMO, str(bs), str(h), str(top_k), str(experts)], capture_output=True, text=True, timeout=100)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert run.stdout.startswith("OK "), run.stdout
