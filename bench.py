@@ -698,10 +698,13 @@ def main():
         torch.cuda.synchronize()
         epoch_counter = [1 << 20]
 
+        stagger = [0]
+
         def producer():
             epoch_counter[0] += 1
             ep.check(ep.tile_producer_probe(expand_x, expert_out, kept_rows, row_bytes, stage_flags, stage_tile_rows,
-                                            epoch_counter[0], args.stage_workgroups, args.stage_tile_ns, stream), "producer")
+                                            epoch_counter[0], args.stage_workgroups, args.stage_tile_ns, stream,
+                                            stagger_ns=stagger[0]), "producer")
             return epoch_counter[0]
 
         def stage_alone():
@@ -734,22 +737,37 @@ def main():
             return (time.perf_counter() - t1) / n * 1e6
 
         n_stage = max(10, args.steps // 4)
-        alone_us = timed(stage_alone, n_stage)
-        serial_us = timed(stage_then_combine, n_stage)
-        y_serial = y.clone()
-        beside_us = timed(stage_beside_combine, n_stage)
-        if status.item() != 0:
-            print("a tile-flag wait expired during the expert-stage leg", file=sys.stderr)
-            sys.exit(1)
-        if not torch.equal(y.view(torch.int16), y_serial.view(torch.int16)):
-            print("combine beside the producer differs from combine after it", file=sys.stderr)
-            sys.exit(1)
+
+        def three_ways():
+            alone = timed(stage_alone, n_stage)
+            serial = timed(stage_then_combine, n_stage)
+            y_serial = y.clone()
+            beside = timed(stage_beside_combine, n_stage)
+            if status.item() != 0:
+                print("a tile-flag wait expired during the expert-stage leg", file=sys.stderr)
+                sys.exit(1)
+            if not torch.equal(y.view(torch.int16), y_serial.view(torch.int16)):
+                print("combine beside the producer differs from combine after it", file=sys.stderr)
+                sys.exit(1)
+            return alone, serial, beside
+
+        alone_us, serial_us, beside_us = three_ways()
+        # the same producer with workgroups that do not move in step: tiles complete at a steady rate instead of
+        # `workgroups` at a time, so the combine is not left with a last wave of tiles to follow
+        stagger[0] = args.stage_tile_ns
+        st_alone_us, st_serial_us, st_beside_us = three_ways()
+        stagger[0] = 0
         expert_stage = {"producer": f"{args.stage_workgroups} workgroups copy expandX to expertOut tile by tile, at least "
                                     f"{args.stage_tile_ns} ns per tile, publish each tile (release at agent scope + flag word)",
                         "tile_rows": stage_tile_rows, "steps": n_stage, "producer_alone_us": round(alone_us, 2),
                         "combine_after_producer_us": round(serial_us, 2), "combine_beside_producer_us": round(beside_us, 2),
-                        "saved_us": round(serial_us - beside_us, 2), "outputs_identical": True}
-        del expert_out, y_serial
+                        "saved_us": round(serial_us - beside_us, 2),
+                        "staggered_workgroups": {"producer_alone_us": round(st_alone_us, 2),
+                                                 "combine_after_producer_us": round(st_serial_us, 2),
+                                                 "combine_beside_producer_us": round(st_beside_us, 2),
+                                                 "saved_us": round(st_serial_us - st_beside_us, 2)},
+                        "outputs_identical": True}
+        del expert_out
 
     # the serial schedule once more with the token rows of every step in a different tensor, enough of them that none
     # is still in the 256 MiB memory-side cache when its turn comes again: what a caller sees whose x was produced long

@@ -272,12 +272,14 @@ int TileXREpMemoryProbe(int pattern, const void *src, void *dst, int64_t bytes, 
 // Measurement aid without a reference counterpart: a stand-in for an expert stage between dispatch and combine, so
 // that a harness can time (and a test can check) a combine that follows a producer which is slower than memory and
 // publishes tiles as it goes.  `workgroups` workgroups copy rows [0, rows) of `rowBytes` bytes (a multiple of 16) from
-// `src` to `dst`, tile by tile (workgroup w takes tiles w, w + workgroups, ...), spend at least `minTileNs` on a tile,
+// `src` to `dst`, tile by tile (workgroup w takes tiles w, w + workgroups, ...), spend at least `minTileNs` on a tile
+// (workgroup w starting w * staggerNs / workgroups late: with staggerNs = minTileNs tiles complete at a steady rate
+// instead of `workgroups` at a time),
 // and publish it the way any producer outside this library has to: rows complete, one release at agent scope, then
 // tileFlags[tile] = (epoch << 32) | rows in the tile.  `rows` is a host value (the kept rows of the dispatch).
 // Asynchronous on `stream`; returns 0, -3 for bad arguments, -2 when the launch fails.
 int TileXREpTileProducerProbe(const void *src, void *dst, int64_t rows, int64_t rowBytes, uint64_t *tileFlags,
-    int64_t tileRows, int64_t epoch, int64_t workgroups, int64_t minTileNs, aclrtStream stream);
+    int64_t tileRows, int64_t epoch, int64_t workgroups, int64_t minTileNs, int64_t staggerNs, aclrtStream stream);
 
 #pragma GCC visibility pop
 }

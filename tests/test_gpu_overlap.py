@@ -309,8 +309,9 @@ def test_combine_beside_a_slow_producer_that_publishes_tiles_as_it_goes(shape, t
             torch.cuda.synchronize()
             print(f"slow producer: shape {shape} tile_rows {tile_rows} epoch {epoch}", flush=True)
             # producer first: a waiting kernel enqueued ahead of it on a shared hardware queue would keep it out
+            # (the second run with workgroups that do not move in step: tiles complete at a steady rate)
             assert ep.tile_producer_probe(out["expand_x"], expert_out, rows, h * 2, flags, tile_rows, epoch, workgroups,
-                                          tile_ns, s.stream) == 0
+                                          tile_ns, s.stream, stagger_ns=tile_ns if epoch == 12 else 0) == 0
             st = ep.combine_memory_ex(expert_out, out["assist"], counts, s.comm, bs, h, K, E, y, ep.DT_BF16, side,
                                       expert_scales=d_w, row_index_map=out["row_map"], tile_flags=flags,
                                       tile_rows=tile_rows, flag_epoch=epoch, wait_timeout_us=10_000_000,
@@ -329,6 +330,8 @@ def test_combine_beside_a_slow_producer_that_publishes_tiles_as_it_goes(shape, t
         assert ep.tile_producer_probe(expert_out, expert_out, 0, 64, flags, 8, 1, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
         assert ep.tile_producer_probe(expert_out, expert_out, 8, 24, flags, 8, 1, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
         assert ep.tile_producer_probe(expert_out, expert_out, 8, 64, flags, 8, 0, 4, 0, s.stream) == ep.ERR_PARA_CHECK_FAIL
+        assert ep.tile_producer_probe(expert_out, expert_out, 8, 64, flags, 8, 1, 4, 0, s.stream,
+                                      stagger_ns=-1) == ep.ERR_PARA_CHECK_FAIL
 
 
 def test_flag_protocol_on_randomised_rounds():
@@ -402,7 +405,8 @@ def test_flag_protocol_on_randomised_rounds():
                 # the stand-in's stream order puts every flag of it after the dispatch)
                 s.sync()
                 assert ep.tile_producer_probe(expand_x, expert_out, n, row_bytes, stage_flags, tile_rows, 1000 + round_,
-                                              int(rng.choice([8, 64, 200])), int(rng.choice([0, 3000])), s.stream) == 0
+                                              int(rng.choice([8, 64, 200])), int(rng.choice([0, 3000])), s.stream,
+                                              stagger_ns=int(rng.choice([0, 3000]))) == 0
                 rows_in, use_flags, use_epoch, consumer = expert_out, stage_flags, 1000 + round_, side
             st = ep.combine_memory_ex(rows_in, assist, counts, s.comm, bs, h, K, E, y, ep.DT_BF16, consumer,
                                       expert_out_quant_mode=qmode, expert_out_scales=scales, expert_scales=d_w,

@@ -159,9 +159,17 @@ __global__ __launch_bounds__(kWave) void ep_probe_gather_narrow_kernel(const u32
 // with a release fence at agent scope and stores the word.  One such fence per tile of tens of rows is cheap; one per row
 // is not (the scatter kernels therefore write rows through instead).
 __global__ __launch_bounds__(kThreads) void ep_probe_tile_producer_kernel(const char *src, char *dst, int rows,
-    int64_t rowBytes, uint64_t *tileFlags, int tileRows, uint64_t epoch, int64_t minTileTicks)
+    int64_t rowBytes, uint64_t *tileFlags, int tileRows, uint64_t epoch, int64_t minTileTicks, int64_t staggerTicks)
 {
     const int tiles = (rows + tileRows - 1) / tileRows;
+    if (staggerTicks > 0) {
+        // workgroups that do not move in step: workgroup w starts w / gridDim.x of the stagger late
+        const uint64_t launch = wall_clock64();
+        const int64_t late = staggerTicks * static_cast<int64_t>(blockIdx.x) / static_cast<int64_t>(gridDim.x);
+        while (static_cast<int64_t>(wall_clock64() - launch) < late) {
+            __builtin_amdgcn_s_sleep(32);
+        }
+    }
     const int64_t vecsPerRow = rowBytes / 16;
     for (int tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
         const uint64_t begin = wall_clock64();
@@ -203,19 +211,19 @@ __global__ __launch_bounds__(kThreads) void ep_probe_tile_producer_kernel(const 
 } // namespace TileXREp
 
 extern "C" int TileXREpTileProducerProbe(const void *src, void *dst, int64_t rows, int64_t rowBytes, uint64_t *tileFlags,
-    int64_t tileRows, int64_t epoch, int64_t workgroups, int64_t minTileNs, aclrtStream stream)
+    int64_t tileRows, int64_t epoch, int64_t workgroups, int64_t minTileNs, int64_t staggerNs, aclrtStream stream)
 {
     using namespace TileXREp;
     if (src == nullptr || dst == nullptr || tileFlags == nullptr || stream == nullptr || !Aligned16(src) || !Aligned16(dst) ||
         rows <= 0 || rows > 0x7fffffff || rowBytes <= 0 || rowBytes % 16 != 0 || tileRows <= 0 || tileRows > 0x7fffffff ||
         epoch <= 0 || epoch > 0xffffffffll || workgroups <= 0 || workgroups > 65535 || minTileNs < 0 ||
-        minTileNs > 1000000000ll) {
+        minTileNs > 1000000000ll || staggerNs < 0 || staggerNs > 1000000000ll) {
         return TileXR::TILEXR_ERROR_PARA_CHECK_FAIL;
     }
     const int64_t ticks = minTileNs / 10;       // wall_clock64() counts at 100 MHz
     hipLaunchKernelGGL(ep_probe_tile_producer_kernel, dim3(static_cast<unsigned>(workgroups)), dim3(kThreads), 0,
         static_cast<hipStream_t>(stream), static_cast<const char *>(src), static_cast<char *>(dst), static_cast<int>(rows),
-        rowBytes, tileFlags, static_cast<int>(tileRows), static_cast<uint64_t>(epoch), ticks);
+        rowBytes, tileFlags, static_cast<int>(tileRows), static_cast<uint64_t>(epoch), ticks, staggerNs / 10);
     return hipGetLastError() == hipSuccess ? TileXR::TILEXR_SUCCESS : TileXR::TILEXR_ERROR_MKIRT;
 }
 

@@ -297,14 +297,15 @@ def memory_probe(pattern, src, dst, nbytes, stream):
     return fn(pattern, _ptr(src), _ptr(dst), int(nbytes), _stream(stream))
 
 
-def tile_producer_probe(src, dst, rows, row_bytes, tile_flags, tile_rows, epoch, workgroups, min_tile_ns, stream):
+def tile_producer_probe(src, dst, rows, row_bytes, tile_flags, tile_rows, epoch, workgroups, min_tile_ns, stream,
+                        stagger_ns=0):
     """A stand-in for an expert stage: copies rows src -> dst tile by tile at a set pace and publishes each tile's
     readiness word (see tilexr_ep.h)."""
     fn = lib().TileXREpTileProducerProbe
     fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
-                   C.c_void_p]
+                   C.c_int64, C.c_void_p]
     return fn(_ptr(src), _ptr(dst), int(rows), int(row_bytes), _ptr(tile_flags), int(tile_rows), int(epoch),
-              int(workgroups), int(min_tile_ns), _stream(stream))
+              int(workgroups), int(min_tile_ns), int(stagger_ns), _stream(stream))
 
 
 class DebugOptions(C.Structure):
