@@ -172,12 +172,13 @@ __global__ __launch_bounds__(THREADS) void ep_scatter_route_kernel(ScatterArgs a
 {
     constexpr int kXcds = 8;
     __shared__ int s_row;
-    const int xcd = blockIdx.x % kXcds;
-    const int j = blockIdx.x / kXcds;
-    const int perToken = a.topK * a.colSlices;
-    const int token = (j / perToken) * kXcds + xcd;
-    const int k = (j % perToken) / a.colSlices;
-    const int colBase = ((j % perToken) % a.colSlices) * (V * THREADS);
+    // grid = (8 * slices, topK, groups of eight tokens): the hardware hands out the three indices, so no workgroup
+    // starts with a division (this kernel runs at the rate its resident workgroups allow: a prologue of sixty scalar
+    // instructions ahead of the first load was a tenth of a workgroup's life).  Workgroups are dealt to the XCDs in
+    // linear order, x fastest, and gridDim.x is a multiple of eight: the XCD is blockIdx.x % 8.
+    const int token = static_cast<int>(blockIdx.z) * kXcds + static_cast<int>(blockIdx.x % kXcds);
+    const int k = blockIdx.y;
+    const int colBase = static_cast<int>(blockIdx.x / kXcds) * (V * THREADS);
     if (token >= a.bs) {
         return;
     }
@@ -482,7 +483,8 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
         case TILEXR_EP_QUANT_NONE:
             // small batches are latency-bound and gain nothing from the extra workgroups
             if (G == kThreads && ScatterCopiesPerRoute(l.x, l.out, l.bs, l.h, l.topK, l.quantMode)) {
-                const dim3 blocks(static_cast<unsigned>(static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK * a.colSlices));
+                const dim3 blocks(static_cast<unsigned>(8 * a.colSlices), static_cast<unsigned>(a.topK),
+                    static_cast<unsigned>((a.bs + 7) / 8));
                 if (l.kernelNameOut != nullptr) {
                     *l.kernelNameOut = "ep_scatter_route_kernel";
                 }
@@ -496,7 +498,8 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
                     constexpr int kWide = 2 * kThreads;
                     ScatterArgs wide = a;
                     wide.colSlices = (a.h / 8 + kRouteVecs * kWide - 1) / (kRouteVecs * kWide);
-                    const dim3 wideBlocks(static_cast<unsigned>(static_cast<int64_t>((a.bs + 7) / 8) * 8 * a.topK * wide.colSlices));
+                    const dim3 wideBlocks(static_cast<unsigned>(8 * wide.colSlices), static_cast<unsigned>(a.topK),
+                        static_cast<unsigned>((a.bs + 7) / 8));
                     hipLaunchKernelGGL((ep_scatter_route_kernel<kWide, kRouteVecs, true>), wideBlocks, dim3(kWide), 0,
                         l.stream, wide);
                 } else if (WriteThrough(a)) {
@@ -550,11 +553,10 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
 bool ScatterCopiesPerRoute(const void *x, const void *out, int64_t bs, int64_t h, int64_t topK, int quantMode)
 {
     const int64_t vecs = h / 8;
-    const int64_t slices = (vecs + kRouteVecs * kThreads - 1) / (kRouteVecs * kThreads);
     // token rows beyond half the memory-side cache (256 MiB) cannot be kept close by: the per-token kernel takes those
     return quantMode == TILEXR_EP_QUANT_NONE && h % 8 == 0 && Aligned16(x) && Aligned16(out) && vecs > 4 * kWave &&
         vecs <= 8 * kThreads && topK > 1 && bs >= 1024 && bs * h * 2 <= (int64_t{128} << 20) &&
-        (bs + 7) / 8 * 8 * topK * slices <= 0x7fffffff;
+        (bs + 7) / 8 <= 65535 && topK <= 65535;
 }
 
 hipError_t LaunchScatter(const ScatterLaunch &l)
