@@ -9,6 +9,7 @@ for the dominant kernel (timed with HIP events around that kernel on the stream 
 timed on this box's host cores as a baseline.
 """
 import argparse
+import ctypes
 import json
 import os
 import sys
@@ -143,6 +144,25 @@ def measured_ceilings(ep, torch, stream, dev, reps=10, narrow=None):
             us = a.elapsed_ms(b) * 1e3 / reps
             rate = round(moved[name] / (us * 1e-6) / 1e9, 1)
             out[name + "_GBps"] = max(rate, out.get(name + "_GBps", 0.0))
+        if mib == sizes[0]:
+            # the runtime's own device-to-device copy, as a yardstick that owes nothing to this library's kernels
+            hip = ctypes.CDLL("libamdhip64.so")
+            hip.hipMemcpyDtoDAsync.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+            raw = ctypes.c_void_p(stream.cuda_stream)
+
+            def runtime_copy():
+                if hip.hipMemcpyDtoDAsync(dst.data_ptr(), src.data_ptr(), nbytes, raw) != 0:
+                    raise RuntimeError("hipMemcpyDtoDAsync failed")
+
+            for _ in range(3):
+                runtime_copy()
+            a, b = ep.HipEvent(timing=True), ep.HipEvent(timing=True)
+            a.record(stream)
+            for _ in range(reps):
+                runtime_copy()
+            b.record(stream)
+            stream.synchronize()
+            out["hipMemcpyDtoD_GBps"] = round(2 * nbytes / (a.elapsed_ms(b) * 1e-3 / reps) / 1e9, 1)
         del src, dst
     if narrow is not None:
         # the quantised reduce's mix with its addresses: rows of 2048 (4096) one-byte payloads, eight (six) per output
