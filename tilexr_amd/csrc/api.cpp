@@ -278,6 +278,16 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     red.flagEpoch = static_cast<uint64_t>(p.flagEpoch) & 0xffffffffull;
     red.producerOrdered = p.tileFlags != nullptr && p.tileFlags == comm->lastFlagWords &&
         red.flagEpoch == comm->lastFlagEpoch && stream == comm->lastFlagStream;
+    if (red.tileFlags != nullptr && !red.producerOrdered) {
+        // a launch that may wait: its workgroups claim their tokens from a shared counter (see ForEachGroup)
+        if (!comm->claimWord.Reserve(256, true)) {
+            return TileXR::TILEXR_ERROR_INTERNAL;
+        }
+        if (ClearScratchWord(comm->claimWord.ptr, stream) != hipSuccess) {
+            return TileXR::TILEXR_ERROR_MKIRT;
+        }
+        red.claimWord = static_cast<uint32_t *>(comm->claimWord.ptr);
+    }
     red.waitTimeoutTicks = (p.waitTimeoutUs > 0 ? p.waitTimeoutUs : kDefaultWaitUs) * kWallClockTicksPerUs;
     red.deviceStatus = p.deviceStatusOut;
     red.numComputeUnits = comm->world->numComputeUnits;

@@ -194,6 +194,7 @@ int TileXRCommDestroy(TileXRCommPtr comm)
     }
     c->dispatchScratch.Release();
     c->combineScratch.Release();
+    c->claimWord.Release();
     c->drainScratch.Release();
     c->tileCounters.Release();
     if (c->dev != nullptr) {

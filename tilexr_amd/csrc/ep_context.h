@@ -115,6 +115,7 @@ struct EpComm {
     std::atomic<int64_t> nextMagic {1};
     DeviceBuffer dispatchScratch;
     DeviceBuffer combineScratch;
+    DeviceBuffer claimWord;           // token claims of a combine that waits on readiness flags
     DeviceBuffer drainScratch;
     DeviceBuffer tileCounters;        // rows landed per readiness tile; all zero whenever no dispatch is in flight
     // The last dispatch of this communicator that published readiness flags: a combine on the same stream that waits for

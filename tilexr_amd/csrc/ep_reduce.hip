@@ -159,6 +159,7 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     a.waitTimeoutTicks = l.waitTimeoutTicks;
     a.deviceStatus = l.deviceStatus;
     a.flagsSettled = (l.tileFlags != nullptr && l.producerOrdered) ? 1 : 0;
+    a.claim = l.claimWord;
     a.colSlices = 1;
     // A kernel that waits on flags must never crowd out the producer it waits for: its waiting waves keep their
     // registers, and with three or more of these workgroups per compute unit a producer workgroup no longer fits

@@ -40,6 +40,7 @@ struct ReduceArgs {
     int64_t waitTimeoutTicks;
     int32_t *deviceStatus;
     int flagsSettled;                // the producer of the flags finished before this launch began (same stream)
+    uint32_t *claim;                 // launches that may wait: zero at launch, the next group nobody has claimed yet
 };
 
 // Launchers of the register-resident kernels, one translation unit per (element type, with / without readiness flags).
@@ -287,24 +288,68 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
             }
             return;
         }
+        // Groups are claimed, a few at a time, from a counter all workgroups share, not owned by block index: a
+        // workgroup holds at most kHeld groups that are not ready yet, and whoever has nothing left to wait for takes
+        // the next ones.  With fixed ownership the tokens of a producer's last tiles were reduced by the few workgroups
+        // that happened to own them, one after the other, while the rest had gone home.  Without a counter (a.claim
+        // null) the groups are dealt by block index as before.
+        constexpr int kHeld = 4;
         __shared__ uint32_t s_notReady;
-        const int first = static_cast<int>(blockIdx.x);
-        const int stride = static_cast<int>(gridDim.x);
-        const int mine = groups > first ? (groups - 1 - first) / stride + 1 : 0;
+        __shared__ int s_group[kHeld];
+        __shared__ int s_base;
         const int perGroup = tokensPerGroup * a.slots;
-        for (int base = 0; base < mine; base += 32) {
-            const int inWindow = mine - base < 32 ? mine - base : 32;
-            uint32_t pending = inWindow == 32 ? 0xffffffffu : ((1u << inWindow) - 1u);
-            // One loop body does the work of all three stages, so that the code of `unit` exists once: `todo` holds
-            // the groups to try now, `mode` says how (first pass: look once; after a scan: trusted; giving up).
-            uint32_t todo = pending;
+        int dealt = static_cast<int>(blockIdx.x);       // next group by block index (no counter)
+        bool more = true;
+        uint32_t pending = 0u;                          // slots of s_group that hold a claimed, unfinished group
+        uint64_t idleSince = wall_clock64();
+        int backoff = 0;
+        for (;;) {
+            uint32_t fresh = 0u;
+            const uint32_t freeSlots = ~pending & ((1u << kHeld) - 1u);
+            if (more && freeSlots != 0u) {
+                const int want = __popc(freeSlots);
+                if (a.claim != nullptr) {
+                    __syncthreads();                    // readers of s_base from the previous refill are done
+                    if (threadIdx.x == 0) {
+                        s_base = static_cast<int>(__hip_atomic_fetch_add(a.claim, static_cast<uint32_t>(want), __ATOMIC_RELAXED,
+                            __HIP_MEMORY_SCOPE_AGENT));
+                    }
+                    __syncthreads();
+                }
+                int next = a.claim != nullptr ? s_base : 0;
+                for (uint32_t m = freeSlots; m != 0u; m &= m - 1u) {
+                    const int slot = __builtin_ctz(m);
+                    int group;
+                    if (a.claim != nullptr) {
+                        group = next++;
+                    } else {
+                        group = dealt;
+                        dealt += static_cast<int>(gridDim.x);
+                    }
+                    if (group >= groups || group < 0) {
+                        more = false;
+                        continue;
+                    }
+                    if (threadIdx.x == 0) {
+                        s_group[slot] = group;
+                    }
+                    fresh |= 1u << slot;
+                }
+                pending |= fresh;
+                __syncthreads();
+            }
+            if (pending == 0u) {
+                break;                                  // nothing held, nothing left to claim
+            }
+            // One loop body does the work of all stages, so that the code of `unit` exists once: `todo` holds the slots
+            // to try now, `mode` says how (a first look at fresh groups; after a scan: trusted; giving up).
+            uint32_t todo = fresh;
             int mode = kRouteCheck;
-            uint64_t idleSince = wall_clock64();
-            int backoff = 0;
-            while (pending != 0u) {
+            for (int pass = 0; pass < 2; ++pass) {
+                bool done = false;
                 for (; todo != 0u; todo &= todo - 1u) {
                     const int i = __builtin_ctz(todo);
-                    const int group = first + (base + i) * stride;
+                    const int group = s_group[i];
                     __syncthreads();
                     const bool waiting = load(group, mode);
                     if (__syncthreads_or((mode == kRouteCheck && waiting) ? 1 : 0) != 0) {
@@ -314,21 +359,22 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
                     pending &= ~(1u << i);
                     idleSince = wall_clock64();
                     backoff = 0;
+                    done = true;
                 }
-                if (pending == 0u || mode == kRouteGiveUp) {
-                    break;
+                if (pass == 1 || pending == 0u || (done && more)) {
+                    break;                              // free slots and groups to claim: refill before looking again
                 }
-                // all lanes together look once at every tile the pending groups need
+                // all lanes together look once at every tile the held groups need
                 if (threadIdx.x == 0) {
                     s_notReady = 0u;
                 }
                 __syncthreads();
-                for (int idx = threadIdx.x; idx < inWindow * perGroup; idx += blockDim.x) {
+                for (int idx = threadIdx.x; idx < kHeld * perGroup; idx += blockDim.x) {
                     const int i = idx / perGroup;
                     if (((pending >> i) & 1u) == 0u) {
                         continue;
                     }
-                    const int token = tokenAt(first + (base + i) * stride, (idx % perGroup) / a.slots);
+                    const int token = tokenAt(s_group[i], (idx % perGroup) / a.slots);
                     if (token < 0) {
                         continue;
                     }
@@ -350,7 +396,7 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
                          __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0);
                 }
                 if (__syncthreads_or(stop ? 1 : 0) != 0) {
-                    todo = pending;                     // the rest is given up: rows of zeros, status word set
+                    todo = pending;                     // what is held is given up: rows of zeros, status word set
                     mode = kRouteGiveUp;
                     continue;
                 }
@@ -358,6 +404,7 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
                     __builtin_amdgcn_s_sleep(127);      // 127 x 64 clocks, about 3.5 us
                 }
                 backoff += backoff < 2 ? 1 : 0;
+                break;
             }
         }
     }
