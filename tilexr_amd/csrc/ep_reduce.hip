@@ -155,6 +155,10 @@ hipError_t LaunchReduce(const ReduceLaunch &l)
     a.y = l.y;
     a.tileFlags = l.tileFlags;
     a.tileRows = static_cast<int>(l.tileRows);
+    a.tileShift = -1;
+    if (l.tileRows > 0 && (l.tileRows & (l.tileRows - 1)) == 0) {
+        a.tileShift = __builtin_ctzll(static_cast<unsigned long long>(l.tileRows));
+    }
     a.flagEpoch = l.flagEpoch;
     a.waitTimeoutTicks = l.waitTimeoutTicks;
     a.deviceStatus = l.deviceStatus;

@@ -36,6 +36,7 @@ struct ReduceArgs {
     int colSlices;                   // slices a row is cut into (vec kernel, wide rows), else 1
     const uint64_t *tileFlags;
     int tileRows;
+    int tileShift;                   // log2(tileRows) where that is a whole number, else -1
     uint64_t flagEpoch;
     int64_t waitTimeoutTicks;
     int32_t *deviceStatus;
@@ -71,6 +72,11 @@ __device__ __forceinline__ int LookupRow(const ReduceArgs &a, int64_t slot)
     return static_cast<unsigned>(row) < static_cast<unsigned>(a.maxRows) ? row : -1;
 }
 
+__device__ __forceinline__ int TileOf(const ReduceArgs &a, int row)
+{
+    return a.tileShift >= 0 ? (row >> a.tileShift) : (row / a.tileRows);
+}
+
 // Bounded wait until the tile holding `row` has been published for this epoch (its word carries the epoch).  The poll itself is a relaxed
 // device-scope load (no cache maintenance per iteration -- an acquire in the loop would invalidate this XCD's L2 on
 // every spin and starve the producer).  What the caller reads afterwards must not come from a stale L2 line: the
@@ -78,7 +84,7 @@ __device__ __forceinline__ int LookupRow(const ReduceArgs &a, int64_t slot)
 // element-granular kernel issues one acquire fence after all its waits have succeeded.
 __device__ inline bool WaitTile(const ReduceArgs &a, int row)
 {
-    const int tile = row / a.tileRows;
+    const int tile = TileOf(a, row);
     const uint64_t start = wall_clock64();
     // every poll is a round trip to memory (agent scope): the gap between polls doubles up to about 3 us
     int backoff = 0;
@@ -160,7 +166,7 @@ __device__ __forceinline__ float ScaleLoad(const float *p)
 // One look at the tile holding `row`: published for this epoch or not.
 __device__ __forceinline__ bool TilePublished(const ReduceArgs &a, int row)
 {
-    const uint64_t w = __hip_atomic_load(&a.tileFlags[row / a.tileRows], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint64_t w = __hip_atomic_load(&a.tileFlags[TileOf(a, row)], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return TileWordReady(w, a.flagEpoch);
 }
 
@@ -170,15 +176,11 @@ __device__ __forceinline__ bool TilePublished(const ReduceArgs &a, int row)
 //                  ("come back later")
 //   kRouteTrusted  nothing: the caller has just seen every tile of this token published
 //   kRouteGiveUp   look once; a tile that is not there turns the slot into an expired one
-//   kRouteSettled  the producer finished before this launch began, so nothing is waited for and no read can come too
-//                  early: the slot gets its row at once and the call returns whether the tile's word says otherwise,
-//                  a value the caller needs only after the rows have been read (the word travels beside the rows
-//                  instead of ahead of them: one dependent round trip less)
 // An expired wait sets the launch's status word and leaves kRowExpired in the slot: the token then gets a row of zeros
 // (AnyExpired), never the sum of the rows that happened to be ready.
 constexpr int kRowExpired = -2;
 constexpr int kRowPending = -3;
-enum RouteMode : int { kRouteCheck = 0, kRouteTrusted = 1, kRouteGiveUp = 2, kRouteSettled = 3 };
+enum RouteMode : int { kRouteCheck = 0, kRouteTrusted = 1, kRouteGiveUp = 2 };
 
 __device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
 {
@@ -189,6 +191,26 @@ __device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
     return expired;
 }
 
+// A launch whose producer finished before it began (flagsSettled) waits for nothing, but a tile word that does not
+// carry the launch's epoch still means that the rows of that tile were never written: the token gets a row of zeros and
+// the launch's status word is set, at once.  Lane k of a wave holds the row of slot k (-1: none).  The word is asked for
+// before the rows and looked at after the last of them has been used: the memory counter runs in order, so by then it
+// has long arrived, and nothing waits for it on the way (an ordinary load: the words are final, this XCD's L2 may keep
+// them).
+__device__ __forceinline__ uint64_t SettledWordLoad(const ReduceArgs &a, int slotRow)
+{
+    return slotRow >= 0 ? a.tileFlags[TileOf(a, slotRow)] : 0ull;
+}
+
+__device__ __forceinline__ bool SettledWordMissing(const ReduceArgs &a, int slotRow, uint64_t word, int waveLane)
+{
+    const bool missing = __ballot(slotRow >= 0 && !TileWordReady(word, a.flagEpoch)) != 0;
+    if (missing && waveLane == 0 && a.deviceStatus != nullptr) {
+        atomicExch(a.deviceStatus, 1);
+    }
+    return missing;
+}
+
 template <bool FENCE, bool BLOCK>
 __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
     float *weights, int mode)
@@ -197,8 +219,7 @@ __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool 
     for (int k = lane; k < a.slots; k += lanes) {
         const int64_t slot = static_cast<int64_t>(tokOk ? token : 0) * a.slots + k;
         int row = tokOk ? LookupRow(a, slot) : -1;
-        const bool settled = !BLOCK && mode == kRouteSettled;
-        if (!settled && row >= 0 && a.tileFlags != nullptr && (BLOCK || mode != kRouteTrusted)) {
+        if (row >= 0 && a.tileFlags != nullptr && (BLOCK || mode != kRouteTrusted)) {
             const bool there = BLOCK ? WaitTile(a, row) : TilePublished(a, row);
             if (!there && !BLOCK && mode == kRouteCheck) {
                 row = kRowPending;
@@ -215,12 +236,6 @@ __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool 
         // (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:650-657)
         weights[k] = (tokOk && a.expertScales != nullptr && k < a.topK) ?
             a.expertScales[static_cast<int64_t>(token) * a.topK + k] : 1.0f;
-        if (settled && row >= 0 && a.tileFlags != nullptr) {
-            // the last load of all: the memory counter runs in order, so nothing that is needed before the rows may
-            // come after it
-            // (an ordinary load: the words are final, this XCD's L2 may keep them)
-            pending |= !TileWordReady(a.tileFlags[row / a.tileRows], a.flagEpoch);
-        }
     }
     if (FENCE && a.tileFlags != nullptr && lane < a.slots) {
         // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
@@ -230,64 +245,36 @@ __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool 
     return pending;
 }
 
-// Runs unit(group, beforeStores) for this workgroup's groups: blockIdx.x, blockIdx.x + gridDim.x, ...  beforeStores is
-// a callable the unit invokes once, after its last load has been used and before its first store.  `load(group, mode)`
+// Runs unit(group) for this workgroup's groups: blockIdx.x, blockIdx.x + gridDim.x, ...  `load(group, mode)`
 // fills the workgroup's route tables for a group and returns (per lane) whether a tile it needs is not published yet;
 // `tokenAt(group, t)` names the t-th of a group's `tokensPerGroup` tokens (-1 = none).
 //
-// Without readiness flags that is a plain loop.  With them (WAITS) a workgroup never sits on one group while others it
-// owes are ready: a token needs the tiles of all its rows, which a producer that works tile by tile finishes at
-// unrelated times, so tokens become ready in no particular order.  The workgroup takes its groups 32 at a time.  A
-// first pass reduces every group whose tiles are there already (all of them when the producer ran earlier on the same
-// stream).  For what is left it then goes in rounds: all lanes together look once at every tile the pending groups need
-// (one round trip for the lot), the groups that have become complete are reduced, and a round without any is followed
-// by a sleep that grows to about 14 us.  When nothing it owes has become ready for the wait bound, or another workgroup
-// has reported an expired wait, the rest is given up: those tokens get rows of zeros and the launch's status word is set.
+// Without readiness flags, or with flags that were all published before the launch began, that is a plain loop.  A
+// launch that may have to wait (WAITS, flags not settled) never sits on one group while others are ready: a token needs
+// the tiles of all its rows, which a producer that works tile by tile finishes at unrelated times, so tokens become
+// ready in no particular order.  A workgroup holds a few groups at a time.  Fresh ones are looked at once and reduced
+// if their tiles are there.  For what is left it goes in rounds: all lanes together look once at every tile the held
+// groups need (one round trip for the lot), the groups that have become complete are reduced, and a round without any
+// is followed by a sleep that grows to about 14 us.  When nothing it holds has become ready for the wait bound, or
+// another workgroup has reported an expired wait, the rest is given up: those tokens get rows of zeros and the launch's
+// status word is set.
 template <bool WAITS, typename TokenAt, typename Load, typename Unit>
 __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, int tokensPerGroup, TokenAt tokenAt,
     Load load, Unit unit)
 {
-    if constexpr (!WAITS) {
+    const bool plainLoop = !WAITS || a.flagsSettled != 0;
+    if (plainLoop) {
+        // no flags, or flags that were all published before this launch began: the route tables trust every tile, and
+        // the kernel looks at the words itself, beside the rows (SettledWordLoad)
         for (int group = blockIdx.x; group < groups; group += gridDim.x) {
             __syncthreads();        // the previous iteration's readers are done with the route tables
             load(group, kRouteTrusted);
             __syncthreads();
-            unit(group, [] {});
+            unit(group);
         }
-    } else {
-        if (a.flagsSettled != 0) {
-            // No barrier of the kind that waits for memory after the rows have been stored: a workgroup that has to see
-            // its stores complete before it may leave stays a store round trip longer (2048-byte fp8 rows: 53 us with
-            // such a barrier, 50 without).  What the tile words said goes through LDS, two slots taken in turn so that
-            // the reset of one is a whole iteration away from its last readers.
-            __shared__ int s_missing[2];
-            int turn = 0;
-            for (int group = blockIdx.x; group < groups; group += gridDim.x, turn ^= 1) {
-                if (threadIdx.x == 0) {
-                    s_missing[turn] = 0;
-                }
-                __syncthreads();
-                const bool missing = load(group, kRouteSettled);
-                LdsBarrier();                       // the tile words are still on their way: nothing waits for them here
-                // what they said is handed over between the last use of the rows and the first store: whoever asks for the
-                // tile word there finds it long since arrived (it was requested ahead of the rows), and the barrier
-                // below does not wait for the stores
-                unit(group, [&] {
-                    if (missing) {
-                        s_missing[turn] = 1;
-                    }
-                });
-                LdsBarrier();
-                if (s_missing[turn] != 0) {
-                    // a word that is not there now never will be: the token gets a row of zeros and the status is set
-                    __syncthreads();
-                    load(group, kRouteGiveUp);
-                    __syncthreads();
-                    unit(group, [] {});
-                }
-            }
-            return;
-        }
+        return;
+    }
+    if constexpr (WAITS) {
         // Groups are claimed, a few at a time, from a counter all workgroups share, not owned by block index: a
         // workgroup holds at most kHeld groups that are not ready yet, and whoever has nothing left to wait for takes
         // the next ones.  With fixed ownership the tokens of a producer's last tiles were reduced by the few workgroups
@@ -355,7 +342,7 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
                     if (__syncthreads_or((mode == kRouteCheck && waiting) ? 1 : 0) != 0) {
                         continue;                       // uniform: every lane gets the same answer
                     }
-                    unit(group, [] {});
+                    unit(group);
                     pending &= ~(1u << i);
                     idleSince = wall_clock64();
                     backoff = 0;

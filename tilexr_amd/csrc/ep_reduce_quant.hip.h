@@ -15,7 +15,7 @@ namespace {
 // row (fp32, k order, separate multiply and add).  Rows are a quarter the bytes of bf16 rows, so a lane owns 16
 // consecutive columns per vector (one 16-byte load) and KB rows are kept in flight at once.
 template <int G, int V, int INQ, bool BF16, bool FL>
-__global__ __launch_bounds__(kThreads, (V == 1 && !FL && BF16) ? 7 : 1) void ep_reduce_quant_kernel(ReduceArgs a)
+__global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL && INQ == TILEXR_EP_QUANT_FP8_BLOCK128) ? 6 : 7) : 1) void ep_reduce_quant_kernel(ReduceArgs a)
 {
     constexpr int kTokens = kThreads / G;
     constexpr int KB = V >= 4 ? 2 : 4;
@@ -36,10 +36,26 @@ __global__ __launch_bounds__(kThreads, (V == 1 && !FL && BF16) ? 7 : 1) void ep_
         const int token = group * kTokens + tg;
         return LoadRoutes<false, false>(a, token, token < a.bs, lane, G, s_row[tg], s_w[tg], mode);
     };
-    auto reduceUnit = [&](int group, auto beforeStores) {
+    auto reduceUnit = [&](int group) {
         const int token = group * kTokens + tg;
         const bool tokOk = token < a.bs;
-        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !(FL && AnyExpired(s_row[tg], a.slots));
+        // Lane k of every wave keeps slot k's row and weight; the K loop takes the slots that have a row, in k order,
+        // KB at a time.  Where tokens lose rows to an expert's capacity that is often one trip to memory, not two
+        // (absent rows are skipped by the sum anyway, so the order of the additions is the same).
+        static_assert(G % kWave == 0, "a wave works on one token");
+        const int waveLane = threadIdx.x % kWave;
+        int slotRow = -1;
+        float myWeight = 0.0f;
+        if (waveLane < a.slots) {
+            slotRow = s_row[tg][waveLane];
+            myWeight = s_w[tg][waveLane];
+        }
+        const bool checkWords = FL && a.flagsSettled != 0;
+        const uint64_t tileWord = checkWords ? SettledWordLoad(a, slotRow) : 0ull;
+        const bool expired = FL && __ballot(slotRow == kRowExpired) != 0;
+        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !expired;
+        const int myRow = active ? slotRow : -1;
+        const uint64_t live = __ballot(myRow >= 0);
 
         float acc[V][16];
         // The K loop.  fp8 rows are decoded by the hardware convert alone, which differs from the reference decode in
@@ -60,15 +76,20 @@ __global__ __launch_bounds__(kThreads, (V == 1 && !FL && BF16) ? 7 : 1) void ep_
                     acc[j][e] = 0.0f;
                 }
             }
-            for (int k0 = 0; k0 < a.slots; k0 += KB) {
+            uint64_t todo = live;
+            while (todo != 0) {
                 u32x4 q[KB][V];
                 float sc[KB][V];
                 int rowOfK[KB];
+                float weightOfK[KB];
 #pragma unroll
                 for (int u = 0; u < KB; ++u) {
-                    const int k = k0 + u;
-                    const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
+                    const bool any = todo != 0;
+                    const int k = any ? __builtin_ctzll(todo) : 0;
+                    todo &= todo - 1;
+                    const int row = any ? __builtin_amdgcn_readlane(myRow, k) : -1;
                     rowOfK[u] = row;
+                    weightOfK[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myWeight), k));
                     // Bounds are the buffer resources' business: an absent row gets resources of zero bytes, so its loads, like
                     // those of the lanes past the end of a row, return zeros without a branch (and without the register
                     // clears a branch would need).
@@ -92,7 +113,7 @@ __global__ __launch_bounds__(kThreads, (V == 1 && !FL && BF16) ? 7 : 1) void ep_
                     if (rowOfK[u] < 0) {
                         continue;                       // uniform across the lanes of a token
                     }
-                    const float w = s_w[tg][k0 + u];
+                    const float w = weightOfK[u];
 #pragma unroll
                     for (int j = 0; j < V; ++j) {
 #pragma unroll
@@ -174,7 +195,7 @@ __global__ __launch_bounds__(kThreads, (V == 1 && !FL && BF16) ? 7 : 1) void ep_
                 }
             }
         }
-        beforeStores();
+        const bool keep = active && !(checkWords && SettledWordMissing(a, slotRow, tileWord, waveLane));
         if (tokOk) {
             u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.y) + static_cast<int64_t>(token) * a.h * 2);
 #pragma unroll
@@ -186,7 +207,7 @@ __global__ __launch_bounds__(kThreads, (V == 1 && !FL && BF16) ? 7 : 1) void ep_
                         u32x4 o;
 #pragma unroll
                         for (int q2 = 0; q2 < 4; ++q2) {
-                            o[q2] = active ? EncodePair16Sat<BF16>(acc[j][half * 8 + 2 * q2], acc[j][half * 8 + 2 * q2 + 1]) : 0u;
+                            o[q2] = keep ? EncodePair16Sat<BF16>(acc[j][half * 8 + 2 * q2], acc[j][half * 8 + 2 * q2 + 1]) : 0u;
                         }
                         // An ordinary store, not a streaming one: a lane's 32 bytes go out as two 16-byte stores, each
                         // of which fills every other 16 bytes of the lines it touches; the L2 puts the halves together

@@ -57,7 +57,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
         const int unit = group * unitsPerGroup + tg;
         return LoadRoutes<false, false>(a, unit / a.colSlices, unit < units, lane, G, s_row[tg], s_w[tg], mode);
     };
-    auto reduceUnit = [&](int group, auto beforeStores) {
+    auto reduceUnit = [&](int group) {
         const int unit = group * unitsPerGroup + tg;
         const bool tokOk = unit < units;
         const int token = unit / a.colSlices;
@@ -68,7 +68,22 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             }
             __syncthreads();
         }
-        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !(FL && AnyExpired(s_row[tg], a.slots));
+        // Lane k of every wave keeps slot k's row and weight (the lanes of a wave share one token); the K loop takes the
+        // slots that have a row, in k order, KB at a time, so a token that lost rows (capacity, masks) makes fewer trips
+        // to memory.  Absent rows are skipped by the sum anyway: the order of the additions is the same.
+        static_assert(G % kWave == 0, "a wave works on one token");
+        const int waveLane = threadIdx.x % kWave;
+        int slotRow = -1;
+        float myWeight = 0.0f;
+        if (waveLane < a.slots) {
+            slotRow = s_row[tg][waveLane];
+            myWeight = s_w[tg][waveLane];
+        }
+        const bool checkWords = FL && a.flagsSettled != 0;
+        const uint64_t tileWord = checkWords ? SettledWordLoad(a, slotRow) : 0ull;
+        const bool expired = FL && __ballot(slotRow == kRowExpired) != 0;
+        const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !expired;
+        const int myRow = active ? slotRow : -1;
 
         float acc[V][8];
 #pragma unroll
@@ -78,16 +93,20 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                 acc[j][e] = 0.0f;
             }
         }
+        uint64_t todo = __ballot(myRow >= 0);
         // control flow below is uniform across the lanes that share a token (the MXFP8 round trip shuffles)
-        for (int k0 = 0; k0 < a.slots; k0 += KB) {
+        while (todo != 0) {
             u32x4 v16[KB][V];
             int rowOfK[KB];
+            float weightOfK[KB];
 #pragma unroll
             for (int u = 0; u < KB; ++u) {
-                const int k = k0 + u;
-                // the lanes of a wave share one token, so the row is wave-uniform
-                const int row = __builtin_amdgcn_readfirstlane((k < a.slots && active) ? s_row[tg][k] : -1);
+                const bool any = todo != 0;
+                const int k = any ? __builtin_ctzll(todo) : 0;
+                todo &= todo - 1;
+                const int row = any ? __builtin_amdgcn_readlane(myRow, k) : -1;
                 rowOfK[u] = row;
+                weightOfK[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myWeight), k));
                 const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
                 const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
 #pragma unroll
@@ -101,7 +120,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                 if (rowOfK[u] < 0) {
                     continue;
                 }
-                const float w = s_w[tg][k0 + u];
+                const float w = weightOfK[u];
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
                     float f[8];
@@ -156,7 +175,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                 }
             }
         }
-        beforeStores();
+        const bool keep = active && !(checkWords && SettledWordMissing(a, slotRow, tileWord, waveLane));
         if (tokOk) {
             u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.y) + static_cast<int64_t>(token) * a.h * 2);
 #pragma unroll
@@ -166,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                     u32x4 o;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
-                        o[q] = active ? EncodePair16Sat<BF16>(acc[j][2 * q], acc[j][2 * q + 1]) : 0u;
+                        o[q] = keep ? EncodePair16Sat<BF16>(acc[j][2 * q], acc[j][2 * q + 1]) : 0u;
                     }
                     __builtin_nontemporal_store(o, dst + idx);
                 }
