@@ -93,7 +93,8 @@ __device__ inline bool WaitTile(const ReduceArgs &a, int row)
         if (TileWordReady(w, a.flagEpoch)) {
             return true;
         }
-        if (static_cast<int64_t>(wall_clock64() - start) > a.waitTimeoutTicks) {
+        // a producer that finished before this launch began has nothing more to publish
+        if (a.flagsSettled != 0 || static_cast<int64_t>(wall_clock64() - start) > a.waitTimeoutTicks) {
             return false;
         }
         // once one wait of the launch has expired the producer is taken to be gone: later waits give up at once,
