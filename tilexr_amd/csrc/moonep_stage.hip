@@ -161,11 +161,38 @@ __device__ __forceinline__ bool SourceWrites(const Route &r, uint8_t direct, uin
     return false;
 }
 
+// Reads 8 KiB of the token rows of source rank blockIdx.y (two 16-byte loads per lane) and drops them, ahead of the
+// per-route scatter.  That kernel is the fastest copy only while the token rows are in the memory-side cache: when its
+// one reading workgroup in K has to fetch a row from HBM between the writes of the others it runs at little more than
+// half its speed.  After this read it finds the rows in that cache whatever their history.
+constexpr int kWarmLoads = 2;
+__device__ __forceinline__ void WarmRows(const DispatchWorld &a, int64_t block, int64_t vecs)
+{
+    const u32x4 *rows = static_cast<const u32x4 *>(a.hiddenSh[blockIdx.y]);
+    const int64_t base = block * (kThreads * kWarmLoads) + threadIdx.x;
+    u32x4 v[kWarmLoads];
+#pragma unroll
+    for (int i = 0; i < kWarmLoads; ++i) {
+        const int64_t at = base + static_cast<int64_t>(i) * kThreads;
+        v[i] = rows[at < vecs ? at : vecs - 1];
+    }
+#pragma unroll
+    for (int i = 0; i < kWarmLoads; ++i) {
+        asm volatile("" ::"v"(v[i]));
+    }
+}
+
 // Saved plans, one thread per route of source rank blockIdx.y: whether the source may write a duplicate's row itself
 // (see SourceWrites).  Done ahead of the scatter so that its workgroups find the answer with the route word, in one
-// round trip, instead of looking up the parent record after decoding it.
-__global__ __launch_bounds__(kThreads) void moon_agree_kernel(DispatchWorld a)
+// round trip, instead of looking up the parent record after decoding it.  The workgroups from `routeBlocks` on read the
+// token rows ahead (WarmRows) when warmVecs is not zero: this launch waits on a few small loads and leaves the memory
+// system idle, so the read costs a saved-plan Dispatch no launch of its own.
+__global__ __launch_bounds__(kThreads) void moon_agree_kernel(DispatchWorld a, unsigned routeBlocks, int64_t warmVecs)
 {
+    if (blockIdx.x >= routeBlocks) {
+        WarmRows(a, static_cast<int64_t>(blockIdx.x - routeBlocks), warmVecs);
+        return;
+    }
     const int src = blockIdx.y;
     const int64_t route = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
     if (route >= a.s * a.k) {
@@ -183,25 +210,10 @@ __global__ __launch_bounds__(kThreads) void moon_agree_kernel(DispatchWorld a)
     a.tables.direct[static_cast<int64_t>(src) * a.tables.stride + route] = direct;
 }
 
-// Reads the token rows of source rank blockIdx.y once (8 KiB per workgroup) and drops them, ahead of the per-route
-// scatter.  That kernel is the fastest copy only while the token rows are in the memory-side cache: when its one reading
-// workgroup in K has to fetch a row from HBM between the writes of the others it runs at little more than half its
-// speed.  After this read it finds the rows in that cache whatever their history.
-constexpr int kWarmLoads = 2;
+// The same read as a launch of its own, for a Dispatch that builds its plan: nothing runs ahead of its scatter.
 __global__ __launch_bounds__(kThreads) void moon_warm_rows_kernel(DispatchWorld a, int64_t vecs)
 {
-    const u32x4 *rows = static_cast<const u32x4 *>(a.hiddenSh[blockIdx.y]);
-    const int64_t base = static_cast<int64_t>(blockIdx.x) * (kThreads * kWarmLoads) + threadIdx.x;
-    u32x4 v[kWarmLoads];
-#pragma unroll
-    for (int i = 0; i < kWarmLoads; ++i) {
-        const int64_t at = base + static_cast<int64_t>(i) * kThreads;
-        v[i] = rows[at < vecs ? at : vecs - 1];
-    }
-#pragma unroll
-    for (int i = 0; i < kWarmLoads; ++i) {
-        asm volatile("" ::"v"(v[i]));
-    }
+    WarmRows(a, static_cast<int64_t>(blockIdx.x), vecs);
 }
 
 // One workgroup per (token, route, slice of 512 vectors) of source rank blockIdx.y.
@@ -1050,13 +1062,6 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
 {
     const unsigned R = static_cast<unsigned>(w.world);
     const unsigned rowBlocks = static_cast<unsigned>((w.nvS + kThreads - 1) / kThreads);
-    if (!w.fresh) {
-        hipLaunchKernelGGL(moon_group_walk_kernel, dim3(rowBlocks, R), dim3(kThreads), 0, stream, w);
-        MOON_LAUNCH_CHECK();
-        const unsigned routeBlocks = static_cast<unsigned>((w.s * w.k + kThreads - 1) / kThreads);
-        hipLaunchKernelGGL(moon_agree_kernel, dim3(routeBlocks, R), dim3(kThreads), 0, stream, w);
-        MOON_LAUNCH_CHECK();
-    }
     bool vec = w.h % 8 == 0;
     for (int r = 0; r < w.world; ++r) {
         vec = vec && TileXREp::Aligned16(w.hiddenSh[r]) && TileXREp::Aligned16(w.hiddenNvsh[r]);
@@ -1070,12 +1075,20 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
     const int64_t worldRowBytes = static_cast<int64_t>(w.world) * w.s * w.h * 2;
     const bool uncachedRows = worldRowBytes > gCachedRowBytes.load();
     const bool perRoute = vec && !(uncachedRows && w.s * tokenSlices <= 0x7fffffff) && blocks <= 0x7fffffff;
-    if (perRoute && worldRowBytes <= kWarmRowBytes) {
-        // up to half the memory-side cache of token rows: read them once so that the per-route kernel finds them there
-        // (one rank's share of 4096 x 7168: 257 -> about 210 us per layer on rows that were not cached, a few us more
-        // on rows that were)
-        const int64_t rowVecs = w.s * vecs;
-        const unsigned warmBlocks = static_cast<unsigned>((rowVecs + kThreads * kWarmLoads - 1) / (kThreads * kWarmLoads));
+    // up to half the memory-side cache of token rows: read them once so that the per-route kernel finds them there
+    // (one rank's share of 4096 x 7168: 257 -> about 210 us per layer on rows that were not cached, a few us more
+    // on rows that were)
+    const bool warm = perRoute && worldRowBytes <= kWarmRowBytes;
+    const int64_t rowVecs = w.s * vecs;
+    const unsigned warmBlocks = warm ? static_cast<unsigned>((rowVecs + kThreads * kWarmLoads - 1) / (kThreads * kWarmLoads)) : 0u;
+    if (!w.fresh) {
+        hipLaunchKernelGGL(moon_group_walk_kernel, dim3(rowBlocks, R), dim3(kThreads), 0, stream, w);
+        MOON_LAUNCH_CHECK();
+        const unsigned routeBlocks = static_cast<unsigned>((w.s * w.k + kThreads - 1) / kThreads);
+        hipLaunchKernelGGL(moon_agree_kernel, dim3(routeBlocks + warmBlocks, R), dim3(kThreads), 0, stream, w, routeBlocks,
+            warm ? rowVecs : int64_t{0});
+        MOON_LAUNCH_CHECK();
+    } else if (warm) {
         hipLaunchKernelGGL(moon_warm_rows_kernel, dim3(warmBlocks, R), dim3(kThreads), 0, stream, w, rowVecs);
         MOON_LAUNCH_CHECK();
     }
