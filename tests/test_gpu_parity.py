@@ -578,6 +578,40 @@ def test_combine_skips_corrupted_tuples(shape, route):
             assert torch.all(edges == 9.0)                  # nothing was stored outside y
 
 
+@pytest.mark.parametrize("h", [1024, 7168])
+@pytest.mark.parametrize("quant", [ep.Q_NONE, ep.Q_TOKEN_INT8, ep.Q_FP8_BLOCK128])
+def test_combine_with_rows_missing_in_any_pattern_of_slots(quant, h):
+    """The reduce takes the slots of a token that have a row first, in k order, a few at a time; the sum must be the
+    one the oracle forms by walking all slots.  Every token here loses a random subset of its eight rows (a tuple whose
+    token is -1 stands for no row): none, all, the leading ones, more than one batch's worth left, exactly one left."""
+    bs, K, E = 96, 8, 32
+    rng = np.random.default_rng(h + quant)
+    ids = ids_for(rng, bs, K, E)
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16, scale=2.0)
+    d = O.mem_dispatch(O.Case(1, bs, h, K, E, dtype=ep.DT_BF16, quant_mode=quant), 0, xb[None], ids[None])
+    w = (0.5 + rng.random((bs, K))).astype(np.float32)
+    keep = rng.random((bs, K)) < rng.random((bs, 1))          # a different share of rows kept for every token
+    keep[0], keep[1], keep[2, :5], keep[2, 5:] = True, False, False, True
+    keep[3], keep[3, 6] = False, True
+    assist = d["assist"].copy()
+    lost = ~keep[assist[:, 1], assist[:, 2]]
+    assist[lost, 1] = -1
+    assert 0 < lost.sum() < bs * K
+    with Session() as s:
+        y = torch.full((bs, h), 7.0, dtype=torch.bfloat16, device=DEV)
+        eo = to_dev(d["expand_x"]) if quant else to_dev(d["expand_x"].view(np.uint16))
+        st = ep.combine_memory_ex(eo, to_dev(assist), to_dev(d["send_counts"]), s.comm, bs, h, K, E, y, ep.DT_BF16,
+                                  s.stream, expert_out_quant_mode=quant,
+                                  expert_out_scales=to_dev(d["dyn_scales"]) if quant else None, expert_scales=to_dev(w))
+        assert st == 0
+        s.sync()
+        host_eo = d["expand_x"][None] if quant else d["expand_x"].view(np.uint16)[None]
+        want = O.mem_combine(O.Case(1, bs, h, K, E, dtype=ep.DT_BF16), 0, host_eo, assist[None], d["send_counts"][None],
+                             expert_scales=w, in_quant=quant, in_scales=d["dyn_scales"] if quant else None)
+        assert np.array_equal(bits16(y), want)
+        assert np.all(bits16(y)[1] == 0)
+
+
 def test_combine_ignores_row_map_entries_outside_the_buffer():
     """The row map dispatch hands to combine is trusted input, but an entry at or beyond bs * topK (or below -1) must
     read as "no row": the kernels never touch memory outside the rows the caller's buffer holds."""
