@@ -219,6 +219,11 @@ __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool 
     bool pending = false;
     for (int k = lane; k < a.slots; k += lanes) {
         const int64_t slot = static_cast<int64_t>(tokOk ? token : 0) * a.slots + k;
+        // shared-expert slots follow the routed ones and carry no gate weight
+        // (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:650-657)
+        // The weight is asked for before the row is looked at: one trip to memory for both, not one after the other.
+        const float weight = (tokOk && a.expertScales != nullptr && k < a.topK) ?
+            a.expertScales[static_cast<int64_t>(token) * a.topK + k] : 1.0f;
         int row = tokOk ? LookupRow(a, slot) : -1;
         if (row >= 0 && a.tileFlags != nullptr && (BLOCK || mode != kRouteTrusted)) {
             const bool there = BLOCK ? WaitTile(a, row) : TilePublished(a, row);
@@ -233,10 +238,7 @@ __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool 
             }
         }
         rows[k] = row;
-        // shared-expert slots follow the routed ones and carry no gate weight
-        // (reference: src/ep/kernels/tilexr_ep_combine_memory_kernel.h:650-657)
-        weights[k] = (tokOk && a.expertScales != nullptr && k < a.topK) ?
-            a.expertScales[static_cast<int64_t>(token) * a.topK + k] : 1.0f;
+        weights[k] = weight;
     }
     if (FENCE && a.tileFlags != nullptr && lane < a.slots) {
         // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
