@@ -17,6 +17,10 @@
 
 namespace TileXREp {
 
+// exponent fields of the divisors for which DivideByShared is used (see there)
+constexpr uint32_t kSharedDivisionMinExponent = 16;
+constexpr uint32_t kSharedDivisionMaxExponent = 254;
+
 typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned int u32x2 __attribute__((ext_vector_type(2)));
 
@@ -177,6 +181,47 @@ __device__ __forceinline__ uint32_t Fp8E4m3EncodePairSat(float lo, float hi)
         code = (code & 0x00ffu) | ((((__float_as_uint(hi) >> 24) & 0x80u) | 0x7fu) << 8);
     }
     return code;
+}
+
+// Four values that are not NaNs -> four e4m3 codes in one word (a | b << 8 | c << 16 | d << 24), same codes as
+// Fp8E4m3EncodePairSat: the second convert writes the upper half of the word the first one started.
+__device__ __forceinline__ uint32_t Fp8E4m3EncodeFourSat(float a, float b, float c, float d)
+{
+    const int lower = __builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(a, -448.0f, 448.0f),
+        __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f), 0, false);
+    return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(__builtin_amdgcn_fmed3f(c, -448.0f, 448.0f),
+        __builtin_amdgcn_fmed3f(d, -448.0f, 448.0f), lower, true));
+}
+
+// x / b for many x and one b > 0, for a caller that encodes the quotient as e4m3: the code is the one the correctly
+// rounded quotient __fdiv_rn(x, b) gives, on every pair a block quantiser can meet.
+// The correctly rounded quotient costs about eleven instructions per element when the compiler expands the division
+// (range scaling, reciprocal, two refinements of the reciprocal, quotient, two remainders, fix-up).  Everything that
+// depends on b alone is done once here (SharedReciprocal): the reciprocal refined to within a rounding of 1 / b.  An
+// element then takes a product, an exact remainder and one correction, plus the sign (b > 0, so the quotient has the
+// sign of x; a zero remainder would otherwise turn -0 into +0).  The long form corrects the quotient twice and scales
+// the operands' ranges; without that the quotient can be off in its last place (about one pair in five hundred) or,
+// for very small divisors, by more.  An exhaustive run over all pairs of 16-bit element patterns and block maxima, bf16
+// and fp16 (tests/cxx/shared_division_check.hip), found no pair whose e4m3 code differs for divisors with the exponent
+// fields that SharedReciprocalHolds accepts; other divisors (block maxima below 2^-102, or infinite) take the long form.
+__device__ __forceinline__ bool SharedReciprocalHolds(float b)
+{
+    const uint32_t exponent = (__float_as_uint(b) >> 23) & 0xffu;
+    return exponent >= kSharedDivisionMinExponent && exponent <= kSharedDivisionMaxExponent;
+}
+
+__device__ __forceinline__ float SharedReciprocal(float b)
+{
+    const float y0 = __builtin_amdgcn_rcpf(b);
+    const float e = __builtin_fmaf(-b, y0, 1.0f);
+    return __builtin_fmaf(e, y0, y0);
+}
+
+__device__ __forceinline__ float DivideByShared(float x, float b, float y)
+{
+    const float q0 = __fmul_rn(x, y);
+    const float r = __builtin_fmaf(-b, q0, x);
+    return __builtin_copysignf(__builtin_fmaf(r, y, q0), x);
 }
 
 // True when one of the four e4m3 codes in `word` is a NaN code (0x7f / 0xff).

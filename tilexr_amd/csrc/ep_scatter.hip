@@ -293,6 +293,7 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
                 f[2 * w + 1] = Decode16<BF16>(v[j][w] >> 16);
             }
             uint32_t bytes[8];
+            uint32_t fp8Words[2] = {0u, 0u};
             if (QMODE == TILEXR_EP_QUANT_MXFP8 || QMODE == TILEXR_EP_QUANT_FP8_BLOCK128) {
                 float amax = 0.0f;
 #pragma unroll
@@ -315,11 +316,36 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
                 } else {
                     const float sc = amax > 0.0f ? __fdiv_rn(amax, 448.0f) : 1.0f;
                     blockScale[j] = sc;
+                    // eight quotients by one divisor: what depends on the divisor alone is done once (ep_numerics.hip.h)
+                    float quot[8];
+                    const bool shortForm = __all(SharedReciprocalHolds(sc) ? 1 : 0) != 0;
+                    if (shortForm) {
+                        const float y = SharedReciprocal(sc);
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            quot[e] = DivideByShared(f[e], sc, y);
+                        }
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; ++e) {
+                            quot[e] = __fdiv_rn(f[e], sc);
+                        }
+                    }
+                    bool anyNan = false;
 #pragma unroll
                     for (int e = 0; e < 8; e += 2) {
-                        const uint32_t pair = Fp8E4m3EncodePairSat(__fdiv_rn(f[e], sc), __fdiv_rn(f[e + 1], sc));
-                        bytes[e] = pair & 0xffu;
-                        bytes[e + 1] = pair >> 8;
+                        anyNan |= __builtin_isunordered(quot[e], quot[e + 1]);
+                    }
+                    if (!anyNan) {
+                        // four codes per word straight from the converts: the second one fills the word's upper half
+                        fp8Words[0] = Fp8E4m3EncodeFourSat(quot[0], quot[1], quot[2], quot[3]);
+                        fp8Words[1] = Fp8E4m3EncodeFourSat(quot[4], quot[5], quot[6], quot[7]);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < 8; e += 4) {
+                            fp8Words[e / 4] = Fp8E4m3EncodePairSat(quot[e], quot[e + 1]) |
+                                (Fp8E4m3EncodePairSat(quot[e + 2], quot[e + 3]) << 16);
+                        }
                     }
                 }
             } else {
@@ -328,8 +354,13 @@ __global__ __launch_bounds__(kThreads) void ep_scatter_vec_kernel(ScatterArgs a)
                     bytes[e] = static_cast<uint32_t>(ClampInt8(__fmul_rn(f[e], rowScaleInv))) & 0xffu;
                 }
             }
-            q[j][0] = bytes[0] | (bytes[1] << 8) | (bytes[2] << 16) | (bytes[3] << 24);
-            q[j][1] = bytes[4] | (bytes[5] << 8) | (bytes[6] << 16) | (bytes[7] << 24);
+            if (QMODE == TILEXR_EP_QUANT_FP8_BLOCK128) {
+                q[j][0] = fp8Words[0];
+                q[j][1] = fp8Words[1];
+            } else {
+                q[j][0] = bytes[0] | (bytes[1] << 8) | (bytes[2] << 16) | (bytes[3] << 24);
+                q[j][1] = bytes[4] | (bytes[5] << 8) | (bytes[6] << 16) | (bytes[7] << 24);
+            }
         }
         const int mxBlocks = (a.h + 31) / 32;
         const int mxScales = (mxBlocks + 1) / 2 * 2;
