@@ -550,8 +550,9 @@ def main():
     steps_by_schedule = {"flags-serial": step_flags_serial, "flags-overlapped": step_overlapped, "plain": step_plain}
     schedule = "flags-overlapped" if args.overlap else args.schedule
     calibration = None
-    # decode-sized calls (at most 2048 routes) take the library's single-launch dispatch, which publishes no flags: two
-    # launches per layer instead of four is what counts there
+    # decode-sized calls (at most 2048 routes) take the library's single-launch dispatch: two launches per layer with or
+    # without flags, and without them nothing waits for written-through rows before a workgroup may leave (16 against
+    # 20 us per layer), which is what counts at this size
     small = bs * K <= 2048
     if schedule == "auto" and small:
         schedule = "plain"

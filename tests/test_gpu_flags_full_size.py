@@ -161,6 +161,19 @@ def test_rows_wider_than_one_publishing_workgroup(two_streams):
                   expect_reduce="ep_reduce_vec_kernel")
 
 
+@pytest.mark.parametrize("tile_rows", [1, 7, 64, 1 << 20])
+@pytest.mark.parametrize("capacity_factor", [0.0, 0.8], ids=["no_limit", "capacity"])
+def test_decode_sized_dispatch_publishes_tiles_from_its_single_launch(capacity_factor, tile_rows):
+    """At most 2048 routes: dispatch is one launch (a workgroup per route, or per token when a capacity limit needs the
+    per-expert histogram), and with flags on one stream it stays one launch: the rows are written through and reported
+    landed by the same kernel.  Outputs, combine result and every readiness word against the oracle, two layers through
+    the same buffers."""
+    w = workloads.Workload(f"decode@{capacity_factor}", 1, 128, 7168, 8, 256, x_dist="normal", routing="gating",
+                           capacity_factor=capacity_factor, seed=11)
+    run_and_check(layers_of(w), tile_rows, False, expect_scatter="ep_dispatch_small_kernel",
+                  expect_reduce="ep_reduce_vec_kernel")
+
+
 def test_two_communicators_share_one_flag_array():
     """Flag epochs come from one counter for the whole process: two communicators that are handed the same flag array
     one after the other can never tag it with the same value, so words left by the first read as not ready to a

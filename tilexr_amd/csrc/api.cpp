@@ -60,9 +60,9 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
             return TileXR::TILEXR_ERROR_MKIRT;
         }
     }
-    if (memoryRoute && p.quantMode == TILEXR_EP_QUANT_NONE && p.xActiveMask == nullptr && p.tileFlagsOut == nullptr &&
-        p.metaReadyEvent == nullptr) {
-        // decode-sized calls: one launch instead of count + scatter
+    if (memoryRoute && p.quantMode == TILEXR_EP_QUANT_NONE && p.xActiveMask == nullptr && p.metaReadyEvent == nullptr) {
+        // decode-sized calls: one launch instead of count + scatter (a consumer that is to run beside the dispatch needs
+        // the row map ahead of the rows, which takes the separate launches)
         SmallDispatchLaunch small {};
         small.x = p.x;
         small.ids = p.expertIds;
@@ -81,8 +81,24 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
         small.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
         small.stream = stream;
         if (SmallDispatchFits(small)) {
+            if (p.tileFlagsOut != nullptr) {
+                // a tile never holds more rows than the dispatch can produce: larger values name the same single tile
+                small.tileRows = std::min<int64_t>(p.tileRows, std::max<int64_t>(n, 1));
+                if (!comm->tileCounters.Reserve(static_cast<size_t>(TileCounterWords(n, small.tileRows)) * sizeof(uint32_t), true)) {
+                    return TileXR::TILEXR_ERROR_INTERNAL;
+                }
+                small.tileFlags = p.tileFlagsOut;
+                small.tileCounters = static_cast<uint32_t *>(comm->tileCounters.ptr);
+                small.epoch = flagEpoch;
+            }
             comm->lastKernel[kKernelScatter] = "ep_dispatch_small_kernel";
-            return Timed(comm, kKernelScatter, stream, "small dispatch", [&] { return LaunchSmallDispatch(small); });
+            const int ret = Timed(comm, kKernelScatter, stream, "small dispatch", [&] { return LaunchSmallDispatch(small); });
+            if (ret == kOk && p.tileFlagsOut != nullptr) {
+                comm->lastFlagWords = p.tileFlagsOut;
+                comm->lastFlagEpoch = flagEpoch;
+                comm->lastFlagStream = stream;
+            }
+            return ret;
         }
     }
     const CountScratchLayout plan = PlanCountScratch(n, numKeys, experts, expertHist);

@@ -62,6 +62,24 @@ __device__ __forceinline__ void WaitOwnStores()
 {
     __builtin_amdgcn_s_waitcnt(0);
 }
+
+// Device side of ep_tile_publish.h: relaxed agent-scope atomics.  The caller has made the row complete in memory
+// first, so has every earlier counter of the tile, and the atomics on one counter are totally ordered: when the last
+// one returns, all rows of the tile are in memory.
+struct DeviceTileOps {
+    __device__ __forceinline__ uint32_t FetchAdd(uint32_t *p)
+    {
+        return __hip_atomic_fetch_add(p, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ void Store(uint32_t *p, uint32_t v)
+    {
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __device__ __forceinline__ void Store(uint64_t *p, uint64_t v)
+    {
+        __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+};
 #endif
 
 } // namespace TileXREp

@@ -195,6 +195,10 @@ struct SmallDispatchLaunch {
     int32_t *sendCountsOut;
     int64_t *expertTokenNumsOut;
     int tokenNumsType;
+    uint64_t *tileFlags;             // optional: a readiness word per tile of rows, as LaunchScatter publishes them
+    uint32_t *tileCounters;          // TileCounterWords(bs * topK, tileRows) zeroed words
+    int64_t tileRows;
+    uint64_t epoch;
     hipStream_t stream;
 };
 bool SmallDispatchFits(const SmallDispatchLaunch &l);

@@ -5,13 +5,16 @@
 // the same expert -- while its token's row is already on its way from HBM, and then writes the row to its topK
 // destination rows.  Workgroup 0 also writes the count outputs.  The results are the same as those of the count +
 // scatter pair (same definitions, reference: src/ep/kernels/tilexr_ep_dispatch_memory_kernel.h:791-818, 1059-1074,
-// 1159-1168, 1240-1258); only the number of launches differs.
+// 1159-1168, 1240-1258); only the number of launches differs.  With readiness flags the rows are written through to memory
+// and reported landed as in the scatter kernels (ep_tile_publish.h); the rows the whole dispatch keeps, which the size of
+// the last tile depends on, every workgroup has counted anyway or counts with four more ballots.
 #include <hip/hip_runtime.h>
 
 #include "ep_block_scan.hip.h"
 #include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
 #include "ep_numerics.hip.h"
+#include "ep_tile_publish.h"
 
 namespace TileXREp {
 namespace {
@@ -34,9 +37,22 @@ struct SmallArgs {
     int32_t *sendCountsOut;
     int64_t *expertTokenNumsOut;
     int tokenNumsType;
+    TilePublishArgs tiles;       // flags == nullptr: none (totalRows is filled in by the kernels)
 };
 
-template <int V>
+// A row's vectors: streaming stores, or -- when readiness flags are published -- stores written through to memory, which
+// are complete for every XCD once the issuing wave's memory counter is zero.
+template <bool WT>
+__device__ __forceinline__ void SmallRowStore(const u32x4 &v, u32x4 *dst, __amdgpu_buffer_rsrc_t rsrc, int idx)
+{
+    if (WT) {
+        __builtin_amdgcn_raw_buffer_store_b128(v, rsrc, idx * 16, 0, kAuxAgentScope);
+    } else {
+        __builtin_nontemporal_store(v, dst + idx);
+    }
+}
+
+template <int V, bool WT>
 __global__ __launch_bounds__(kThreads) void ep_dispatch_small_kernel(SmallArgs a)
 {
     __shared__ int s_hist[kMaxKeys];     // routes per expert, then exclusive row offsets
@@ -100,7 +116,7 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_kernel(SmallArgs a
         s_hist[k] = kept;
     }
     __syncthreads();
-    BlockExclusiveScan(s_hist, a.numExperts, s_part);
+    const int totalRows = BlockExclusiveScan(s_hist, a.numExperts, s_part);
     if (tid < a.topK) {
         const int key = s_key[tid];
         int row = -1;
@@ -133,12 +149,24 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_kernel(SmallArgs a
             continue;
         }
         u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2);
+        const __amdgpu_buffer_rsrc_t rsrc = RowResource(dst, vecs * 16);
 #pragma unroll
         for (int j = 0; j < V; ++j) {
             const int idx = j * kThreads + tid;
             if (idx < vecs) {
-                __builtin_nontemporal_store(v[j], dst + idx);
+                SmallRowStore<WT>(v[j], dst, rsrc, idx);
             }
+        }
+    }
+    if (WT) {
+        // every wave waits for its own stores, the barrier collects the waves, then the rows are reported landed
+        WaitOwnStores();
+        __syncthreads();
+        if (tid < a.topK && s_pos[tid] >= 0) {
+            TilePublishArgs t = a.tiles;
+            t.totalRows = totalRows;
+            DeviceTileOps ops;
+            PublishLanded(ops, t, s_pos[tid], 1);
         }
     }
 }
@@ -161,10 +189,10 @@ __device__ __forceinline__ void AddBallots(const bool (&pred)[kIdsPerLane], int 
 // so one workgroup per route counts those two sets over the id table and writes its one row.  Workgroup b < E also
 // counts expert b's routes for the count outputs.  Eight times as many workgroups as tokens spread a decode batch
 // over the whole chip.
-template <int V>
+template <int V, bool WT>
 __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(SmallArgs a)
 {
-    __shared__ int s_sum[4];     // smaller ids, earlier equal ids, ids equal to blockIdx, ids not above blockIdx
+    __shared__ int s_sum[5];     // smaller ids, earlier equal ids, ids equal to blockIdx, ids not above blockIdx, valid ids
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
@@ -189,7 +217,7 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
     }
     const int mine = a.ids[route];
     const int key = (mine >= 0 && mine < a.numExperts) ? mine : -1;
-    if (tid < 4) {
+    if (tid < 5) {
         s_sum[tid] = 0;
     }
     __syncthreads();
@@ -205,6 +233,15 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
     }
     AddBallots(less, &s_sum[0], lane);
     AddBallots(before, &s_sum[1], lane);
+    if (WT) {
+        // rows the whole dispatch keeps: the size of the last tile
+        bool valid[kIdsPerLane];
+#pragma unroll
+        for (int j = 0; j < kIdsPerLane; ++j) {
+            valid[j] = e[j] >= 0;
+        }
+        AddBallots(valid, &s_sum[4], lane);
+    }
     if (expert < a.numExperts) {
         AddBallots(same, &s_sum[2], lane);
         AddBallots(upTo, &s_sum[3], lane);
@@ -233,11 +270,22 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
         return;
     }
     u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.out) + static_cast<int64_t>(row) * a.h * 2);
+    const __amdgpu_buffer_rsrc_t rsrc = RowResource(dst, vecs * 16);
 #pragma unroll
     for (int j = 0; j < V; ++j) {
         const int idx = j * kThreads + tid;
         if (idx < vecs) {
-            __builtin_nontemporal_store(v[j], dst + idx);
+            SmallRowStore<WT>(v[j], dst, rsrc, idx);
+        }
+    }
+    if (WT) {
+        WaitOwnStores();
+        __syncthreads();        // uniform: a workgroup without a row has left as a whole
+        if (tid == 0) {
+            TilePublishArgs t = a.tiles;
+            t.totalRows = s_sum[4];
+            DeviceTileOps ops;
+            PublishLanded(ops, t, row, 1);
         }
     }
 }
@@ -268,26 +316,36 @@ hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l)
     a.sendCountsOut = l.sendCountsOut;
     a.expertTokenNumsOut = l.expertTokenNumsOut;
     a.tokenNumsType = l.tokenNumsType;
+    const bool flags = l.tileFlags != nullptr;
+    if (flags) {
+        a.tiles.flags = l.tileFlags;
+        a.tiles.counters = l.tileCounters;
+        a.tiles.tileRows = static_cast<int>(l.tileRows);
+        a.tiles.maxTiles = static_cast<int>((l.bs * l.topK + l.tileRows - 1) / l.tileRows);
+        a.tiles.epoch = l.epoch;
+    }
     const int64_t vecs = l.h / 8;
+    const int v = vecs <= 2 * kThreads ? 2 : (vecs <= 4 * kThreads ? 4 : 8);
+    auto launch = [&](auto kernel, dim3 grid) { hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 0, l.stream, a); };
     if (l.capacity <= 0 && l.bs * l.topK >= l.numExperts) {
         // one workgroup per route (there are enough of them to cover the experts' count outputs)
         const dim3 routes(static_cast<unsigned>(l.bs * l.topK));
-        if (vecs <= 2 * kThreads) {
-            hipLaunchKernelGGL(ep_dispatch_small_route_kernel<2>, routes, dim3(kThreads), 0, l.stream, a);
-        } else if (vecs <= 4 * kThreads) {
-            hipLaunchKernelGGL(ep_dispatch_small_route_kernel<4>, routes, dim3(kThreads), 0, l.stream, a);
+        if (v == 2) {
+            flags ? launch(ep_dispatch_small_route_kernel<2, true>, routes) : launch(ep_dispatch_small_route_kernel<2, false>, routes);
+        } else if (v == 4) {
+            flags ? launch(ep_dispatch_small_route_kernel<4, true>, routes) : launch(ep_dispatch_small_route_kernel<4, false>, routes);
         } else {
-            hipLaunchKernelGGL(ep_dispatch_small_route_kernel<8>, routes, dim3(kThreads), 0, l.stream, a);
+            flags ? launch(ep_dispatch_small_route_kernel<8, true>, routes) : launch(ep_dispatch_small_route_kernel<8, false>, routes);
         }
         return hipGetLastError();
     }
     const dim3 grid(static_cast<unsigned>(l.bs));
-    if (vecs <= 2 * kThreads) {
-        hipLaunchKernelGGL(ep_dispatch_small_kernel<2>, grid, dim3(kThreads), 0, l.stream, a);
-    } else if (vecs <= 4 * kThreads) {
-        hipLaunchKernelGGL(ep_dispatch_small_kernel<4>, grid, dim3(kThreads), 0, l.stream, a);
+    if (v == 2) {
+        flags ? launch(ep_dispatch_small_kernel<2, true>, grid) : launch(ep_dispatch_small_kernel<2, false>, grid);
+    } else if (v == 4) {
+        flags ? launch(ep_dispatch_small_kernel<4, true>, grid) : launch(ep_dispatch_small_kernel<4, false>, grid);
     } else {
-        hipLaunchKernelGGL(ep_dispatch_small_kernel<8>, grid, dim3(kThreads), 0, l.stream, a);
+        flags ? launch(ep_dispatch_small_kernel<8, true>, grid) : launch(ep_dispatch_small_kernel<8, false>, grid);
     }
     return hipGetLastError();
 }
