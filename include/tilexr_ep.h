@@ -163,7 +163,8 @@ struct TileXREpCombineExOptions {
     const uint64_t *tileFlags;    // optional: before a row is read, wait until the upper half of its tile's word
                                   //      equals flagEpoch; the rows are then read from memory, not from a cache.
                                   //      A producer other than the dispatch above (an expert stage) completes its
-                                  //      rows with a release at agent scope, then stores the word.  The producer's
+                                  //      rows with a release at agent scope that it waits for (the write-back of
+                                  //      its L2 has to be over), then stores the word.  The producer's
                                   //      work must be enqueued BEFORE this call: streams of a process may share a
                                   //      hardware queue, where a waiting kernel keeps later kernels behind it
                                   //      Waiting workgroups stay resident (two per compute unit): a producer

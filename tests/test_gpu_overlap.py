@@ -384,6 +384,7 @@ def test_flag_protocol_on_randomised_rounds():
             elif qmode == ep.Q_FP8_BLOCK128:
                 scales = pool_scales[:n * ((h + 127) // 128)].view(n, (h + 127) // 128)
             y = pool_y[:bs * h].view(bs, h)
+            y.fill_(-1234.0)                 # tells a token that was never written from one that was summed wrongly
             assist = torch.empty((n, 4), dtype=torch.int32, device=DEV)
             token_nums = torch.empty((E,), dtype=torch.int64, device=DEV)
             counts = torch.empty((E,), dtype=torch.int32, device=DEV)
@@ -423,11 +424,39 @@ def test_flag_protocol_on_randomised_rounds():
             case = O.Case(1, bs, h, K, E, dtype=O.DT_BF16, quant_mode=oq, token_nums_type=1)
             want = O.mem_dispatch(case, 0, xb[None], ids[None])
             assert np.array_equal(expand_x.cpu().numpy(), want["expand_x"]), f"round {round_}: rows"
+            # the row map the combine was given: row of (token, k) as the oracle's tuples have it
+            want_map = np.full((bs, K), -1, np.int32)
+            live = want["assist"][:want["rows"]]
+            want_map[live[:, 1], live[:, 2]] = np.arange(want["rows"], dtype=np.int32)
+            assert np.array_equal(row_map.cpu().numpy(), want_map), f"round {round_}: row map"
+            assert np.array_equal(assist.cpu().numpy()[:want["rows"]], live), f"round {round_}: assist tuples"
+            if schedule == "expert_stage":
+                assert torch.equal(expert_out, expand_x), f"round {round_}: the stand-in's copy of the rows"
+                f = stage_flags[:(n + tile_rows - 1) // tile_rows].cpu().numpy().astype(np.uint64)
+                assert np.all(f >> np.uint64(32) == np.uint64(1000 + round_)), f"round {round_}: the stand-in's words"
             eo = want["expand_x"][None] if oq else want["expand_x"].view(np.uint16)[None]
             wy = O.mem_combine(O.Case(1, bs, h, K, E, dtype=O.DT_BF16), 0, eo, want["assist"][None],
                                want["send_counts"][None], expert_scales=w, in_quant=oq,
                                in_scales=want["dyn_scales"] if oq else None)
-            assert np.array_equal(bits16(y), wy), f"round {round_}: y"
+            got_y = bits16(y)
+            bad = np.flatnonzero((got_y != wy).any(axis=1))
+            untouched = int((got_y[bad] == bits16(torch.tensor([-1234.0], dtype=torch.bfloat16))[0]).all(axis=1).sum())
+            detail = ""
+            if bad.size:
+                t = int(bad[0])
+                cols = np.flatnonzero(got_y[t] != wy[t])
+                rows_t = row_map.cpu().numpy()[t]
+                src = (expert_out if schedule == "expert_stage" else expand_x).cpu().numpy()
+                detail = (f"; token {t}: {cols.size} columns differ, first {cols[:6].tolist()} last {cols[-3:].tolist()}, "
+                          f"got {got_y[t][cols[:4]].tolist()} want {wy[t][cols[:4]].tolist()}, weights {w[t].tolist()}")
+                if qmode == ep.Q_NONE:
+                    f32 = lambda bits: (bits.astype(np.uint32) << 16).view(np.float32)
+                    parts = [f32(src[r].view(np.uint16)) * np.float32(w[t, k]) for k, r in enumerate(rows_t) if r >= 0]
+                    for k, part in enumerate(parts):
+                        alone = ((part.view(np.uint32) + 0x7fff + ((part.view(np.uint32) >> 16) & 1)) >> 16).astype(np.uint16)
+                        detail += f", equals slot {k} alone on {int((got_y[t][cols] == alone[cols]).sum())} of them"
+            assert bad.size == 0, (f"round {round_}: y differs for {bad.size} tokens ({untouched} of them never written), "
+                                   f"first {bad[:8].tolist()}, rows {row_map.cpu().numpy()[bad[:4]].tolist()}" + detail)
             rounds += 1
         assert rounds >= 8
         meta_ready.destroy()

@@ -63,6 +63,19 @@ __device__ __forceinline__ void WaitOwnStores()
     __builtin_amdgcn_s_waitcnt(0);
 }
 
+// Release at agent scope for rows written with ordinary stores: when the call returns, everything this wave has
+// stored -- and, after a barrier that followed their own waits, what the other waves of its workgroup have stored --
+// is in memory, so a readiness word stored next can never be seen ahead of the rows.  The fence writes this XCD's L2
+// back (`buffer_wbl2 sc1`).  The wait for that write-back is spelled out here: in the code hipcc 7.2 generates for the
+// fence alone the write-back is followed directly by the next store (the wait the fence asks for after it does not
+// survive the compiler's wait-count pass), and the word then reaches memory first now and then: one row in a few
+// thousand was read before it was there.
+__device__ __forceinline__ void ReleaseRowsToAgent()
+{
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+
 // Device side of ep_tile_publish.h: relaxed agent-scope atomics.  The caller has made the row complete in memory
 // first, so has every earlier counter of the tile, and the atomics on one counter are totally ordered: when the last
 // one returns, all rows of the tile are in memory.

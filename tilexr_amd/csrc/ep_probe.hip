@@ -200,7 +200,7 @@ __global__ __launch_bounds__(kThreads) void ep_probe_tile_producer_kernel(const 
         WaitOwnStores();
         __syncthreads();
         if (threadIdx.x == 0) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            ReleaseRowsToAgent();
             __hip_atomic_store(&tileFlags[tile], (epoch << 32) | static_cast<uint32_t>(count), __ATOMIC_RELAXED,
                 __HIP_MEMORY_SCOPE_AGENT);
         }

@@ -130,7 +130,7 @@ __device__ __forceinline__ void PublishRows(const ScatterArgs &a, const int *pos
     }
     if (lane < a.topK) {
         if (!WT) {
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+            ReleaseRowsToAgent();
         }
         for (int k = lane; k < a.topK; k += G) {
             const int row = pos[k];
