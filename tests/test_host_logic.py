@@ -25,7 +25,7 @@ def test_library_exports_every_declared_symbol():
     for header in ("tilexr_ep.h", "tilexr_api.h"):
         text = open(os.path.join(ROOT, "include", header)).read()
         declared |= set(re.findall(r"^(?:int|const char \*)\s*\*?(TileXR\w+)\(", text, flags=re.M))
-    assert len(declared) == 22, sorted(declared)
+    assert len(declared) == 20, sorted(declared)
     assert declared == set(ep.EXPORTS)
     for name in declared:
         assert getattr(lib, name) is not None
@@ -46,6 +46,9 @@ def test_library_exports_nothing_but_the_declared_entry_points():
     hooks = subprocess.run(["nm", "-D", "--defined-only", H.HOOKS_PATH], check=True, capture_output=True, text=True).stdout
     names = {line.split()[-1] for line in hooks.splitlines() if line.strip()}
     assert names and all(n.startswith(("TileXREpHook", "TileXREpTrace")) for n in names), sorted(names)
+    probes = subprocess.run(["nm", "-D", "--defined-only", ep.PROBES_PATH], check=True, capture_output=True, text=True).stdout
+    assert {line.split()[-1] for line in probes.splitlines() if line.strip()} == \
+        {"TileXREpMemoryProbe", "TileXREpTileProducerProbe"}
 
 
 # ---------------------------------------------------------------------------------------------

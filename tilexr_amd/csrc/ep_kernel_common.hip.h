@@ -6,6 +6,8 @@
 
 #if defined(__HIPCC__)
 #include <hip/hip_runtime.h>
+
+#include "tilexr_ep_publish.hip.h"
 #endif
 
 namespace TileXREp {
@@ -60,20 +62,24 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t RowResource(const void *row, i
 // Waits until every store this wave has issued is complete (vmcnt, expcnt and lgkmcnt all zero).
 __device__ __forceinline__ void WaitOwnStores()
 {
-    __builtin_amdgcn_s_waitcnt(0);
+    TileXREpWaitOwnStores();
 }
 
-// Release at agent scope for rows written with ordinary stores: when the call returns, everything this wave has
-// stored -- and, after a barrier that followed their own waits, what the other waves of its workgroup have stored --
-// is in memory, so a readiness word stored next can never be seen ahead of the rows.  The fence writes this XCD's L2
-// back (`buffer_wbl2 sc1`).  The wait for that write-back is spelled out here: in the code hipcc 7.2 generates for the
-// fence alone the write-back is followed directly by the next store (the wait the fence asks for after it does not
-// survive the compiler's wait-count pass), and the word then reaches memory first now and then: one row in a few
-// thousand was read before it was there.
+// Release / acquire at agent scope for rows that move with ordinary stores and loads: the installed header
+// tilexr_ep_publish.hip.h holds the one implementation (and the ordering rule), so that a producer or consumer outside
+// the library runs the same instructions as the kernels here.  Both spell out the wait that follows the cache
+// operation: in the code hipcc 7.2 generates for the fence alone, the L2 write-back of a release is followed directly
+// by the next store (the wait the fence asks for does not survive the compiler's wait-count pass), and a readiness word
+// then reaches memory ahead of the rows now and then: one row in a few thousand was read before it was there.  The
+// acquire side gets the same treatment, and every wave that reads rows with ordinary loads issues its own.
 __device__ __forceinline__ void ReleaseRowsToAgent()
 {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    TileXREpReleaseRowsToAgent();
+}
+
+__device__ __forceinline__ void AcquireRowsFromAgent()
+{
+    TileXREpAcquireRowsFromAgent();
 }
 
 // Device side of ep_tile_publish.h: relaxed agent-scope atomics.  The caller has made the row complete in memory

@@ -19,7 +19,8 @@
 
 #include "ep_kernel_common.hip.h"
 #include "ep_numerics.hip.h"
-#include "tilexr_ep.h"
+#include "ep_probe.h"
+#include "tilexr_ep_publish.hip.h"
 #include "tilexr_types.h"
 
 namespace TileXREp {
@@ -197,12 +198,13 @@ __global__ __launch_bounds__(kThreads) void ep_probe_tile_producer_kernel(const 
         while (static_cast<int64_t>(wall_clock64() - begin) < minTileTicks) {
             __builtin_amdgcn_s_sleep(32);
         }
-        WaitOwnStores();
+        // the publishing rule of tilexr_ep_publish.hip.h, with that header's functions and nothing else, as a producer
+        // outside the library would write it
+        TileXREpWaitOwnStores();
         __syncthreads();
         if (threadIdx.x == 0) {
-            ReleaseRowsToAgent();
-            __hip_atomic_store(&tileFlags[tile], (epoch << 32) | static_cast<uint32_t>(count), __ATOMIC_RELAXED,
-                __HIP_MEMORY_SCOPE_AGENT);
+            TileXREpReleaseRowsToAgent();
+            TileXREpPublishTile(tileFlags, tile, epoch, count);
         }
     }
 }

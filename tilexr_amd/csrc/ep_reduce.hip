@@ -34,8 +34,14 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_generic_kernel(ReduceArgs 
     const int b128 = (a.h + 127) / 128;
     for (int token = blockIdx.x; token < a.bs; token += gridDim.x) {
         __syncthreads();
-        LoadRoutes<true, true>(a, token, true, tid, kThreads, s_row, s_w, kRouteCheck);
+        LoadRoutes<true>(a, token, true, tid, kThreads, s_row, s_w, kRouteCheck);
         __syncthreads();
+        if (a.tileFlags != nullptr) {
+            // pairs with the producer's release.  Every wave reads rows with ordinary loads below, so every wave
+            // invalidates for itself, after the barrier behind which all the token's waits have succeeded and before
+            // its first row load: an invalidate issued by one wave says nothing about when a sibling's load may issue
+            AcquireRowsFromAgent();
+        }
         if (kind == kReducePerAdd) {
             if (tid == 0) {
                 SortRows(s_row, a.slots, a.orderKeys);

@@ -80,8 +80,8 @@ __device__ __forceinline__ int TileOf(const ReduceArgs &a, int row)
 // Bounded wait until the tile holding `row` has been published for this epoch (its word carries the epoch).  The poll itself is a relaxed
 // device-scope load (no cache maintenance per iteration -- an acquire in the loop would invalidate this XCD's L2 on
 // every spin and starve the producer).  What the caller reads afterwards must not come from a stale L2 line: the
-// register-resident kernels read published rows with agent-scope loads, which are served from memory; the
-// element-granular kernel issues one acquire fence after all its waits have succeeded.
+// register-resident kernels read published rows with agent-scope loads, which are served from memory; in the
+// element-granular kernel every wave issues an acquire of its own once all the token's waits have succeeded.
 __device__ inline bool WaitTile(const ReduceArgs &a, int row)
 {
     const int tile = TileOf(a, row);
@@ -212,7 +212,7 @@ __device__ __forceinline__ bool SettledWordMissing(const ReduceArgs &a, int slot
     return missing;
 }
 
-template <bool FENCE, bool BLOCK>
+template <bool BLOCK>
 __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool tokOk, int lane, int lanes, int *rows,
     float *weights, int mode)
 {
@@ -239,11 +239,6 @@ __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool 
         }
         rows[k] = row;
         weights[k] = weight;
-    }
-    if (FENCE && a.tileFlags != nullptr && lane < a.slots) {
-        // pairs with the producer's release: rows read after this fence (by this wave, or by the other waves of the
-        // workgroup after the barrier that follows) are at least as new as the flag values seen above
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     }
     return pending;
 }

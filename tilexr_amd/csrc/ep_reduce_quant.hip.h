@@ -34,7 +34,7 @@ __global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL && INQ == TILEXR_
     };
     auto load = [&](int group, int mode) {
         const int token = group * kTokens + tg;
-        return LoadRoutes<false, false>(a, token, token < a.bs, lane, G, s_row[tg], s_w[tg], mode);
+        return LoadRoutes<false>(a, token, token < a.bs, lane, G, s_row[tg], s_w[tg], mode);
     };
     auto reduceUnit = [&](int group) {
         const int token = group * kTokens + tg;

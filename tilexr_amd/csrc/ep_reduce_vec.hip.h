@@ -55,7 +55,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
     };
     auto load = [&](int group, int mode) {
         const int unit = group * unitsPerGroup + tg;
-        return LoadRoutes<false, false>(a, unit / a.colSlices, unit < units, lane, G, s_row[tg], s_w[tg], mode);
+        return LoadRoutes<false>(a, unit / a.colSlices, unit < units, lane, G, s_row[tg], s_w[tg], mode);
     };
     auto reduceUnit = [&](int group) {
         const int unit = group * unitsPerGroup + tg;

@@ -13,6 +13,8 @@
 
 #include <cstdint>
 
+#include "tilexr_ep_publish.hip.h"
+
 #if defined(__HIPCC__)
 #define TILEXR_EP_HD __host__ __device__ inline __attribute__((always_inline))
 #else
@@ -42,14 +44,15 @@ struct TilePublishArgs {
 
 // The word a complete tile is published with, and the consumer's test of a polled word: ready means "published for
 // exactly this epoch".  A word of an older epoch, a word of a newer one and a zero-filled word all read as not ready.
+// (One definition, in the installed header that producers and consumers outside the library include.)
 TILEXR_EP_HD uint64_t TileReadyWord(uint64_t epoch, int rowsInTile)
 {
-    return (epoch << 32) | static_cast<uint32_t>(rowsInTile);
+    return TileXREpTileReadyWord(epoch, rowsInTile);
 }
 
 TILEXR_EP_HD bool TileWordReady(uint64_t word, uint64_t epoch)
 {
-    return (word >> 32) == epoch;
+    return TileXREpTileWordReady(word, epoch);
 }
 
 template <typename Ops>

@@ -9,6 +9,8 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libtilexr-ep.so")
+# test- and bench-only companion (memory-system yardsticks, a stand-in expert stage): not part of the product library
+PROBES_PATH = os.path.join(_HERE, "lib", "libtilexr-ep-probes.so")
 
 # status codes (include/tilexr_types.h)
 SUCCESS, ERR_NOT_INITIALIZED, ERR_MKIRT, ERR_PARA_CHECK_FAIL, ERR_INTERNAL, ERR_TIMEOUT, ERR_NOT_SUPPORT, \
@@ -23,7 +25,7 @@ EXPORTS = (
     "TileXRMoeEpDispatch", "TileXRMoeEpDispatchV2", "TileXRMoeEpDispatchMemory", "TileXRMoeEpDispatchMemoryV2",
     "TileXRMoeEpCombine", "TileXRMoeEpCombineV2", "TileXRMoeEpCombineMemory", "TileXRMoeEpCombineMemoryV2",
     "TileXRMoeEpDispatchMemoryEx", "TileXRMoeEpCombineMemoryEx", "TileXRMoeEpDispatchMemoryNoAlloc", "TileXREpVersion", "TileXREpSetKernelTimingEvents",
-    "TileXREpLastKernelName", "TileXREpMemoryProbe", "TileXREpTileProducerProbe", "TileXREpSetDebugOptions",
+    "TileXREpLastKernelName", "TileXREpSetDebugOptions",
     "TileXRCommInitRankLocal", "TileXRCommDestroy", "TileXRGetCommArgsHost", "TileXRGetCommArgsDev",
     "TileXRCommNextMagic",
 )
@@ -290,9 +292,22 @@ PROBE_READ, PROBE_WRITE, PROBE_COPY, PROBE_FAN_OUT, PROBE_FAN_IN, PROBE_GATHER_R
     PROBE_GATHER_ROWS_4K_X6 = range(8)
 
 
+_probes = None
+
+
+def probes():
+    """The probe library (csrc/ep_probe.h), loaded once; raises if it has not been built."""
+    global _probes
+    if _probes is None:
+        if not os.path.exists(PROBES_PATH):
+            raise ImportError(f"{PROBES_PATH} is missing: build it with `make -C tilexr_amd/csrc`")
+        _probes = C.CDLL(PROBES_PATH)
+    return _probes
+
+
 def memory_probe(pattern, src, dst, nbytes, stream):
-    """One launch of a kernel that does nothing but the memory traffic of `pattern` (see tilexr_ep.h)."""
-    fn = lib().TileXREpMemoryProbe
+    """One launch of a kernel that does nothing but the memory traffic of `pattern` (see csrc/ep_probe.h)."""
+    fn = probes().TileXREpMemoryProbe
     fn.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_void_p]
     return fn(pattern, _ptr(src), _ptr(dst), int(nbytes), _stream(stream))
 
@@ -300,8 +315,8 @@ def memory_probe(pattern, src, dst, nbytes, stream):
 def tile_producer_probe(src, dst, rows, row_bytes, tile_flags, tile_rows, epoch, workgroups, min_tile_ns, stream,
                         stagger_ns=0):
     """A stand-in for an expert stage: copies rows src -> dst tile by tile at a set pace and publishes each tile's
-    readiness word (see tilexr_ep.h)."""
-    fn = lib().TileXREpTileProducerProbe
+    readiness word (see csrc/ep_probe.h)."""
+    fn = probes().TileXREpTileProducerProbe
     fn.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_void_p, C.c_int64, C.c_int64, C.c_int64, C.c_int64,
                    C.c_int64, C.c_void_p]
     return fn(_ptr(src), _ptr(dst), int(rows), int(row_bytes), _ptr(tile_flags), int(tile_rows), int(epoch),
