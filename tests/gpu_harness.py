@@ -5,6 +5,8 @@ Stream discipline of the tests: inside a Session torch's own work (fills, host c
 session's stream, the one the library calls use.  Multi-rank worlds and side streams use torch's default stream for
 that work and wait for it (`torch.cuda.synchronize()`) before a library call is issued on another stream.  Library
 results are read after the stream of the call has been synchronised."""
+import os
+
 import numpy as np
 import torch
 
@@ -37,9 +39,22 @@ def bits16(t):
 class Session:
     """One communicator (single rank) + a non-default stream."""
 
-    def __init__(self, rank_size=1, rank=0):
+    def __init__(self, rank_size=1, rank=0, legacy_routing=False):
+        """legacy_routing: the communicator's dispatches route with the count + place launches even where the
+        one-launch routing applies (the library reads TILEXR_EP_ROUTING when a communicator is created)."""
         torch.cuda.set_device(0)
-        self.comm = ep.Comm(rank_size, rank)
+        previous = os.environ.get("TILEXR_EP_ROUTING")
+        if legacy_routing:
+            os.environ["TILEXR_EP_ROUTING"] = "legacy"
+        else:
+            os.environ.pop("TILEXR_EP_ROUTING", None)
+        try:
+            self.comm = ep.Comm(rank_size, rank)
+        finally:
+            if previous is None:
+                os.environ.pop("TILEXR_EP_ROUTING", None)
+            else:
+                os.environ["TILEXR_EP_ROUTING"] = previous
         self.stream = torch.cuda.Stream()
         # torch's own work (fills, host copies, comparisons) goes on the same stream as the library calls, as a
         # caller that keeps a whole layer on one stream would have it

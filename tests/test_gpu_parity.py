@@ -44,12 +44,15 @@ SHAPES = [(7, 8, 2, 5), (64, 64, 4, 16), (33, 40, 3, 7), (16, 33, 2, 4), (300, 1
 
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
-def test_memory_dispatch_matches_oracle(shape, dtype):
+@pytest.mark.parametrize("legacy_routing", [False, True])
+def test_memory_dispatch_matches_oracle(shape, dtype, legacy_routing):
     bs, h, K, E = shape
+    if legacy_routing and bs * K <= 2048:
+        pytest.skip("batches this small take the single-launch dispatch under either setting")
     rng = np.random.default_rng(sum(shape) + dtype)
     ids = ids_for(rng, bs, K, E, invalid=0.1)
     xt, xb = x_for(rng, bs, h, dtype)
-    with Session() as s:
+    with Session(legacy_routing=legacy_routing) as s:
         for mask_type in (ep.MASK_NONE, ep.MASK_TOKEN, ep.MASK_EXPERT):
             mask = None
             if mask_type == ep.MASK_TOKEN:
@@ -69,6 +72,89 @@ def test_memory_dispatch_matches_oracle(shape, dtype):
                 want = O.mem_dispatch(case, 0, xb[None], ids[None], None if mask is None else mask[None])
                 check_dispatch(got, want)
                 assert np.array_equal(got["send_counts"], want["send_counts"])
+
+
+ROUTING_SHAPES = [
+    # bs, h, K, E, invalid share, what the shape is there for
+    (1024, 16, 3, 5, 0.1),          # 3072 routes: not a multiple of 256 per wave, slots 1
+    (2049, 16, 1, 1, 0.0),          # one expert, topK 1
+    (683, 16, 3, 2048, 0.05),       # as many experts as the tables hold, most of them without a route
+    (4096, 16, 8, 256, 0.0),        # 32 768 routes: the largest table of the eight-slot kernel
+    (4097, 16, 8, 256, 0.02),       # just beyond it: sixteen slots, the last waves hold nothing but padding
+    (8192, 16, 8, 64, 0.0),         # 65 536 routes: the largest table the one-launch routing takes
+    (8193, 16, 8, 64, 0.0),         # one token more: count + place
+    (3000, 16, 7, 37, 1.0),         # no route names an expert
+    (3000, 16, 6, 9, 0.0),          # few experts: thousands of routes per key, several per lane and slot
+]
+
+
+@pytest.mark.parametrize("case", ROUTING_SHAPES)
+def test_one_launch_routing_matches_oracle(case):
+    """The routing kernel that resolves every route's row in one launch (memory route, no mask, no capacity limit, up
+    to 65 536 routes), at the edges of what it takes; ids drawn with repeats within a token too.  Compared with the
+    oracle and, bit for bit, with the count + place routing on the same inputs."""
+    bs, h, K, E, invalid = case
+    rng = np.random.default_rng(bs * 31 + K * 7 + E)
+    ids = rng.integers(0, E, (bs, K)).astype(np.int32)          # repeats within a token allowed
+    if E == 9:
+        ids[:, 0] = 4                                           # one expert takes a route of every token
+    bad = rng.random(ids.shape) < invalid
+    ids[bad] = rng.choice([-1, -9, E, E + 3, 2 ** 31 - 1, -2 ** 31], size=int(bad.sum()))
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+    results = []
+    for legacy in (False, True):
+        with Session(legacy_routing=legacy) as s:
+            for nums_type in (0, 1):
+                out = alloc_dispatch_outputs(bs, h, K, E)
+                counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
+                st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                              out["token_nums"], counts, ep.DT_BF16, s.stream,
+                                              token_nums_type=nums_type, row_index_map=out["row_map"])
+                assert st == 0
+                s.sync()
+                expect = "ep_route_count_kernel" if legacy or bs * K > 65536 else "ep_route_rows_kernel"
+                assert ep.last_kernel_name(s.comm, ep.K_COUNT) == expect
+                got = fetch(out, "send_counts", counts)
+                want = O.mem_dispatch(O.Case(1, bs, h, K, E, token_nums_type=nums_type), 0, xb[None], ids[None])
+                check_dispatch(got, want)
+                assert np.array_equal(got["send_counts"], want["send_counts"])
+                # the row map is the inverse of the tuples, -1 where a route has no row
+                rm = np.full(bs * K, -1, np.int32)
+                n = want["rows"]
+                rm[want["assist"][:n, 1] * K + want["assist"][:n, 2]] = np.arange(n, dtype=np.int32)
+                assert np.array_equal(got["row_map"].reshape(-1), rm)
+                results.append(got)
+    for name in ("assist", "expand_x", "token_nums", "send_counts", "row_map"):
+        assert np.array_equal(results[0][name], results[2][name]), name
+
+
+def test_one_launch_routing_with_unaligned_tables():
+    """An id table that is not 16-byte aligned takes the count + place routing; an unaligned tuple array takes the
+    one-launch routing with four-byte stores."""
+    bs, h, K, E = 1500, 32, 4, 24
+    rng = np.random.default_rng(77)
+    ids = ids_for(rng, bs, K, E, invalid=0.05)
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+    want = O.mem_dispatch(O.Case(1, bs, h, K, E, token_nums_type=1), 0, xb[None], ids[None])
+    n = want["rows"]
+    with Session() as s:
+        for shift_ids, shift_assist in ((1, 0), (0, 1)):
+            out = alloc_dispatch_outputs(bs, h, K, E)
+            counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
+            d_ids = torch.zeros((bs * K + 4,), dtype=torch.int32, device=DEV)
+            d_ids[shift_ids:shift_ids + bs * K] = torch.from_numpy(ids.reshape(-1)).to(DEV)
+            assist = torch.full((bs * K * 4 + 4,), -77, dtype=torch.int32, device=DEV)
+            torch.cuda.synchronize()
+            st = ep.dispatch_memory(xt, d_ids[shift_ids:], s.comm, bs, h, K, E, out["expand_x"], out["token_nums"], counts,
+                                    assist[shift_assist:], ep.DT_BF16, s.stream)
+            assert st == 0
+            s.sync()
+            assert ep.last_kernel_name(s.comm, ep.K_COUNT) == ("ep_route_count_kernel" if shift_ids else "ep_route_rows_kernel")
+            got = assist.cpu().numpy()[shift_assist:shift_assist + bs * K * 4].reshape(-1, 4)
+            assert np.array_equal(got[:n], want["assist"][:n])
+            assert np.all(got[n:] == -77)
+            assert np.array_equal(out["expand_x"].cpu().numpy()[:n], want["expand_x"][:n])
+            assert np.array_equal(counts.cpu().numpy(), want["send_counts"])
 
 
 @pytest.mark.parametrize("shape", SHAPES[:6])

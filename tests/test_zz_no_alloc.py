@@ -26,11 +26,14 @@ def _call(fn, s, x, ids, bs, h, K, E, out):
               ep.DT_BF16, s.stream)
 
 
-def test_no_alloc_dispatch_matches_the_allocating_entry_point():
-    # every shape takes the count + scatter path (more than 2048 routes), which is the one that needs scratch
+@pytest.mark.parametrize("legacy_routing", [False, True])
+def test_no_alloc_dispatch_matches_the_allocating_entry_point(legacy_routing):
+    # every shape has more than 2048 routes: routing launch(es) + scatter, the path that needs scratch (the row of every
+    # route and the kept-row count with the one-launch routing; ranks, histograms, offsets and the ticket word, which the
+    # call has to clear, with the count + place routing)
     shapes = [(4096, 1024, 8, 256), (700, 512, 6, 48), (4096, 1024, 8, 256), (1031, 264, 4, 7)]
     rng = np.random.default_rng(20)
-    with Session() as s:
+    with Session(legacy_routing=legacy_routing) as s:
         free_before = None
         for call, (bs, h, K, E) in enumerate(shapes):
             ids = np.stack([rng.permutation(E)[:K] for _ in range(bs)]).astype(np.int32)

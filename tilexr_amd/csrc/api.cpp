@@ -102,6 +102,16 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
         }
     }
     const CountScratchLayout plan = PlanCountScratch(n, numKeys, experts, expertHist);
+    int maskMode = kMaskNone;
+    if (p.xActiveMask != nullptr && !memoryRoute) {
+        maskMode = kMaskPerToken;              // reference: tilexr_ep_dispatch_helpers.h:3-21
+    } else if (p.xActiveMask != nullptr) {
+        maskMode = p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT ? kMaskPerRoute : kMaskTokenPrefix;
+    }
+    // One launch resolves every route's row where the id table is small enough for every workgroup to read all of it
+    // (ep_rows.hip); otherwise count (ticket, last workgroup scans) and place, the latter folded into the scatter
+    // unless something needs the rows ahead of it.
+    const bool oneLaunch = memoryRoute && !comm->legacyRouting && RouteRowsFits(p.expertIds, n, numKeys, maskMode, p.expertCapacity);
     void *scratchBase = nullptr;
     if (p.noAlloc) {
         // this call may not allocate: the per-GPU static array or nothing
@@ -113,8 +123,9 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
             return TileXR::TILEXR_ERROR_NOT_SUPPORT;     // DispatchMemory has said why
         }
         scratchBase = staticScratch;
-        // the array keeps what the previous call left: the count kernel's ticket has to start at zero
-        if (ClearScratchWord(scratchBase, stream) != hipSuccess) {
+        // the array keeps what the previous call left: the count kernel's ticket has to start at zero (the one-launch
+        // routing keeps nothing in scratch but its outputs)
+        if (!oneLaunch && ClearScratchWord(scratchBase, stream) != hipSuccess) {
             return TileXR::TILEXR_ERROR_MKIRT;
         }
     } else {
@@ -126,65 +137,30 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     const CountScratch scratch = CarveCountScratch(scratchBase, plan, expertHist);
     int32_t *rowOf = p.rowIndexMapOut != nullptr ? p.rowIndexMapOut :
         reinterpret_cast<int32_t *>(static_cast<char *>(scratchBase) + plan.rowOfOff);
-
-    RouteCountLaunch count {};
-    count.ids = p.expertIds;
-    count.mask = reinterpret_cast<const uint8_t *>(p.xActiveMask);
-    if (p.xActiveMask == nullptr) {
-        count.maskMode = kMaskNone;
-    } else if (!memoryRoute) {
-        count.maskMode = kMaskPerToken;        // reference: tilexr_ep_dispatch_helpers.h:3-21
-    } else {
-        count.maskMode = p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT ? kMaskPerRoute : kMaskTokenPrefix;
-    }
-    count.bs = p.bs;
-    count.topK = p.topK;
-    count.numExperts = experts;
-    count.keyDiv = keyDiv;
-    count.numKeys = numKeys;
-    count.capacity = p.expertCapacity;
-    count.scratch = scratch;
-    count.sendCountsOut = memoryRoute ? p.epRecvCountsOut : nullptr;
-    count.recvCountOut = memoryRoute ? nullptr : p.epRecvCountsOut;
-    count.expertTokenNumsOut = p.expertTokenNumsOut;
-    count.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
-    count.stream = stream;
     // the scatter kernel that copies per route wants the token rows close by
     const bool warm = ScatterCopiesPerRoute(p.x, p.expandXOut, p.bs, p.h, p.topK, static_cast<int>(p.quantMode));
-    count.warmRows = warm ? p.x : nullptr;
-    count.warmBytes = p.bs * p.h * 2;
-    int ret = Timed(comm, kKernelCount, stream, "route count", [&] { return LaunchRouteCount(count); });
-    if (ret != kOk) {
-        return ret;
-    }
-    if (!memoryRoute && p.tpRecvCountsOut != nullptr) {
-        // reference: tilexr_ep_combine_helpers.h:93-95 mirrors the per-source count into tpRecvCounts
-        if (hipMemcpyAsync(p.tpRecvCountsOut, p.epRecvCountsOut, sizeof(int32_t), hipMemcpyDeviceToDevice, stream) !=
-            hipSuccess) {
-            return TileXR::TILEXR_ERROR_INTERNAL;
-        }
-    }
-
+    int ret = kOk;
     RoutePlaceLaunch place {};
-    place.ids = p.expertIds;
-    place.bs = p.bs;
-    place.topK = p.topK;
-    place.keyDiv = keyDiv;
-    place.numKeys = numKeys;
-    place.capacity = p.expertCapacity;
-    place.scratch = scratch;
-    place.srcRank = comm->rank;
-    place.expertIdBias = static_cast<int32_t>(p.sharedExpertNum);
-    place.rowOf = rowOf;
-    place.assist = p.assistInfoForCombineOut;
-    place.stream = stream;
-    // The scatter kernel can resolve the rows of its own tokens.  A separate launch is needed when the row map and the
-    // assist tuples have to be complete before the first row lands (metaReadyEvent), and it pays when readiness flags
-    // are published: a workgroup that publishes stays until its stores have landed, and resolving the row first (three
-    // dependent loads) makes that stay longer (measured on 4096 x 7168 x top-8: scatter 105 us fused, 87 + 4 us apart).
-    const bool separatePlace = p.tileFlagsOut != nullptr || p.metaReadyEvent != nullptr;
-    if (separatePlace) {
-        ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
+    bool separatePlace = false;
+    if (oneLaunch) {
+        RouteRowsLaunch rows {};
+        rows.ids = p.expertIds;
+        rows.bs = p.bs;
+        rows.topK = p.topK;
+        rows.numKeys = numKeys;
+        rows.srcRank = comm->rank;
+        rows.expertIdBias = static_cast<int32_t>(p.sharedExpertNum);
+        rows.rowOf = rowOf;
+        rows.assist = p.assistInfoForCombineOut;
+        rows.totalRowsOut = scratch.keyOffset + numKeys;
+        rows.sendCountsOut = p.epRecvCountsOut;
+        rows.expertTokenNumsOut = p.expertTokenNumsOut;
+        rows.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
+        rows.warmRows = warm ? p.x : nullptr;
+        rows.warmBytes = p.bs * p.h * 2;
+        rows.stream = stream;
+        comm->lastKernel[kKernelCount] = "ep_route_rows_kernel";
+        ret = Timed(comm, kKernelCount, stream, "route rows", [&] { return LaunchRouteRows(rows); });
         if (ret != kOk) {
             return ret;
         }
@@ -193,13 +169,73 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
             return TileXR::TILEXR_ERROR_INTERNAL;
         }
     } else {
-        place.rowOf = p.rowIndexMapOut;      // only written when the caller asked for the map
+        RouteCountLaunch count {};
+        count.ids = p.expertIds;
+        count.mask = reinterpret_cast<const uint8_t *>(p.xActiveMask);
+        count.maskMode = maskMode;
+        count.bs = p.bs;
+        count.topK = p.topK;
+        count.numExperts = experts;
+        count.keyDiv = keyDiv;
+        count.numKeys = numKeys;
+        count.capacity = p.expertCapacity;
+        count.scratch = scratch;
+        count.sendCountsOut = memoryRoute ? p.epRecvCountsOut : nullptr;
+        count.recvCountOut = memoryRoute ? nullptr : p.epRecvCountsOut;
+        count.expertTokenNumsOut = p.expertTokenNumsOut;
+        count.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
+        count.stream = stream;
+        count.warmRows = warm ? p.x : nullptr;
+        count.warmBytes = p.bs * p.h * 2;
+        comm->lastKernel[kKernelCount] = "ep_route_count_kernel";
+        ret = Timed(comm, kKernelCount, stream, "route count", [&] { return LaunchRouteCount(count); });
+        if (ret != kOk) {
+            return ret;
+        }
+        if (!memoryRoute && p.tpRecvCountsOut != nullptr) {
+            // reference: tilexr_ep_combine_helpers.h:93-95 mirrors the per-source count into tpRecvCounts
+            if (hipMemcpyAsync(p.tpRecvCountsOut, p.epRecvCountsOut, sizeof(int32_t), hipMemcpyDeviceToDevice, stream) !=
+                hipSuccess) {
+                return TileXR::TILEXR_ERROR_INTERNAL;
+            }
+        }
+
+        place.ids = p.expertIds;
+        place.bs = p.bs;
+        place.topK = p.topK;
+        place.keyDiv = keyDiv;
+        place.numKeys = numKeys;
+        place.capacity = p.expertCapacity;
+        place.scratch = scratch;
+        place.srcRank = comm->rank;
+        place.expertIdBias = static_cast<int32_t>(p.sharedExpertNum);
+        place.rowOf = rowOf;
+        place.assist = p.assistInfoForCombineOut;
+        place.stream = stream;
+        // The scatter kernel can resolve the rows of its own tokens.  A separate launch is needed when the row map and
+        // the assist tuples have to be complete before the first row lands (metaReadyEvent), and it pays when readiness
+        // flags are published: a workgroup that publishes stays until its stores have landed, and resolving the row
+        // first (three dependent loads) makes that stay longer (measured on 4096 x 7168 x top-8: scatter 105 us fused,
+        // 87 + 4 us apart).
+        separatePlace = p.tileFlagsOut != nullptr || p.metaReadyEvent != nullptr;
+        if (separatePlace) {
+            ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
+            if (ret != kOk) {
+                return ret;
+            }
+            if (p.metaReadyEvent != nullptr &&
+                hipEventRecord(static_cast<hipEvent_t>(p.metaReadyEvent), stream) != hipSuccess) {
+                return TileXR::TILEXR_ERROR_INTERNAL;
+            }
+        } else {
+            place.rowOf = p.rowIndexMapOut;      // only written when the caller asked for the map
+        }
     }
 
     ScatterLaunch scatter {};
     scatter.x = p.x;
     scatter.rowOf = rowOf;
-    scatter.fusedPlace = separatePlace ? nullptr : &place;
+    scatter.fusedPlace = (oneLaunch || separatePlace) ? nullptr : &place;
     scatter.bs = p.bs;
     scatter.h = p.h;
     scatter.topK = p.topK;
@@ -546,8 +582,7 @@ const char *TileXREpLastKernelName(TileXRCommPtr comm, int kernel)
     if (c == nullptr || kernel < 0 || kernel > kKernelReduce) {
         return nullptr;
     }
-    static const char *const fixed[5] = {"ep_route_count_kernel", "ep_route_place_kernel", nullptr, "ep_invert_kernel",
-        nullptr};
+    static const char *const fixed[5] = {nullptr, "ep_route_place_kernel", nullptr, "ep_invert_kernel", nullptr};
     std::lock_guard<std::mutex> lock(c->mu);
     return fixed[kernel] != nullptr ? fixed[kernel] : c->lastKernel[kernel];
 }

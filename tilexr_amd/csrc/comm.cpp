@@ -3,6 +3,7 @@
 // Stands in for the part of libtile-comm that the EP host code calls (reference: src/comm/comm_wrap.cpp:173-182,
 // src/comm/tilexr_comm.cpp:1235-1238).  Nothing here talks to another process or another device.
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <unordered_set>
 
@@ -160,6 +161,8 @@ int TileXRCommInitRankLocal(int rankSize, int rank, TileXRCommPtr *comm)
     EpComm *c = new EpComm();
     c->world = world;
     c->rank = rank;
+    const char *routing = std::getenv("TILEXR_EP_ROUTING");
+    c->legacyRouting = routing != nullptr && std::strcmp(routing, "legacy") == 0;
     c->host.rank = rank;
     c->host.localRank = rank;
     c->host.rankSize = rankSize;

@@ -123,6 +123,8 @@ struct EpComm {
     const void *lastFlagWords = nullptr;
     uint64_t lastFlagEpoch = 0;
     hipStream_t lastFlagStream = nullptr;
+    bool legacyRouting = false;       // TILEXR_EP_ROUTING=legacy when the communicator was created: dispatches route with
+                                      // the count + place launches even where the one-launch routing applies (tests)
     DebugState debug;                 // TileXREpSetDebugOptions
     hipEvent_t timing[5][2] = {};     // optional (start, stop) pairs around each kernel, see tilexr_ep.h
     const char *lastKernel[5] = {};   // name of the kernel template last launched for each kernel id

@@ -10,6 +10,7 @@
 #include <hip/hip_runtime.h>
 
 #include "ep_block_scan.hip.h"
+#include "ep_chunk_rank.hip.h"
 #include "ep_kernel_common.hip.h"
 #include "ep_launch.h"
 #include "ep_numerics.hip.h"
@@ -19,11 +20,6 @@
 namespace TileXREp {
 namespace {
 
-
-__device__ __forceinline__ unsigned long long LaneMaskLt()
-{
-    return (1ull << (threadIdx.x & (kWave - 1))) - 1ull;
-}
 
 // -------------------------------------------------------------------------------------------------------------
 // count: stable rank of every live route within (chunk, key), per-chunk key histogram, and -- in the last
@@ -36,15 +32,7 @@ __device__ __forceinline__ unsigned long long LaneMaskLt()
 // Route liveness: ids outside [0, E) are skipped (:686-687); mask modes are described in ep_launch.h.
 // -------------------------------------------------------------------------------------------------------------
 struct RouteCountArgs {
-    const int32_t *ids;
-    const uint8_t *mask;
-    int maskMode;
-    int bs;
-    int topK;
-    int numExperts;
-    int keyDiv;
-    int numKeys;
-    int keyBits;
+    ChunkRouteArgs r;
     int capacity;
     int numChunks;
     CountScratch s;
@@ -56,13 +44,10 @@ struct RouteCountArgs {
     int64_t warmVecs;
 };
 
-constexpr int kWarmLoads = 2;    // 16-byte loads per lane of a warming workgroup (8 KiB per workgroup; 11.4 us for 58.7 MB, 14.3 us with eight)
-
 // BPW = batches of 64 routes per wave: a workgroup counts 256 * BPW consecutive routes.
 template <int BPW>
 __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs a)
 {
-    constexpr int kChunkRoutes = kThreads * BPW;
     __shared__ int s_cnt[kWavesPerBlock * kMaxKeys];
     __shared__ int s_exp[kMaxKeys];
     __shared__ int s_tot[kMaxKeys];     // single-chunk launches: the chunk's (= the launch's) routes per key
@@ -70,35 +55,22 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     __shared__ int s_misc[4];
 
     const int tid = threadIdx.x;
-    const int wave = tid / kWave;
-    const int lane = tid & (kWave - 1);
-    const int n = a.bs * a.topK;
+    const int numKeys = a.r.numKeys;
+    const int numExperts = a.r.numExperts;
+    const int n = a.r.bs * a.r.topK;
     const int chunk = blockIdx.x;
     const bool expHist = a.s.chunkExpHist != nullptr;
 
     if (a.warmRows != nullptr && chunk >= a.numChunks) {
-        // Not a counting workgroup: reads 8 KiB of the token rows and drops them.  The scatter that follows finds the
-        // rows in the memory-side cache; when it has to fetch them from HBM between its own writes it runs at little
-        // more than half its speed (4096 x 7168 x top-8: 140 us instead of 83).
-        const int64_t base = static_cast<int64_t>(chunk - a.numChunks) * (kThreads * kWarmLoads) + tid;
-        u32x4 v[kWarmLoads];
-#pragma unroll
-        for (int i = 0; i < kWarmLoads; ++i) {
-            const int64_t at = base + static_cast<int64_t>(i) * kThreads;
-            v[i] = a.warmRows[at < a.warmVecs ? at : a.warmVecs - 1];
-        }
-#pragma unroll
-        for (int i = 0; i < kWarmLoads; ++i) {
-            asm volatile("" ::"v"(v[i]));
-        }
+        WarmTokenRows(a.warmRows, a.warmVecs, chunk - a.numChunks);     // not a counting workgroup
         return;
     }
 
-    for (int i = tid; i < kWavesPerBlock * a.numKeys; i += kThreads) {
+    for (int i = tid; i < kWavesPerBlock * numKeys; i += kThreads) {
         s_cnt[i] = 0;
     }
     if (expHist) {
-        for (int i = tid; i < a.numExperts; i += kThreads) {
+        for (int i = tid; i < numExperts; i += kThreads) {
             s_exp[i] = 0;
         }
     }
@@ -107,85 +79,21 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     }
     __syncthreads();
 
-    int liveLimit = n;
-    if (a.maskMode == kMaskTokenPrefix) {
-        // activeCnt = sum(mask); only the first activeCnt tokens are dispatched
-        // (reference: tilexr_ep_dispatch_memory_kernel.h:1387-1410, 1538-1544)
-        int local = 0;
-        for (int t = tid; t < a.bs; t += kThreads) {
-            local += a.mask[t] != 0 ? 1 : 0;
-        }
-        for (int off = kWave / 2; off >= 1; off >>= 1) {
-            local += __shfl_xor(local, off);
-        }
-        if (lane == 0) {
-            atomicAdd(&s_misc[0], local);
-        }
-        __syncthreads();
-        liveLimit = s_misc[0] * a.topK;
-    }
-
-    // phase A: load the wave's 64 * BPW consecutive routes (all loads in flight together), decide liveness and key
+    // phase A: the lane's routes, their keys, their peers within each batch of 64
+    const int liveLimit = ChunkLiveLimit(a.r, &s_misc[0]);
     int keys[BPW];
-    {
-        int e[BPW];
-        int m[BPW];
-#pragma unroll
-        for (int b = 0; b < BPW; ++b) {
-            const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
-            const bool inRange = i < n && i < liveLimit;
-            e[b] = inRange ? a.ids[i] : -1;
-            m[b] = 1;
-            if (a.maskMode == kMaskPerToken) {
-                m[b] = inRange ? a.mask[i / a.topK] : 0;
-            } else if (a.maskMode == kMaskPerRoute) {
-                m[b] = inRange ? a.mask[i] : 0;
-            }
-        }
-#pragma unroll
-        for (int b = 0; b < BPW; ++b) {
-            const bool live = e[b] >= 0 && e[b] < a.numExperts && m[b] != 0;
-            keys[b] = live ? (a.keyDiv == 1 ? e[b] : e[b] / a.keyDiv) : -1;
-            if (expHist && live) {
-                atomicAdd(&s_exp[e[b]], 1);
-            }
-        }
-    }
-    // lanes of a batch with equal keys find each other with one ballot per key bit; the bit loop is outermost so
-    // that the BPW batches give independent instruction streams
-    unsigned long long peers[BPW];
-#pragma unroll
-    for (int b = 0; b < BPW; ++b) {
-        peers[b] = __ballot(keys[b] >= 0);
-    }
-    for (int bit = 0; bit < a.keyBits; ++bit) {
-#pragma unroll
-        for (int b = 0; b < BPW; ++b) {
-            const bool one = keys[b] >= 0 && ((keys[b] >> bit) & 1);
-            const unsigned long long bal = __ballot(one);
-            peers[b] &= one ? bal : ~bal;
-        }
-    }
-    const unsigned long long lt = LaneMaskLt();
-    int packed[BPW];            // lanes of the same key before this one | lanes of the same key << 8
-#pragma unroll
-    for (int b = 0; b < BPW; ++b) {
-        const int before = __popcll(peers[b] & lt);
-        const int same = __popcll(peers[b]);
-        packed[b] = before | (same << 8);
-        if (keys[b] >= 0 && before == 0) {
-            atomicAdd(&s_cnt[wave * a.numKeys + keys[b]], same);      // one LDS atomic per distinct key of a batch
-        }
-    }
+    int packed[BPW];
+    ChunkRouteKeys<BPW>(a.r, chunk, liveLimit, expHist ? s_exp : nullptr, keys);
+    ChunkMatchPeers<BPW>(a.r, keys, s_cnt, packed);
     __syncthreads();
 
     // phase B: exclusive sum over the four waves; chunk totals to HBM
-    for (int key = tid; key < a.numKeys; key += kThreads) {
+    for (int key = tid; key < numKeys; key += kThreads) {
         int run = 0;
 #pragma unroll
         for (int w = 0; w < kWavesPerBlock; ++w) {
-            const int v = s_cnt[w * a.numKeys + key];
-            s_cnt[w * a.numKeys + key] = run;
+            const int v = s_cnt[w * numKeys + key];
+            s_cnt[w * numKeys + key] = run;
             run += v;
         }
         if (a.numChunks == 1) {
@@ -196,33 +104,19 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
         }
         // written through (agent scope): complete for the scanning workgroup, on whatever XCD it runs, once this
         // wave's stores have drained, with no write-back of the L2
-        __hip_atomic_store(&a.s.chunkHist[static_cast<int64_t>(chunk) * a.numKeys + key], run, __ATOMIC_RELAXED,
+        __hip_atomic_store(&a.s.chunkHist[static_cast<int64_t>(chunk) * numKeys + key], run, __ATOMIC_RELAXED,
             __HIP_MEMORY_SCOPE_AGENT);
     }
     if (expHist && a.numChunks > 1) {
-        for (int e = tid; e < a.numExperts; e += kThreads) {
-            __hip_atomic_store(&a.s.chunkExpHist[static_cast<int64_t>(chunk) * a.numExperts + e], s_exp[e],
+        for (int e = tid; e < numExperts; e += kThreads) {
+            __hip_atomic_store(&a.s.chunkExpHist[static_cast<int64_t>(chunk) * numExperts + e], s_exp[e],
                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
     }
     __syncthreads();
 
-    // phase C: batches in order; the running count of a key within the wave lives in LDS (a wave's LDS operations
-    // execute in program order, the barriers only stop the compiler from reordering them)
-    volatile int *cnt = s_cnt + wave * a.numKeys;
-#pragma unroll
-    for (int b = 0; b < BPW; ++b) {
-        const int key = keys[b];
-        const bool live = key >= 0;
-        const int before = packed[b] & 0xff;
-        const int base = live ? cnt[key] : 0;
-        __builtin_amdgcn_wave_barrier();
-        if (live && before == 0) {
-            cnt[key] = base + (packed[b] >> 8);
-        }
-        __builtin_amdgcn_wave_barrier();
-        packed[b] = live ? base + before : -1;
-    }
+    // phase C: rank of every route within (chunk, key)
+    ChunkRankRoutes<BPW>(a.r, keys, s_cnt, packed);
 
     // The last workgroup to arrive performs the scans.  Only the chunk histograms (stored in phase B, long since
     // on their way) have to be complete for it, so the ticket is taken before the rank stores are issued.
@@ -238,7 +132,7 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     }
 #pragma unroll
     for (int b = 0; b < BPW; ++b) {
-        const int i = chunk * kChunkRoutes + wave * (kChunkRoutes / kWavesPerBlock) + b * kWave + lane;
+        const int i = ChunkRouteIndex<BPW>(chunk, b);
         if (i < n) {
             a.s.localRank[i] = packed[b];
         }
@@ -250,7 +144,7 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
 
     // per key: exclusive sum over chunks (becomes the chunk's base rank within the key), total, kept
     int *kept = s_cnt;                 // reuse: [numKeys]
-    for (int key = tid; key < a.numKeys; key += kThreads) {
+    for (int key = tid; key < numKeys; key += kThreads) {
         int run = a.numChunks == 1 ? s_tot[key] : 0;
         // the loads of a batch are independent: one round trip per 32 chunks.  Whole batches run without a test per
         // load: this workgroup is alone on the launch's critical path and runs code nobody has fetched before it, so
@@ -258,7 +152,7 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
         // (hence also buffer accesses: the chunk's offset is a scalar, one instruction per load)
         constexpr int kBatch = 32;
         int32_t *col = a.s.chunkHist + key;
-        const int rowBytes = a.numKeys * 4;
+        const int rowBytes = numKeys * 4;
         int c0 = 0;
         if (a.numChunks > 1 && static_cast<int64_t>(a.numChunks) * rowBytes < (int64_t{1} << 31)) {
             // chunks past the last one lie outside the buffer: their loads return zero, their stores are dropped
@@ -290,14 +184,14 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int c = c0 + u;
-                v[u] = c < a.numChunks ? __hip_atomic_load(col + static_cast<int64_t>(c) * a.numKeys, __ATOMIC_RELAXED,
+                v[u] = c < a.numChunks ? __hip_atomic_load(col + static_cast<int64_t>(c) * numKeys, __ATOMIC_RELAXED,
                     __HIP_MEMORY_SCOPE_AGENT) : 0;
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 const int c = c0 + u;
                 if (c < a.numChunks) {
-                    col[static_cast<int64_t>(c) * a.numKeys] = run;
+                    col[static_cast<int64_t>(c) * numKeys] = run;
                     run += v[u];
                 }
             }
@@ -308,19 +202,19 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     }
     LdsBarrier();
     int *offs = s_cnt + kMaxKeys;      // [numKeys] exclusive offsets
-    for (int key = tid; key < a.numKeys; key += kThreads) {
+    for (int key = tid; key < numKeys; key += kThreads) {
         offs[key] = kept[key];
     }
     LdsBarrier();
-    const int totalRows = BlockExclusiveScan(offs, a.numKeys, s_part);
-    for (int key = tid; key < a.numKeys; key += kThreads) {
+    const int totalRows = BlockExclusiveScan(offs, numKeys, s_part);
+    for (int key = tid; key < numKeys; key += kThreads) {
         a.s.keyOffset[key] = offs[key];
         if (a.sendCountsOut != nullptr) {
             a.sendCountsOut[key] = offs[key] + kept[key];
         }
     }
     if (tid == 0) {
-        a.s.keyOffset[a.numKeys] = totalRows;
+        a.s.keyOffset[numKeys] = totalRows;
         if (a.recvCountOut != nullptr) {
             a.recvCountOut[0] = totalRows;
         }
@@ -331,41 +225,41 @@ __global__ __launch_bounds__(kThreads) void ep_route_count_kernel(RouteCountArgs
     //   coarser keys:    live routes per expert (reference: tilexr_ep_combine_helpers.h:49-80)
     int *etot = s_cnt + 2 * kMaxKeys;  // [numExperts]
     if (expHist) {
-        for (int e = tid; e < a.numExperts; e += kThreads) {
+        for (int e = tid; e < numExperts; e += kThreads) {
             int run = a.numChunks == 1 ? s_exp[e] : 0;
             for (int c = 0; c < a.numChunks && a.numChunks > 1; ++c) {
-                run += __hip_atomic_load(&a.s.chunkExpHist[static_cast<int64_t>(c) * a.numExperts + e], __ATOMIC_RELAXED,
+                run += __hip_atomic_load(&a.s.chunkExpHist[static_cast<int64_t>(c) * numExperts + e], __ATOMIC_RELAXED,
                     __HIP_MEMORY_SCOPE_AGENT);
             }
             etot[e] = run;
         }
     } else {
-        for (int e = tid; e < a.numExperts; e += kThreads) {
-            etot[e] = e < a.numKeys ? kept[e] : 0;
+        for (int e = tid; e < numExperts; e += kThreads) {
+            etot[e] = e < numKeys ? kept[e] : 0;
         }
     }
     LdsBarrier();
-    for (int e = tid; e < a.numExperts; e += kThreads) {
+    for (int e = tid; e < numExperts; e += kThreads) {
         a.s.expertTotal[e] = etot[e];
     }
     if (a.expertTokenNumsOut != nullptr) {
         if (a.tokenNumsType == 0 && !expHist) {
             // keys are experts: the inclusive prefix sum is the one already computed for the counts output
-            for (int e = tid; e < a.numExperts; e += kThreads) {
-                a.expertTokenNumsOut[e] = e < a.numKeys ? static_cast<int64_t>(offs[e]) + kept[e] : totalRows;
+            for (int e = tid; e < numExperts; e += kThreads) {
+                a.expertTokenNumsOut[e] = e < numKeys ? static_cast<int64_t>(offs[e]) + kept[e] : totalRows;
             }
         } else if (a.tokenNumsType == 0) {
             int *pref = s_cnt + 3 * kMaxKeys;
-            for (int e = tid; e < a.numExperts; e += kThreads) {
+            for (int e = tid; e < numExperts; e += kThreads) {
                 pref[e] = etot[e];
             }
             LdsBarrier();
-            BlockExclusiveScan(pref, a.numExperts, s_part);
-            for (int e = tid; e < a.numExperts; e += kThreads) {
+            BlockExclusiveScan(pref, numExperts, s_part);
+            for (int e = tid; e < numExperts; e += kThreads) {
                 a.expertTokenNumsOut[e] = static_cast<int64_t>(pref[e]) + etot[e];
             }
         } else {
-            for (int e = tid; e < a.numExperts; e += kThreads) {
+            for (int e = tid; e < numExperts; e += kThreads) {
                 a.expertTokenNumsOut[e] = etot[e];
             }
         }
@@ -455,15 +349,6 @@ __global__ __launch_bounds__(kThreads) void ep_invert_kernel(InvertArgs a)
     }
 }
 
-int KeyBits(int64_t numKeys)
-{
-    int bits = 0;
-    while ((1ll << bits) < numKeys) {
-        ++bits;
-    }
-    return bits;
-}
-
 } // namespace
 
 // -------------------------------------------------------------------------------------------------------------
@@ -501,15 +386,15 @@ CountScratchLayout PlanCountScratch(int64_t routes, int64_t numKeys, int64_t num
 hipError_t LaunchRouteCount(const RouteCountLaunch &l)
 {
     RouteCountArgs a {};
-    a.ids = l.ids;
-    a.mask = l.mask;
-    a.maskMode = l.maskMode;
-    a.bs = static_cast<int>(l.bs);
-    a.topK = static_cast<int>(l.topK);
-    a.numExperts = static_cast<int>(l.numExperts);
-    a.keyDiv = static_cast<int>(l.keyDiv);
-    a.numKeys = static_cast<int>(l.numKeys);
-    a.keyBits = KeyBits(l.numKeys);
+    a.r.ids = l.ids;
+    a.r.mask = l.mask;
+    a.r.maskMode = l.maskMode;
+    a.r.bs = static_cast<int>(l.bs);
+    a.r.topK = static_cast<int>(l.topK);
+    a.r.numExperts = static_cast<int>(l.numExperts);
+    a.r.keyDiv = static_cast<int>(l.keyDiv);
+    a.r.numKeys = static_cast<int>(l.numKeys);
+    a.r.keyBits = KeyBits(l.numKeys);
     a.capacity = static_cast<int>(l.capacity);
     const int64_t n = l.bs * l.topK;
     const int shift = l.scratch.chunkShift;
@@ -523,7 +408,7 @@ hipError_t LaunchRouteCount(const RouteCountLaunch &l)
     if (a.numChunks > 0 && l.warmRows != nullptr && l.warmBytes >= 16 && Aligned16(l.warmRows)) {
         a.warmRows = static_cast<const u32x4 *>(l.warmRows);
         a.warmVecs = l.warmBytes / 16;
-        blocks += static_cast<unsigned>((a.warmVecs + kThreads * kWarmLoads - 1) / (kThreads * kWarmLoads));
+        blocks += WarmWorkgroups(a.warmVecs);
     }
     const dim3 grid(blocks);
     switch (shift) {

@@ -70,6 +70,29 @@ struct RouteCountLaunch {
     hipStream_t stream;
 };
 
+// Memory route, one rank, keys = experts, no mask, no capacity limit: rows and assist tuples of all routes in one launch
+// (ep_rows.hip), for id tables small enough that every workgroup reads the whole table itself.
+constexpr int kRowsTableRoutes = 65536;
+struct RouteRowsLaunch {
+    const int32_t *ids;
+    int64_t bs;
+    int64_t topK;
+    int64_t numKeys;
+    int32_t srcRank;
+    int32_t expertIdBias;
+    int32_t *rowOf;              // [n] out: row of each route, -1 = none
+    int32_t *assist;             // [rows, 4] out
+    int32_t *totalRowsOut;       // [1] out: rows kept
+    int32_t *sendCountsOut;      // optional [numKeys] inclusive sum of kept rows
+    int64_t *expertTokenNumsOut; // optional [numKeys]
+    int tokenNumsType;
+    const void *warmRows;        // as RouteCountLaunch
+    int64_t warmBytes;
+    hipStream_t stream;
+};
+bool RouteRowsFits(const int32_t *ids, int64_t routes, int64_t numKeys, int maskMode, int64_t capacity);
+hipError_t LaunchRouteRows(const RouteRowsLaunch &l);
+
 struct RoutePlaceLaunch {
     const int32_t *ids;
     int64_t bs;

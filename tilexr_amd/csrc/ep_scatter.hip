@@ -149,6 +149,7 @@ __device__ __forceinline__ void PublishRows(const ScatterArgs &a, const int *pos
 // 448 lanes per workgroup), 92-95 us with three to fourteen, 105-130 us with one; 93 us for "one workgroup writes all
 // topK rows", and 132 us when the workgroups of a token are spread over the XCDs.
 constexpr int kRouteVecs = 2;
+constexpr unsigned kRouteCapLdsBytes = 27 * 1024;    // 160 KiB of LDS per compute unit: five workgroups fit
 template <int THREADS, int V, bool WT>
 __global__ __launch_bounds__(THREADS) void ep_scatter_route_kernel(ScatterArgs a)
 {
@@ -519,7 +520,12 @@ void LaunchByMode(const ScatterLaunch &l, const ScatterArgs &a)
                     hipLaunchKernelGGL((ep_scatter_route_kernel<kThreads, kRouteVecs, true>), blocks, dim3(kThreads), 0,
                         l.stream, a);
                 } else {
-                    hipLaunchKernelGGL((ep_scatter_route_kernel<kThreads, kRouteVecs, false>), blocks, dim3(kThreads), 0,
+                    // Workgroups that only look their row up in the row map are short-lived, and eight of them per
+                    // compute unit keep more stores in flight than this memory system digests (4096 x 7168 x top-8:
+                    // 88.9 us; seven 86.5, five 81.7, four 85.3, three 98.2).  Unused dynamic LDS caps them at five.
+                    // Workgroups that resolve their row themselves (three dependent loads) are slow enough as they are.
+                    const unsigned capLds = a.place.ids == nullptr ? kRouteCapLdsBytes : 0u;
+                    hipLaunchKernelGGL((ep_scatter_route_kernel<kThreads, kRouteVecs, false>), blocks, dim3(kThreads), capLds,
                         l.stream, a);
                 }
             } else {

@@ -296,6 +296,7 @@ int RunDispatchMulti(EpComm *comm, const EpDispatchParams &p, bool memoryRoute, 
     count.scratch = scratch;
     count.tokenNumsType = static_cast<int>(p.expertTokenNumsType);
     count.stream = stream;
+    comm->lastKernel[kKernelCount] = "ep_route_count_kernel";
     int ret = Timed(comm, kKernelCount, stream, "route count", [&] { return LaunchRouteCount(count); });
     if (ret != kOk) {
         return ret;
