@@ -40,21 +40,90 @@ def measured_traffic(workload, kernel):
     return None
 
 
-def trace_avg_us(workload, kernel):
-    """Average duration of a kernel from the committed rocprofv3 kernel-trace summary of this workload
-    (profiles/ep_dispatch_combine_<workload>_kernel_stats.txt: table rows `<kernel template> calls avg_us ...`), or
-    None.  Event-bracketed times read a few microseconds above it (an event record holds the queue)."""
-    path = os.path.join(ROOT, "profiles", f"ep_dispatch_combine_{workload}_kernel_stats.txt")
+def trace_avg_us(path, section, kernel):
+    """Average duration of a kernel from a committed rocprofv3 kernel-trace summary (profiles/*_kernel_stats.txt): the
+    table row `<kernel template> calls avg_us ...` of the section whose header line `== [<section>] ...` names the
+    configuration that was run, or None.  Event-bracketed times read a few microseconds above it (an event record
+    holds the queue)."""
+    path = os.path.join(ROOT, path)
     if not os.path.exists(path) or not kernel:
         return None
+    inside = False
     for line in open(path):
-        if line.startswith(kernel):
+        if line.startswith("=="):
+            inside = f"[{section}]" in line
+        elif inside and line.startswith(kernel):
             parts = line.rsplit(None, 5)
             try:
                 return float(parts[-4])
             except (ValueError, IndexError):
                 return None
     return None
+
+
+def run_timed_passes(torch, ep, step, steps, comm, use_events, stride):
+    """The timed region, twice over exactly `steps` steps each.  The first pass carries nothing but the steps: `value`
+    comes from it.  The second records a (start, stop) pair of HIP events around the scatter and the reduce kernel on
+    every `stride`-th step (the library records them on the stream the kernels are launched on); an event record between
+    two kernels holds the queue for about 5 us on this GPU (about 22 us per bracketed step), which is why the pass that
+    `value` is taken from has none.  Returns (seconds of pass 1, seconds of pass 2 or None, {step: event pairs})."""
+    import time as _time
+    torch.cuda.synchronize()
+    t0 = _time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    elapsed = _time.perf_counter() - t0
+    if not use_events:
+        return elapsed, None, {}
+    sampled = [i for i in range(steps) if i % stride == 0]
+    pairs = {i: [(ep.HipEvent(timing=True), ep.HipEvent(timing=True)) for _ in range(2)] for i in sampled}
+    torch.cuda.synchronize()
+    t0 = _time.perf_counter()
+    for i in range(steps):
+        if i in pairs:
+            ep.set_kernel_timing_events(comm, ep.K_SCATTER, *pairs[i][0])
+            ep.set_kernel_timing_events(comm, ep.K_REDUCE, *pairs[i][1])
+            step()
+            ep.set_kernel_timing_events(comm, ep.K_SCATTER, None, None)
+            ep.set_kernel_timing_events(comm, ep.K_REDUCE, None, None)
+        else:
+            step()
+    torch.cuda.synchronize()
+    return elapsed, _time.perf_counter() - t0, pairs
+
+
+def kernel_event_stats(pairs, byte_counts):
+    """Per-kernel figures from the event pairs of run_timed_passes: {name: {...}} for (scatter, reduce)."""
+    kernels = {}
+    for which, (name, nbytes) in enumerate(byte_counts):
+        times = sorted(p[which][0].elapsed_ms(p[which][1]) * 1e3 for p in pairs.values())
+        avg = sum(times) / len(times)
+        kernels[name] = {"avg_us": round(avg, 2), "min_us": round(times[0], 2), "p50_us": round(times[len(times) // 2], 2),
+                         "max_us": round(times[-1], 2), "launches_timed": len(times), "algorithmic_bytes": nbytes,
+                         "achieved_GBps": round(nbytes / (avg * 1e-6) / 1e9, 1)}
+    return kernels
+
+
+def roofline_of(kernels, dom, kernel_name, traffic, traffic_source, trace_us, trace_source):
+    """The roofline object of the dominant kernel.  `achieved` / `frac` price the kernel by the committed rocprofv3
+    kernel-trace summary when it holds a row for the very kernel template that was launched (no event records between
+    kernels there); the figure from this run's HIP events stands beside it under `event_timed` and takes its place when
+    no summary matches."""
+    nbytes = kernels[dom]["algorithmic_bytes"]
+    event = {"avg_launch_us": kernels[dom]["avg_us"], "launches_timed": kernels[dom]["launches_timed"],
+             "achieved": kernels[dom]["achieved_GBps"], "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4)}
+    roofline = {"bound": "hbm", "kernel": kernel_name, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "algorithmic_bytes_per_launch": nbytes, "traffic": traffic, "traffic_source": traffic_source if traffic else None,
+                "event_timed": event}
+    if trace_us:
+        achieved = nbytes / (trace_us * 1e-6) / 1e9
+        roofline.update(achieved=round(achieved, 1), frac=round(achieved / HBM_PEAK_GBPS, 4), avg_launch_us=trace_us,
+                        frac_source=f"rocprofv3 kernel trace, {trace_source}")
+    else:
+        roofline.update(achieved=event["achieved"], frac=event["frac"], avg_launch_us=event["avg_launch_us"],
+                        frac_source="HIP events of this run (no committed kernel-trace row for this kernel template)")
+    return roofline
 
 
 def parse():
@@ -101,8 +170,9 @@ def parse():
                    help="skip the memory-system yardsticks (probe kernels of the library) reported under `ceilings`")
     p.add_argument("--no-rotate-leg", action="store_true",
                    help="skip the extra leg that feeds every step a different input tensor (inputs not cache-resident)")
-    p.add_argument("--event-stride", type=int, default=10,
-                   help="record the per-kernel events on every N-th timed step")
+    p.add_argument("--event-stride", type=int, default=0,
+                   help="record the per-kernel events on every N-th step of the second timed pass (0: steps // 16, at "
+                        "least 1, so that even a short run brackets eight launches and more)")
     p.add_argument("--calibrate-copy", action="store_true",
                    help="also launch a plain 256 MiB read + 256 MiB write kernel before the warm-up, as the known-size "
                         "yardstick for hardware-counter runs")
@@ -359,22 +429,9 @@ def main_moonep(args):
 
     dispatch_bytes, combine_bytes = workloads.moonep_algorithmic_bytes(s, k, h)
     use_events = not args.no_kernel_events
-    stride = max(1, args.event_stride)
-    sampled = [i for i in range(args.steps) if i % stride == 0] if use_events else []
-    pairs = {i: [(ep.HipEvent(timing=True), ep.HipEvent(timing=True)) for _ in range(2)] for i in sampled}
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        if i in pairs:       # the events are set on rank 0's communicator and bracket the launch for the whole world
-            ep.set_kernel_timing_events(comms[0], ep.K_SCATTER, *pairs[i][0])
-            ep.set_kernel_timing_events(comms[0], ep.K_REDUCE, *pairs[i][1])
-            step()
-            ep.set_kernel_timing_events(comms[0], ep.K_SCATTER, None, None)
-            ep.set_kernel_timing_events(comms[0], ep.K_REDUCE, None, None)
-        else:
-            step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    stride = args.event_stride if args.event_stride > 0 else max(1, args.steps // 16)
+    # the events are set on rank 0's communicator and bracket the launch for the whole world
+    elapsed, event_pass_s, pairs = run_timed_passes(torch, ep, step, args.steps, comms[0], use_events, stride)
     names = {"scatter": ep.last_kernel_name(comms[0], ep.K_SCATTER), "reduce": ep.last_kernel_name(comms[0], ep.K_REDUCE)}
 
     ev = [ep.HipEvent(timing=True) for _ in range(3)]
@@ -421,17 +478,14 @@ def main_moonep(args):
     kernels, roofline = {}, None
     if use_events:
         # one launch of the scatter / reduce kernel covers every rank of the world
-        for which, (name, nbytes) in enumerate((("scatter", world * dispatch_bytes), ("reduce", world * combine_bytes))):
-            times = sorted(pairs[i][which][0].elapsed_ms(pairs[i][which][1]) * 1e3 for i in sampled)
-            avg = sum(times) / len(times)
-            kernels[name] = {"avg_us": round(avg, 2), "min_us": round(times[0], 2), "p50_us": round(times[len(times) // 2], 2),
-                             "max_us": round(times[-1], 2), "launches_timed": len(times), "algorithmic_bytes": nbytes,
-                             "achieved_GBps": round(nbytes / (avg * 1e-6) / 1e9, 1)}
+        kernels = kernel_event_stats(pairs, (("scatter", world * dispatch_bytes), ("reduce", world * combine_bytes)))
         dom = "scatter" if kernels["scatter"]["avg_us"] >= kernels["reduce"]["avg_us"] else "reduce"
-        roofline = {"bound": "hbm", "kernel": names[dom], "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS,
-                    "unit": "GB/s", "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4),
-                    "traffic": measured_traffic(f"{w.name}_r{world}", dom), "avg_launch_us": kernels[dom]["avg_us"],
-                    "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
+        trace_file = f"profiles/moonep_dispatch_combine_{w.name}_kernel_stats.txt"
+        section = f"ranks={world} {'saved' if args.moon_saved else 'built'} plan"
+        roofline = roofline_of(kernels, dom, names[dom], measured_traffic(f"{w.name}_r{world}", dom),
+                               f"profiles/hbm_traffic_{w.name}_r{world}.txt", trace_avg_us(trace_file, section, names[dom]),
+                               trace_file)
+        roofline["event_pass_us_per_layer"] = round(event_pass_s / args.steps * 1e6, 2)
     ceilings = None
     if not args.no_ceilings:
         ceilings = measured_ceilings(ep, torch, streams[0], dev)
@@ -588,29 +642,9 @@ def main():
     kept_rows = int(send_counts[-1].item())
     dispatch_bytes, combine_bytes = workloads.algorithmic_bytes(w, kept_rows, inverse_index=True)
 
-    # Per-kernel HIP events inside the timed region, on a sample of the steps only: an event record between two
-    # kernels holds the queue for about 5 us on this GPU, so bracketing both kernels on every step would add about
-    # 20 us to a 200 us step.  Every `stride`-th step carries a (start, stop) pair around the scatter and the
-    # reduce kernel; the library records them on the stream the kernels are launched on.
     use_events = not args.no_kernel_events
-    stride = max(1, args.event_stride)
-    sampled = [i for i in range(args.steps) if i % stride == 0] if use_events else []
-    pairs = {i: [(ep.HipEvent(timing=True), ep.HipEvent(timing=True)) for _ in range(2)] for i in sampled}
-    d_ev = [ep.HipEvent(timing=True) for _ in range(3)]
-
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(args.steps):
-        if i in pairs:
-            ep.set_kernel_timing_events(comm, ep.K_SCATTER, *pairs[i][0])
-            ep.set_kernel_timing_events(comm, ep.K_REDUCE, *pairs[i][1])
-            step()
-            ep.set_kernel_timing_events(comm, ep.K_SCATTER, None, None)
-            ep.set_kernel_timing_events(comm, ep.K_REDUCE, None, None)
-        else:
-            step()
-    torch.cuda.synchronize()
-    elapsed = time.perf_counter() - t0
+    stride = args.event_stride if args.event_stride > 0 else max(1, args.steps // 16)
+    elapsed, event_pass_s, pairs = run_timed_passes(torch, ep, step, args.steps, comm, use_events, stride)
     kernel_names = {"scatter": ep.last_kernel_name(comm, ep.K_SCATTER), "reduce": ep.last_kernel_name(comm, ep.K_REDUCE)}
 
     if status.item() != 0:
@@ -844,24 +878,18 @@ def main():
     roofline = None
     kernels = {}
     if use_events:
-        for which, (name, nbytes) in enumerate((("scatter", dispatch_bytes), ("reduce", combine_bytes))):
-            times = sorted(pairs[i][which][0].elapsed_ms(pairs[i][which][1]) * 1e3 for i in sampled)
-            avg = sum(times) / len(times)
-            kernels[name] = {"avg_us": round(avg, 2), "min_us": round(times[0], 2), "p50_us": round(times[len(times) // 2], 2),
-                             "max_us": round(times[-1], 2), "launches_timed": len(times), "algorithmic_bytes": nbytes,
-                             "achieved_GBps": round(nbytes / (avg * 1e-6) / 1e9, 1)}
+        kernels = kernel_event_stats(pairs, (("scatter", dispatch_bytes), ("reduce", combine_bytes)))
         dom = "scatter" if kernels["scatter"]["avg_us"] >= kernels["reduce"]["avg_us"] else "reduce"
-        roofline = {"bound": "hbm", "kernel": kernel_names[dom],
-                    "achieved": kernels[dom]["achieved_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": round(kernels[dom]["achieved_GBps"] / HBM_PEAK_GBPS, 4),
-                    "traffic": measured_traffic(w.name, dom),
-                    "avg_launch_us": kernels[dom]["avg_us"], "algorithmic_bytes_per_launch": kernels[dom]["algorithmic_bytes"]}
-        # the same kernel by the committed rocprofv3 kernel trace of this workload (no event records between kernels)
-        trace_us = trace_avg_us(w.name, kernel_names[dom])
-        if trace_us:
-            roofline["kernel_trace"] = {"avg_launch_us": trace_us, "source": f"profiles/ep_dispatch_combine_{w.name}_kernel_stats.txt",
-                                        "achieved": round(kernels[dom]["algorithmic_bytes"] / (trace_us * 1e-6) / 1e9, 1),
-                                        "frac": round(kernels[dom]["algorithmic_bytes"] / (trace_us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+        trace_file = f"profiles/ep_dispatch_combine_{w.name}_kernel_stats.txt"
+        roofline = roofline_of(kernels, dom, kernel_names[dom], measured_traffic(w.name, dom), f"profiles/hbm_traffic_{w.name}.txt",
+                               trace_avg_us(trace_file, schedule, kernel_names[dom]), trace_file)
+        # what the whole dispatch fetches and writes by the same counters: the scatter plus the routing launch, whose
+        # extra workgroups read the token rows once so that the scatter finds them in the memory-side cache
+        side_traffic = {k: measured_traffic(w.name, k) for k in ("scatter", "routing")}
+        if all(side_traffic.values()):
+            total = sum(side_traffic.values())
+            roofline["dispatch_traffic"] = dict(side_traffic, total=total, over_algorithmic=round(total / dispatch_bytes, 4))
+        roofline["event_pass_us_per_layer"] = round(event_pass_s / args.steps * 1e6, 2)
 
     ceilings = None
     if not args.no_ceilings:
@@ -881,7 +909,7 @@ def main():
         "ms_per_step": round(ms_per_step, 5), "us_per_layer": round(ms_per_step * 1e3, 2),
         "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": dict(workloads.describe(w, ids), schedule=SCHEDULES[schedule],
+        "config": dict(workloads.describe(w, ids), schedule=SCHEDULES[schedule], overlap=schedule == "flags-overlapped",
                        tile_rows=args.tile_rows if uses_flags else None, schedule_calibration_us=calibration,
                        other_schedules=other, expert_stage=expert_stage, graph_replay=graph_replay, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),

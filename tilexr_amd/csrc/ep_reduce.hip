@@ -130,11 +130,13 @@ void LaunchVecKernels(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, 
 
 void LaunchQuantKernels(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
 {
+    // flags that were all published before this launch began take the kernels without the waiting code
     const bool flags = a.tileFlags != nullptr;
+    const bool settled = flags && a.flagsSettled != 0;
     if (l.bf16) {
-        (flags ? LaunchReduceQuantBf16Flags : LaunchReduceQuantBf16)(g, v, l, a, gridLimit);
+        (settled ? LaunchReduceQuantBf16Settled : flags ? LaunchReduceQuantBf16Flags : LaunchReduceQuantBf16)(g, v, l, a, gridLimit);
     } else {
-        (flags ? LaunchReduceQuantFp16Flags : LaunchReduceQuantFp16)(g, v, l, a, gridLimit);
+        (settled ? LaunchReduceQuantFp16Settled : flags ? LaunchReduceQuantFp16Flags : LaunchReduceQuantFp16)(g, v, l, a, gridLimit);
     }
 }
 

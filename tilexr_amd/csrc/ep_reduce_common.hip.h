@@ -55,6 +55,8 @@ void LaunchReduceQuantBf16(int g, int v, const ReduceLaunch &l, const ReduceArgs
 void LaunchReduceQuantBf16Flags(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
 void LaunchReduceQuantFp16(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
 void LaunchReduceQuantFp16Flags(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceQuantBf16Settled(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
+void LaunchReduceQuantFp16Settled(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit);
 
 namespace {
 
@@ -198,14 +200,17 @@ __device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
 // before the rows and looked at after the last of them has been used: the memory counter runs in order, so by then it
 // has long arrived, and nothing waits for it on the way (an ordinary load: the words are final, this XCD's L2 may keep
 // them).
-__device__ __forceinline__ uint64_t SettledWordLoad(const ReduceArgs &a, int slotRow)
+// (Only the half of the word that holds the epoch is loaded: one register less for the whole K loop, and the kernels
+// that use this are tuned to the register.)
+__device__ __forceinline__ uint32_t SettledWordLoad(const ReduceArgs &a, int slotRow)
 {
-    return slotRow >= 0 ? a.tileFlags[TileOf(a, slotRow)] : 0ull;
+    static_assert(__BYTE_ORDER__ == __ORDER_LITTLE_ENDIAN__, "the epoch is the word's upper half");
+    return slotRow >= 0 ? reinterpret_cast<const uint32_t *>(a.tileFlags + TileOf(a, slotRow))[1] : 0u;
 }
 
-__device__ __forceinline__ bool SettledWordMissing(const ReduceArgs &a, int slotRow, uint64_t word, int waveLane)
+__device__ __forceinline__ bool SettledWordMissing(const ReduceArgs &a, int slotRow, uint32_t epochOfWord, int waveLane)
 {
-    const bool missing = __ballot(slotRow >= 0 && !TileWordReady(word, a.flagEpoch)) != 0;
+    const bool missing = __ballot(slotRow >= 0 && epochOfWord != static_cast<uint32_t>(a.flagEpoch)) != 0;
     if (missing && waveLane == 0 && a.deviceStatus != nullptr) {
         atomicExch(a.deviceStatus, 1);
     }

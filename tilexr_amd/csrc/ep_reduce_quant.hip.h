@@ -1,6 +1,10 @@
 // reduce of quantised rows (int8 with a scale per row, fp8 e4m3 with a scale per 128 columns): ep_reduce.hip says what
-// is computed.  Compiled once per (element type, with / without readiness flags): the including file sets
-// TILEXR_REDUCE_BF16, TILEXR_REDUCE_FLAGS and TILEXR_REDUCE_ENTRY.
+// is computed.  Compiled once per (element type, readiness flags): the including file sets TILEXR_REDUCE_BF16,
+// TILEXR_REDUCE_FLAGS and TILEXR_REDUCE_ENTRY.  TILEXR_REDUCE_FLAGS: 0 no flags; 1 flags that may still be pending
+// (the launch can wait: tokens are claimed, rows and scales are read past the L2); 2 flags that were all published
+// before the launch began (a dispatch earlier on the same stream): nothing waits, every wave only looks at the words
+// of its token's tiles, and the kernel carries none of the waiting code -- with it in the same kernel the registers
+// of the claim loop cost the fp8 kernel a wave per SIMD and the settled case ran 4 us behind the kernel without flags.
 #if !defined(TILEXR_REDUCE_BF16) || !defined(TILEXR_REDUCE_FLAGS) || !defined(TILEXR_REDUCE_ENTRY)
 #error "include from ep_reduce_quant_*.hip"
 #endif
@@ -14,8 +18,12 @@ namespace {
 // columns.  Each value is dequantised, rounded to the output element type, then accumulated exactly like an ordinary
 // row (fp32, k order, separate multiply and add).  Rows are a quarter the bytes of bf16 rows, so a lane owns 16
 // consecutive columns per vector (one 16-byte load) and KB rows are kept in flight at once.
-template <int G, int V, int INQ, bool BF16, bool FL>
-__global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL && INQ == TILEXR_EP_QUANT_FP8_BLOCK128) ? 6 : 7) : 1) void ep_reduce_quant_kernel(ReduceArgs a)
+constexpr int kFlagsNone = 0;
+constexpr int kFlagsMayWait = 1;
+constexpr int kFlagsSettled = 2;
+
+template <int G, int V, int INQ, bool BF16, int FL>
+__global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL == kFlagsMayWait && INQ == TILEXR_EP_QUANT_FP8_BLOCK128) ? 6 : 7) : 1) void ep_reduce_quant_kernel(ReduceArgs a)
 {
     constexpr int kTokens = kThreads / G;
     constexpr int KB = V >= 4 ? 2 : 4;
@@ -50,11 +58,12 @@ __global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL && INQ == TILEXR_
             slotRow = s_row[tg][waveLane];
             myWeight = s_w[tg][waveLane];
         }
-        const bool checkWords = FL && a.flagsSettled != 0;
-        const uint64_t tileWord = checkWords ? SettledWordLoad(a, slotRow) : 0ull;
-        const bool expired = FL && __ballot(slotRow == kRowExpired) != 0;
+        constexpr bool checkWords = FL == kFlagsSettled;
+        const bool expired = FL == kFlagsMayWait && __ballot(slotRow == kRowExpired) != 0;
         const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !expired;
         const int myRow = active ? slotRow : -1;
+        // (an inactive token's output is zeros whatever its words say: only the rows that are read are asked about)
+        const uint32_t tileWord = checkWords ? SettledWordLoad(a, myRow) : 0u;
         const uint64_t live = __ballot(myRow >= 0);
 
         float acc[V][16];
@@ -151,7 +160,7 @@ __global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL && INQ == TILEXR_
                 }
             }
         };
-        const bool throughMemory = FL && a.flagsSettled == 0;
+        constexpr bool throughMemory = FL == kFlagsMayWait;
         if (throughMemory) {
             accumulate(std::false_type {}, std::true_type {});
         } else {
@@ -195,12 +204,18 @@ __global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL && INQ == TILEXR_
                 }
             }
         }
-        const bool keep = active && !(checkWords && SettledWordMissing(a, slotRow, tileWord, waveLane));
+        const bool keep = active && !(checkWords && SettledWordMissing(a, myRow, tileWord, waveLane));
         if (tokOk) {
             u32x4 *dst = reinterpret_cast<u32x4 *>(static_cast<char *>(a.y) + static_cast<int64_t>(token) * a.h * 2);
+            // the lane index once more, from the thread index and out of the optimiser's sight: values derived from it
+            // for these stores are then computed here instead of being kept (or spilled) across the K loop, where every
+            // register counts towards the seventh wave per SIMD
+            int storeThread = threadIdx.x;
+            asm volatile("" : "+v"(storeThread));
+            const int storeLane = storeThread % G;
 #pragma unroll
             for (int j = 0; j < V; ++j) {
-                const int idx = j * G + lane;
+                const int idx = j * G + storeLane;
                 if (idx < vecs) {
 #pragma unroll
                     for (int half = 0; half < 2; ++half) {
@@ -219,11 +234,11 @@ __global__ __launch_bounds__(kThreads, (V == 1 && BF16) ? ((FL && INQ == TILEXR_
             }
         }
     };
-    ForEachGroup<FL>(a, groups, kTokens, tokenAt, load, reduceUnit);
+    ForEachGroup<FL == kFlagsMayWait>(a, groups, kTokens, tokenAt, load, reduceUnit);
 }
 
 
-template <int G, int V, bool BF16, bool FL>
+template <int G, int V, bool BF16, int FL>
 void LaunchQuant(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
 {
     constexpr int kTokens = kThreads / G;
@@ -245,7 +260,7 @@ void LaunchQuant(const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
 void TILEXR_REDUCE_ENTRY(int g, int v, const ReduceLaunch &l, const ReduceArgs &a, int gridLimit)
 {
     constexpr bool kBf16 = TILEXR_REDUCE_BF16;
-    constexpr bool kFlags = TILEXR_REDUCE_FLAGS;
+    constexpr int kFlags = TILEXR_REDUCE_FLAGS;
     if (g == kWave && v == 1) {
         LaunchQuant<kWave, 1, kBf16, kFlags>(l, a, gridLimit);
     } else if (g == 2 * kWave && v == 1) {

@@ -1,5 +1,5 @@
-// One compilation of ep_reduce_quant.hip.h: bf16 rows, without tile readiness flags.
+// One compilation of ep_reduce_quant.hip.h: bf16 rows, no tile readiness flags.
 #define TILEXR_REDUCE_BF16 true
-#define TILEXR_REDUCE_FLAGS false
+#define TILEXR_REDUCE_FLAGS 0
 #define TILEXR_REDUCE_ENTRY LaunchReduceQuantBf16
 #include "ep_reduce_quant.hip.h"

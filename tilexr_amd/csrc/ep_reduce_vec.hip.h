@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             myWeight = s_w[tg][waveLane];
         }
         const bool checkWords = FL && a.flagsSettled != 0;
-        const uint64_t tileWord = checkWords ? SettledWordLoad(a, slotRow) : 0ull;
+        const uint32_t tileWord = checkWords ? SettledWordLoad(a, slotRow) : 0u;
         const bool expired = FL && __ballot(slotRow == kRowExpired) != 0;
         const bool active = tokOk && (a.tokenMask == nullptr || a.tokenMask[token] != 0) && !expired;
         const int myRow = active ? slotRow : -1;
