@@ -15,12 +15,15 @@ import pytest
 
 import hostlib as H
 
-(LAUNCH, ROW_WRITE, COUNTER_ADD, COUNTER_RESET, FLAG_STORE, FLAG_POLL, WAIT_EXPIRED, ROW_READ, ROUND_END) = range(9)
+(LAUNCH, ROW_WRITE, COUNTER_ADD, COUNTER_RESET, FLAG_STORE, FLAG_POLL, WAIT_EXPIRED, ROW_READ, ROUND_END, TOKEN_CLAIM,
+ TOKEN_REDUCED, TOKEN_ZEROED, SLEEP) = range(13)
 (READ_BEFORE_WRITE, FLAG_STALE_EPOCH, FLAG_NO_PRODUCER, DEADLOCK, DOUBLE_PUBLISH, PUBLISH_BEFORE_LANDED,
- COUNTER_NOT_ZERO, WRONG_WORD, READ_WITHOUT_WAIT, WAIT_EXPIRED_EARLY) = range(1, 11)
+ COUNTER_NOT_ZERO, WRONG_WORD, READ_WITHOUT_WAIT, WAIT_EXPIRED_EARLY, TOKEN_REDUCED_WHILE_PENDING, TOKEN_CLAIMED_TWICE,
+ TOKEN_NEVER_CLAIMED) = range(1, 14)
 SERIAL, ROUND_ROBIN, RANDOM, CONSUMER_EAGER = range(4)
 (INJECT_NONE, INJECT_READ_WITHOUT_WAIT, INJECT_ACCEPT_ANY_EPOCH, INJECT_MISSING_PRODUCER, INJECT_DOUBLE_REPORT,
- INJECT_REPORT_BEFORE_WRITE, INJECT_CONSUMER_ENQUEUED_FIRST, INJECT_OLD_EPOCH_CONSUMER) = range(8)
+ INJECT_REPORT_BEFORE_WRITE, INJECT_CONSUMER_ENQUEUED_FIRST, INJECT_OLD_EPOCH_CONSUMER, INJECT_TRUST_WITHOUT_SCAN,
+ INJECT_CLAIM_NOT_ATOMIC, INJECT_CLAIM_SKIPS, INJECT_IMPATIENT_CONSUMER) = range(12)
 
 
 class Event(C.Structure):
@@ -33,7 +36,7 @@ class Finding(C.Structure):
 
 
 class Shape(C.Structure):
-    _fields_ = [(n, C.c_int32) for n in ("totalRows", "maxRows", "tileRows", "parts")]
+    _fields_ = [(n, C.c_int32) for n in ("totalRows", "maxRows", "tileRows", "parts", "tokens")]
 
 
 class Case(C.Structure):
@@ -75,7 +78,7 @@ def word(epoch, rows):
 # ---------------------------------------------------------------------------------------------------------------
 # (1) the rules, on hand-written traces: two rows of one part in one tile, one producer (agent 0), one consumer (1)
 # ---------------------------------------------------------------------------------------------------------------
-SHAPE = Shape(2, 2, 2, 1)
+SHAPE = Shape(2, 2, 2, 1, 0)
 E = 7
 
 
@@ -154,12 +157,56 @@ def test_publisher_side_rules():
     assert lib().TileXREpTraceFindingName(DEADLOCK) == b"DEADLOCK"
 
 
+def consumer_trace():
+    """The good trace with the consumer's token bookkeeping: one token (0) made of the tile's two rows, claimed, found
+    pending at the first look, seen ready by a scan, read and summed."""
+    t = good_trace()
+    t.insert(4, ev(TOKEN_CLAIM, 1, 1, part=4, word=0, epoch=E))                  # takes tokens [0, 4): only token 0 exists
+    t.insert(-1, ev(TOKEN_REDUCED, 1, 1, row=0, epoch=E))
+    return t
+
+
+def test_consumer_side_rules():
+    shape = Shape(2, 2, 2, 1, 1)
+    assert check(shape, consumer_trace()) == []
+    # the token is summed from a row that was read before its tile was published: the sum is the finding, on top of the read's own
+    t = consumer_trace()
+    store = next(i for i, e in enumerate(t) if e.kind == FLAG_STORE)
+    first_read = next(i for i, e in enumerate(t) if e.kind == ROW_READ)
+    t.insert(store, t.pop(first_read))
+    f = check(shape, t)
+    assert TOKEN_REDUCED_WHILE_PENDING in kinds(f)
+    assert [(x.row, x.tile) for x in f if x.kind == TOKEN_REDUCED_WHILE_PENDING] == [(0, 0)]
+    # two claims that overlap
+    t = consumer_trace()
+    t.insert(6, ev(TOKEN_CLAIM, 2, 1, part=2, word=0, epoch=E))
+    assert kinds(check(shape, t)) == [TOKEN_CLAIMED_TWICE]
+    # a token finished twice (summed, and given a row of zeros by somebody else)
+    t = consumer_trace()
+    t.insert(-1, ev(TOKEN_ZEROED, 2, 1, row=0, epoch=E))
+    assert kinds(check(shape, t)) == [TOKEN_CLAIMED_TWICE]
+    # claimed but never finished; and never claimed at all
+    t = [e for e in consumer_trace() if e.kind != TOKEN_REDUCED]
+    f = check(shape, t)
+    assert kinds(f) == [TOKEN_NEVER_CLAIMED] and f[0].row == 0
+    t = [e for e in consumer_trace() if e.kind != TOKEN_CLAIM]
+    assert kinds(check(shape, t)) == [TOKEN_NEVER_CLAIMED]
+    # a second round has to claim and finish its tokens again
+    t = consumer_trace() + [ev(ROUND_END, agent=-1, epoch=E + 1, round_=2)]
+    f = check(shape, t)
+    assert kinds(f) == [TOKEN_NEVER_CLAIMED] and f[0].round == 2
+    # without a token count the claim rules are off
+    assert check(SHAPE, [e for e in consumer_trace() if e.kind != TOKEN_CLAIM]) == []
+    assert lib().TileXREpTraceFindingName(TOKEN_REDUCED_WHILE_PENDING) == b"TOKEN_REDUCED_WHILE_PENDING"
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # (2) + (3) the model
 # ---------------------------------------------------------------------------------------------------------------
 def run(total, max_rows, tile_rows, parts, top_k=4, producers=4, consumers=3, rounds=2, scheduler=RANDOM, inject=0,
         budget=10_000, seed=1):
-    c = Case(Shape(total, max_rows, tile_rows, parts), top_k, producers, consumers, rounds, scheduler, inject, budget, seed)
+    tokens = (total + top_k - 1) // top_k
+    c = Case(Shape(total, max_rows, tile_rows, parts, tokens), top_k, producers, consumers, rounds, scheduler, inject, budget, seed)
     cap = 400_000
     events = (Event * cap)()
     n, wrong = C.c_int32(), C.c_int32()
@@ -186,6 +233,61 @@ def test_clean_runs_have_no_findings(shape, scheduler):
         assert sum(e.kind == ROW_WRITE for e in events) == 3 * total * parts
 
 
+@pytest.mark.parametrize("scheduler", [ROUND_ROBIN, RANDOM, CONSUMER_EAGER])
+def test_consumers_claim_hold_scan_and_reduce_as_the_kernels_do(scheduler):
+    """What the waiting combine's control flow promises, read off the trace of a clean run: every token is claimed once
+    and summed once, a consumer never holds more than four unfinished tokens, a sleep only follows a scan that found
+    nothing ready, and rows are only read by a consumer that has seen their tile published."""
+    total, top_k, consumers, rounds = 130, 4, 3, 2
+    tokens = (total + top_k - 1) // top_k
+    events, findings, wrong = run(total, 160, 16, 2, top_k=top_k, consumers=consumers, rounds=rounds, scheduler=scheduler, seed=9)
+    assert findings == [] and wrong == 0
+    for rnd in range(1, rounds + 1):
+        ev_r = [e for e in events if e.round == rnd]
+        claimed = sorted(t for e in ev_r if e.kind == TOKEN_CLAIM for t in range(e.word, e.word + e.part) if t < tokens)
+        assert claimed == list(range(tokens))
+        assert sorted(e.row for e in ev_r if e.kind == TOKEN_REDUCED) == list(range(tokens))
+        assert not any(e.kind in (TOKEN_ZEROED, WAIT_EXPIRED) for e in ev_r)
+        for agent in {e.agent for e in ev_r if e.kind == TOKEN_CLAIM}:
+            held = 0
+            polls_since_progress = 0
+            for e in (x for x in ev_r if x.agent == agent):
+                if e.kind == TOKEN_CLAIM:
+                    held += sum(1 for t in range(e.word, e.word + e.part) if t < tokens)
+                    assert held <= 4
+                elif e.kind == TOKEN_REDUCED:
+                    held -= 1
+                    polls_since_progress = 0
+                elif e.kind == FLAG_POLL:
+                    polls_since_progress += 1
+                elif e.kind == SLEEP:
+                    assert polls_since_progress > 0 and held > 0      # it looked, found nothing, and still owes tokens
+            assert held == 0
+    if scheduler == CONSUMER_EAGER:
+        assert any(e.kind == SLEEP for e in events)       # consumers that run ahead of their producers do back off
+
+
+def test_tokens_of_a_tile_that_is_never_published_get_zeros_not_partial_sums():
+    events, findings, wrong = run(100, 128, 8, 2, scheduler=RANDOM, inject=INJECT_MISSING_PRODUCER, budget=40, rounds=1, seed=5)
+    assert wrong == 0 and FLAG_NO_PRODUCER in kinds(findings)
+    zeroed = {e.row for e in events if e.kind == TOKEN_ZEROED}
+    assert zeroed
+    stored = {e.tile for e in events if e.kind == FLAG_STORE}
+    # a zeroed token contributes no row read, and no token was summed from a row of the tile that never came
+    for agent in {e.agent for e in events if e.kind == TOKEN_ZEROED}:
+        reads = 0
+        for e in (x for x in events if x.agent == agent):
+            if e.kind == ROW_READ:
+                reads += 1
+                assert e.tile in stored
+            elif e.kind == TOKEN_REDUCED:
+                assert reads > 0
+                reads = 0
+            elif e.kind == TOKEN_ZEROED:
+                assert reads == 0
+    assert TOKEN_REDUCED_WHILE_PENDING not in kinds(findings) and TOKEN_NEVER_CLAIMED not in kinds(findings)
+
+
 def test_trace_covers_the_two_level_counters():
     # tiles wider than 16 rows count groups first: both levels show up as counters of the trace
     events, findings, _ = run(130, 160, 64, 4, rounds=1)
@@ -205,6 +307,11 @@ def test_trace_covers_the_two_level_counters():
     (INJECT_CONSUMER_ENQUEUED_FIRST, RANDOM, {DEADLOCK}, False),
     (INJECT_OLD_EPOCH_CONSUMER, SERIAL, {FLAG_STALE_EPOCH}, None),          # polls meet the newer words
     (INJECT_OLD_EPOCH_CONSUMER, CONSUMER_EAGER, {FLAG_NO_PRODUCER}, None),  # the first dispatch + combine pair waits for an epoch nobody stores
+    # the consumer's own logic (ep_token_claim.h runs in the model; the mistakes are planted in its operations)
+    (INJECT_TRUST_WITHOUT_SCAN, CONSUMER_EAGER, {TOKEN_REDUCED_WHILE_PENDING, READ_BEFORE_WRITE, READ_WITHOUT_WAIT}, True),
+    (INJECT_CLAIM_NOT_ATOMIC, ROUND_ROBIN, {TOKEN_CLAIMED_TWICE}, None),
+    (INJECT_CLAIM_SKIPS, RANDOM, {TOKEN_NEVER_CLAIMED}, False),
+    (INJECT_IMPATIENT_CONSUMER, CONSUMER_EAGER, {WAIT_EXPIRED_EARLY}, False),
 ])
 def test_each_planted_mistake_is_reported(inject, scheduler, expect, wrong_tokens):
     events, findings, wrong = run(100, 128, 8, 2, scheduler=scheduler, inject=inject, budget=60, rounds=2, seed=5)
@@ -226,8 +333,8 @@ def test_each_planted_mistake_is_reported(inject, scheduler, expect, wrong_token
 
 
 def test_bad_cases_are_rejected():
-    c = Case(Shape(10, 5, 4, 1), 2, 1, 1, 1, 0, 0, 10, 1)          # maxRows < totalRows
+    c = Case(Shape(10, 5, 4, 1, 0), 2, 1, 1, 1, 0, 0, 10, 1)          # maxRows < totalRows
     n = C.c_int32()
     assert lib().TileXREpTraceRun(C.byref(c), None, 0, C.byref(n), None) == -1
-    c = Case(Shape(10, 16, 4, 1), 2, 1, 1, 1, 0, 0, 10, 1)
+    c = Case(Shape(10, 16, 4, 1, 5), 2, 1, 1, 1, 0, 0, 10, 1)
     assert lib().TileXREpTraceRun(C.byref(c), None, 0, C.byref(n), None) == -2 and n.value > 0     # trace does not fit

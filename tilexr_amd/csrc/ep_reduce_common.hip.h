@@ -12,6 +12,7 @@
 #include "ep_launch.h"
 #include "ep_numerics.hip.h"
 #include "ep_tile_publish.h"
+#include "ep_token_claim.h"
 #include "tilexr_ep.h"
 
 namespace TileXREp {
@@ -174,17 +175,13 @@ __device__ __forceinline__ bool TilePublished(const ReduceArgs &a, int row)
 }
 
 // Fills s_row / s_w for one token and deals with tile flags.  BLOCK: every slot waits (bounded) for its tile.  Otherwise
-// `mode` says what a slot does about its tile:
+// `mode` says what a slot does about its tile (ep_token_claim.h: SlotLooksAtTile, JudgeSlot):
 //   kRouteCheck    look once; a tile that is not there yet leaves kRowPending in the slot and the call returns true
 //                  ("come back later")
 //   kRouteTrusted  nothing: the caller has just seen every tile of this token published
 //   kRouteGiveUp   look once; a tile that is not there turns the slot into an expired one
 // An expired wait sets the launch's status word and leaves kRowExpired in the slot: the token then gets a row of zeros
 // (AnyExpired), never the sum of the rows that happened to be ready.
-constexpr int kRowExpired = -2;
-constexpr int kRowPending = -3;
-enum RouteMode : int { kRouteCheck = 0, kRouteTrusted = 1, kRouteGiveUp = 2 };
-
 __device__ __forceinline__ bool AnyExpired(const int *rows, int slots)
 {
     bool expired = false;
@@ -230,12 +227,13 @@ __device__ __forceinline__ bool LoadRoutes(const ReduceArgs &a, int token, bool 
         const float weight = (tokOk && a.expertScales != nullptr && k < a.topK) ?
             a.expertScales[static_cast<int64_t>(token) * a.topK + k] : 1.0f;
         int row = tokOk ? LookupRow(a, slot) : -1;
-        if (row >= 0 && a.tileFlags != nullptr && (BLOCK || mode != kRouteTrusted)) {
+        if (row >= 0 && a.tileFlags != nullptr && SlotLooksAtTile(BLOCK, mode)) {
             const bool there = BLOCK ? WaitTile(a, row) : TilePublished(a, row);
-            if (!there && !BLOCK && mode == kRouteCheck) {
+            const int verdict = JudgeSlot(BLOCK, mode, there);
+            if (verdict == kSlotComeBack) {
                 row = kRowPending;
                 pending = true;
-            } else if (!there) {
+            } else if (verdict == kSlotExpire) {
                 if (a.deviceStatus != nullptr) {
                     atomicExch(a.deviceStatus, 1);
                 }
@@ -278,128 +276,117 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
         return;
     }
     if constexpr (WAITS) {
-        // Groups are claimed, a few at a time, from a counter all workgroups share, not owned by block index: a
-        // workgroup holds at most kHeld groups that are not ready yet, and whoever has nothing left to wait for takes
-        // the next ones.  With fixed ownership the tokens of a producer's last tiles were reduced by the few workgroups
-        // that happened to own them, one after the other, while the rest had gone home.  Without a counter (a.claim
-        // null) the groups are dealt by block index as before.
-        constexpr int kHeld = 4;
+        // the control flow is ClaimAndReduce of ep_token_claim.h (the host-side model of the protocol runs the same
+        // code); what follows are its operations for a workgroup: atomics, barriers, LDS
         __shared__ uint32_t s_notReady;
-        __shared__ int s_group[kHeld];
+        __shared__ int s_group[kClaimHeld];
         __shared__ int s_base;
-        const int perGroup = tokensPerGroup * a.slots;
-        int dealt = static_cast<int>(blockIdx.x);       // next group by block index (no counter)
-        bool more = true;
-        uint32_t pending = 0u;                          // slots of s_group that hold a claimed, unfinished group
-        uint64_t idleSince = wall_clock64();
-        int backoff = 0;
-        for (;;) {
-            uint32_t fresh = 0u;
-            const uint32_t freeSlots = ~pending & ((1u << kHeld) - 1u);
-            if (more && freeSlots != 0u) {
-                const int want = __popc(freeSlots);
-                if (a.claim != nullptr) {
-                    __syncthreads();                    // readers of s_base from the previous refill are done
-                    if (threadIdx.x == 0) {
-                        s_base = static_cast<int>(__hip_atomic_fetch_add(a.claim, static_cast<uint32_t>(want), __ATOMIC_RELAXED,
-                            __HIP_MEMORY_SCOPE_AGENT));
-                    }
-                    __syncthreads();
+        struct WorkgroupEnv {
+            const ReduceArgs &a;
+            TokenAt &tokenAt;
+            Load &load;
+            Unit &unit;
+            uint32_t *notReady;
+            int *group;
+            int *base;
+            int perGroup;                   // (token, slot) pairs of a group
+            int tokensPerGroup;
+            int dealt;                      // next group by block index (launches without a claim counter)
+            uint64_t idleSince;
+
+            __device__ __forceinline__ int Claim(int want)
+            {
+                if (a.claim == nullptr) {
+                    return 0;
                 }
-                int next = a.claim != nullptr ? s_base : 0;
-                for (uint32_t m = freeSlots; m != 0u; m &= m - 1u) {
-                    const int slot = __builtin_ctz(m);
-                    int group;
-                    if (a.claim != nullptr) {
-                        group = next++;
-                    } else {
-                        group = dealt;
-                        dealt += static_cast<int>(gridDim.x);
-                    }
-                    if (group >= groups || group < 0) {
-                        more = false;
-                        continue;
-                    }
-                    if (threadIdx.x == 0) {
-                        s_group[slot] = group;
-                    }
-                    fresh |= 1u << slot;
-                }
-                pending |= fresh;
-                __syncthreads();
-            }
-            if (pending == 0u) {
-                break;                                  // nothing held, nothing left to claim
-            }
-            // One loop body does the work of all stages, so that the code of `unit` exists once: `todo` holds the slots
-            // to try now, `mode` says how (a first look at fresh groups; after a scan: trusted; giving up).
-            uint32_t todo = fresh;
-            int mode = kRouteCheck;
-            for (int pass = 0; pass < 2; ++pass) {
-                bool done = false;
-                for (; todo != 0u; todo &= todo - 1u) {
-                    const int i = __builtin_ctz(todo);
-                    const int group = s_group[i];
-                    __syncthreads();
-                    const bool waiting = load(group, mode);
-                    if (__syncthreads_or((mode == kRouteCheck && waiting) ? 1 : 0) != 0) {
-                        continue;                       // uniform: every lane gets the same answer
-                    }
-                    unit(group);
-                    pending &= ~(1u << i);
-                    idleSince = wall_clock64();
-                    backoff = 0;
-                    done = true;
-                }
-                if (pass == 1 || pending == 0u || (done && more)) {
-                    break;                              // free slots and groups to claim: refill before looking again
-                }
-                // all lanes together look once at every tile the held groups need
+                __syncthreads();            // readers of *base from the previous refill are done
                 if (threadIdx.x == 0) {
-                    s_notReady = 0u;
+                    *base = static_cast<int>(__hip_atomic_fetch_add(a.claim, static_cast<uint32_t>(want), __ATOMIC_RELAXED,
+                        __HIP_MEMORY_SCOPE_AGENT));
                 }
                 __syncthreads();
-                for (int idx = threadIdx.x; idx < kHeld * perGroup; idx += blockDim.x) {
+                return *base;
+            }
+            __device__ __forceinline__ int NextGroup(int *next)
+            {
+                if (a.claim != nullptr) {
+                    return (*next)++;
+                }
+                const int mine = dealt;
+                dealt += static_cast<int>(gridDim.x);
+                return mine;
+            }
+            __device__ __forceinline__ void Hold(int slot, int g)
+            {
+                if (threadIdx.x == 0) {
+                    group[slot] = g;
+                }
+            }
+            __device__ __forceinline__ void HoldDone()
+            {
+                __syncthreads();
+            }
+            __device__ __forceinline__ bool Try(int slot, int mode)
+            {
+                const int g = group[slot];
+                __syncthreads();
+                const bool waiting = load(g, mode);
+                if (__syncthreads_or((mode == kRouteCheck && waiting) ? 1 : 0) != 0) {
+                    return false;           // uniform: every lane gets the same answer
+                }
+                unit(g);
+                return true;
+            }
+            __device__ __forceinline__ uint32_t Scan(uint32_t pending)
+            {
+                // all lanes together look once at every tile the held groups need: one round trip for the lot
+                if (threadIdx.x == 0) {
+                    *notReady = 0u;
+                }
+                __syncthreads();
+                for (int idx = threadIdx.x; idx < kClaimHeld * perGroup; idx += blockDim.x) {
                     const int i = idx / perGroup;
                     if (((pending >> i) & 1u) == 0u) {
                         continue;
                     }
-                    const int token = tokenAt(s_group[i], (idx % perGroup) / a.slots);
+                    const int token = tokenAt(group[i], (idx % perGroup) / a.slots);
                     if (token < 0) {
                         continue;
                     }
                     const int row = LookupRow(a, static_cast<int64_t>(token) * a.slots + idx % a.slots);
                     if (row >= 0 && !TilePublished(a, row)) {
-                        atomicOr(&s_notReady, 1u << i);
+                        atomicOr(notReady, 1u << i);
                     }
                 }
                 __syncthreads();
-                todo = pending & ~s_notReady;
-                mode = kRouteTrusted;
-                if (todo != 0u) {
-                    continue;
-                }
+                return *notReady;
+            }
+            __device__ __forceinline__ bool GiveUpNow()
+            {
                 bool stop = false;
                 if (threadIdx.x == 0) {
                     stop = static_cast<int64_t>(wall_clock64() - idleSince) > a.waitTimeoutTicks ||
                         (a.deviceStatus != nullptr &&
                          __hip_atomic_load(a.deviceStatus, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0);
                 }
-                if (__syncthreads_or(stop ? 1 : 0) != 0) {
-                    todo = pending;                     // what is held is given up: rows of zeros, status word set
-                    mode = kRouteGiveUp;
-                    continue;
-                }
-                for (int r = 0; r < (1 << backoff); ++r) {
+                return __syncthreads_or(stop ? 1 : 0) != 0;
+            }
+            __device__ __forceinline__ void Touch()
+            {
+                idleSince = wall_clock64();
+            }
+            __device__ __forceinline__ void Sleep(int level)
+            {
+                for (int r = 0; r < (1 << level); ++r) {
                     __builtin_amdgcn_s_sleep(127);      // 127 x 64 clocks, about 3.5 us
                 }
-                backoff += backoff < 2 ? 1 : 0;
-                break;
             }
-        }
+        };
+        WorkgroupEnv env {a, tokenAt, load, unit, &s_notReady, s_group, &s_base, tokensPerGroup * a.slots, tokensPerGroup,
+            static_cast<int>(blockIdx.x), 0};
+        ClaimAndReduce(env, groups);
     }
 }
-
 
 } // namespace
 } // namespace TileXREp

@@ -2,12 +2,16 @@
 // consumer agents on host threads, one memory operation per step, and the ordering rules that a trace must obey.
 //
 // The producers call PublishLanded from ep_tile_publish.h -- the code the scatter kernels compile -- through an `Ops`
-// whose three memory operations are steps of the scheduler; the consumers apply TileWordReady, the test WaitTile
-// applies on the device.  What the model cannot see is the memory system below these operations (write-through
-// stores, per-XCD L2s): it checks the protocol's logic, the GPU tests check its implementation.
+// whose three memory operations are steps of the scheduler.  The consumers run ClaimAndReduce from ep_token_claim.h --
+// the control flow of a combine launch that may have to wait: tokens claimed from a shared counter, at most four held,
+// first look, scan, trusted pass, give-up -- through an `Env` whose looks at tile words, row reads and claims are steps
+// of the scheduler, with JudgeSlot deciding what a slot does about a tile that is not there and TileWordReady as the
+// acceptance test, all as on the device.  What the model cannot see is the memory system below these operations
+// (write-through stores, per-XCD L2s): it checks the protocol's logic, the GPU tests check its implementation.
 #include "flag_trace.h"
 
 #include <algorithm>
+#include <atomic>
 #include <condition_variable>
 #include <map>
 #include <mutex>
@@ -18,10 +22,19 @@
 #include <vector>
 
 #include "ep_tile_publish.h"
+#include "ep_token_claim.h"
 
 namespace {
 
+using TileXREp::ClaimAndReduce;
+using TileXREp::JudgeSlot;
+using TileXREp::kClaimHeld;
+using TileXREp::kRouteCheck;
+using TileXREp::kRouteTrusted;
+using TileXREp::kSlotComeBack;
+using TileXREp::kSlotExpire;
 using TileXREp::PublishLanded;
+using TileXREp::SlotLooksAtTile;
 using TileXREp::TileCounterWords;
 using TileXREp::TilePublishArgs;
 using TileXREp::TileWordReady;
@@ -188,6 +201,191 @@ struct TraceOps {
     }
 };
 
+// The operations of ep_token_claim.h for one consumer of the model: every look at a tile word, every row read and every
+// claim is a step of the scheduler and an event of the trace.  A group is one token.
+struct TraceClaimEnv {
+    Scheduler *sched;
+    const TileXREpTraceCase *c;
+    int agent;
+    int me;                                 // index among the consumers
+    uint64_t epoch;                         // what the rows of this round hold
+    uint64_t want;                          // the epoch this consumer waits for
+    const std::vector<int> *rowOf;          // [tokens, topK] rows of a token, -1 = none
+    const std::vector<uint64_t> *flags;
+    const std::vector<uint64_t> *contents;  // epoch that last wrote each (row, part)
+    uint32_t *claimCounter;
+    std::atomic<int> *status;               // the launch's status word
+    int *wrongTokens;
+    int held[kClaimHeld] = {-1, -1, -1, -1};
+    int idleScans = 0;
+
+    int RowOf(int token, int k) const { return (*rowOf)[static_cast<size_t>(token) * c->topK + k]; }
+    bool Ready(uint64_t word) const
+    {
+        return c->inject == TILEXR_INJECT_ACCEPT_ANY_EPOCH ? word != 0 : TileWordReady(word, want);
+    }
+    // one look at the word of the tile that holds `row`
+    bool Look(int row, bool *yield)
+    {
+        const int tile = row / c->shape.tileRows;
+        bool ok = false;
+        sched->Step(agent, yield, [&](TileXREpTraceEvent &e) {
+            const uint64_t w = (*flags)[static_cast<size_t>(tile)];
+            ok = Ready(w);
+            e.kind = TILEXR_TRACE_FLAG_POLL;
+            e.tile = tile;
+            e.row = row;
+            e.word = w;
+            e.epoch = want;
+            e.accepted = ok ? 1 : 0;
+            if (yield != nullptr) {
+                *yield = !ok;
+            }
+        });
+        return ok;
+    }
+
+    int Claim(int wantGroups)
+    {
+        uint32_t before = 0;
+        auto record = [&](TileXREpTraceEvent &e) {
+            e.kind = TILEXR_TRACE_TOKEN_CLAIM;
+            e.word = before;
+            e.part = wantGroups;
+            e.epoch = want;
+        };
+        if (c->inject == TILEXR_INJECT_CLAIM_NOT_ATOMIC) {
+            // read, then write back in a second step: another consumer's claim in between is lost
+            sched->Step(agent, nullptr, [&](TileXREpTraceEvent &e) {
+                before = *claimCounter;
+                e.kind = TILEXR_TRACE_SLEEP;
+                e.part = -1;
+            });
+            sched->Step(agent, nullptr, [&](TileXREpTraceEvent &e) {
+                *claimCounter = before + static_cast<uint32_t>(wantGroups);
+                record(e);
+            });
+            return static_cast<int>(before);
+        }
+        sched->Step(agent, nullptr, [&](TileXREpTraceEvent &e) {
+            before = *claimCounter;
+            *claimCounter += static_cast<uint32_t>(wantGroups);
+            if (c->inject == TILEXR_INJECT_CLAIM_SKIPS && me == 0) {
+                before += 1;                // takes [before + 1, before + 1 + want): one token falls through
+                *claimCounter += 1;
+            }
+            record(e);
+        });
+        return static_cast<int>(before);
+    }
+    int NextGroup(int *next) { return (*next)++; }
+    void Hold(int slot, int group) { held[slot] = group; }
+    void HoldDone() {}
+
+    bool Try(int slot, int mode)
+    {
+        const int token = held[slot];
+        // a consumer that does not wait reads whatever is there (the injected mistake of the first consumer)
+        if (c->inject == TILEXR_INJECT_READ_WITHOUT_WAIT && me == 0) {
+            mode = kRouteTrusted;
+        }
+        // the route table of the token: every slot with a row looks at its tile as the mode says (LoadRoutes)
+        bool comeBack = false;
+        int expiredRow = -1;
+        for (int k = 0; k < c->topK; ++k) {
+            const int row = RowOf(token, k);
+            if (row < 0 || !SlotLooksAtTile(false, mode)) {
+                continue;
+            }
+            bool yield = false;
+            const bool there = Look(row, mode == kRouteCheck ? &yield : nullptr);
+            const int verdict = JudgeSlot(false, mode, there);
+            comeBack |= verdict == kSlotComeBack;
+            if (verdict == kSlotExpire && expiredRow < 0) {
+                expiredRow = row;
+            }
+        }
+        if (mode == kRouteCheck && comeBack) {
+            return false;
+        }
+        if (expiredRow >= 0) {
+            sched->Step(agent, nullptr, [&](TileXREpTraceEvent &e) {
+                *status = 1;
+                e.kind = TILEXR_TRACE_WAIT_EXPIRED;
+                e.tile = expiredRow / c->shape.tileRows;
+                e.row = expiredRow;
+                e.epoch = want;
+            });
+            sched->Step(agent, nullptr, [&](TileXREpTraceEvent &e) {
+                e.kind = TILEXR_TRACE_TOKEN_ZEROED;      // a row of zeros, never a partial sum: nothing is read
+                e.row = token;
+                e.epoch = want;
+            });
+            return true;
+        }
+        bool bad = false;
+        for (int k = 0; k < c->topK; ++k) {
+            const int row = RowOf(token, k);
+            if (row < 0) {
+                continue;
+            }
+            sched->Step(agent, nullptr, [&](TileXREpTraceEvent &e) {
+                for (int p = 0; p < c->shape.parts; ++p) {
+                    bad |= (*contents)[static_cast<size_t>(row) * c->shape.parts + p] != epoch;
+                }
+                e.kind = TILEXR_TRACE_ROW_READ;
+                e.row = row;
+                e.tile = row / c->shape.tileRows;
+                e.epoch = want;
+            });
+        }
+        sched->Step(agent, nullptr, [&](TileXREpTraceEvent &e) {
+            e.kind = TILEXR_TRACE_TOKEN_REDUCED;
+            e.row = token;
+            e.epoch = want;
+        });
+        *wrongTokens += bad ? 1 : 0;
+        return true;
+    }
+
+    uint32_t Scan(uint32_t pending)
+    {
+        if (c->inject == TILEXR_INJECT_TRUST_WITHOUT_SCAN && me == 0) {
+            return 0u;                      // "all ready" without a look
+        }
+        uint32_t notReady = 0u;
+        for (int slot = 0; slot < kClaimHeld; ++slot) {
+            if (((pending >> slot) & 1u) == 0u) {
+                continue;
+            }
+            for (int k = 0; k < c->topK; ++k) {
+                const int row = RowOf(held[slot], k);
+                if (row >= 0 && !Look(row, nullptr)) {
+                    notReady |= 1u << slot;
+                }
+            }
+        }
+        return notReady;
+    }
+    bool GiveUpNow()
+    {
+        if (c->inject == TILEXR_INJECT_IMPATIENT_CONSUMER && me == 0) {
+            return true;
+        }
+        return ++idleScans > c->pollBudget || *status != 0;
+    }
+    void Touch() { idleScans = 0; }
+    void Sleep(int level)
+    {
+        bool yield = true;                  // nothing was ready: somebody else gets the turn
+        sched->Step(agent, &yield, [&](TileXREpTraceEvent &e) {
+            e.kind = TILEXR_TRACE_SLEEP;
+            e.part = level;
+            e.epoch = want;
+        });
+    }
+};
+
 int Priority(int kind)
 {
     switch (kind) {
@@ -196,6 +394,9 @@ int Priority(int kind)
         case TILEXR_FINDING_FLAG_NO_PRODUCER: return 2;
         case TILEXR_FINDING_READ_BEFORE_WRITE: return 3;
         case TILEXR_FINDING_READ_WITHOUT_WAIT: return 4;
+        case TILEXR_FINDING_TOKEN_REDUCED_WHILE_PENDING: return 4;
+        case TILEXR_FINDING_TOKEN_CLAIMED_TWICE: return 4;
+        case TILEXR_FINDING_TOKEN_NEVER_CLAIMED: return 4;
         case TILEXR_FINDING_PUBLISH_BEFORE_LANDED: return 5;
         case TILEXR_FINDING_DOUBLE_PUBLISH: return 6;
         case TILEXR_FINDING_WRONG_WORD: return 7;
@@ -221,6 +422,9 @@ const char *TileXREpTraceFindingName(int32_t kind)
         case TILEXR_FINDING_WRONG_WORD: return "WRONG_WORD";
         case TILEXR_FINDING_READ_WITHOUT_WAIT: return "READ_WITHOUT_WAIT";
         case TILEXR_FINDING_WAIT_EXPIRED_EARLY: return "WAIT_EXPIRED_EARLY";
+        case TILEXR_FINDING_TOKEN_REDUCED_WHILE_PENDING: return "TOKEN_REDUCED_WHILE_PENDING";
+        case TILEXR_FINDING_TOKEN_CLAIMED_TWICE: return "TOKEN_CLAIMED_TWICE";
+        case TILEXR_FINDING_TOKEN_NEVER_CLAIMED: return "TOKEN_NEVER_CLAIMED";
         default: return "UNKNOWN";
     }
 }
@@ -234,7 +438,8 @@ int TileXREpTraceRun(const TileXREpTraceCase *c, TileXREpTraceEvent *events, int
     const TileXREpTraceShape &sh = c->shape;
     if (sh.totalRows < 0 || sh.maxRows < sh.totalRows || sh.maxRows <= 0 || sh.tileRows <= 0 || sh.parts <= 0 ||
         sh.parts > 64 || c->topK <= 0 || c->producers <= 0 || c->consumers <= 0 || c->producers + c->consumers > 64 ||
-        c->rounds <= 0 || c->pollBudget <= 0 || c->scheduler < 0 || c->scheduler > TILEXR_SCHED_CONSUMER_EAGER) {
+        c->rounds <= 0 || c->pollBudget <= 0 || c->scheduler < 0 || c->scheduler > TILEXR_SCHED_CONSUMER_EAGER ||
+        (sh.tokens != 0 && sh.tokens != (sh.totalRows + c->topK - 1) / c->topK)) {
         return -1;
     }
     const int maxTiles = (sh.maxRows + sh.tileRows - 1) / sh.tileRows;
@@ -289,7 +494,8 @@ int TileXREpTraceRun(const TileXREpTraceCase *c, TileXREpTraceEvent *events, int
 
         Scheduler sched(agents, c->scheduler, rng(), &log, round);
         std::vector<int> wrongPerConsumer(static_cast<size_t>(c->consumers), 0);
-        int status = 0;      // the launch's status word: set by the first expired wait (only touched under the turn)
+        std::atomic<int> status {0};    // the launch's status word: set by the first expired wait
+        uint32_t claimCounter = 0;      // the device word a waiting launch's workgroups claim their tokens from: cleared per launch
         std::vector<std::thread> pool;
         for (int a = 0; a < agentsN; ++a) {
             if (a < c->producers) {
@@ -334,69 +540,9 @@ int TileXREpTraceRun(const TileXREpTraceCase *c, TileXREpTraceEvent *events, int
             } else {
                 pool.emplace_back([&, a] {
                     const int me = a - c->producers;
-                    const bool skipWait = c->inject == TILEXR_INJECT_READ_WITHOUT_WAIT && me == 0;
-                    const uint64_t want = c->inject == TILEXR_INJECT_OLD_EPOCH_CONSUMER ? epoch - 1 : epoch;
-                    for (int token = me; token < tokens; token += c->consumers) {
-                        bool expired = false;
-                        for (int k = 0; k < c->topK && !skipWait; ++k) {
-                            const int row = rowOf[static_cast<size_t>(token) * c->topK + k];
-                            if (row < 0) {
-                                continue;
-                            }
-                            const int tile = row / sh.tileRows;
-                            int failed = 0;
-                            while (true) {
-                                bool notReady = false;
-                                bool giveUp = false;
-                                sched.Step(a, &notReady, [&](TileXREpTraceEvent &e) {
-                                    const uint64_t w = flags[static_cast<size_t>(tile)];
-                                    const bool ok = c->inject == TILEXR_INJECT_ACCEPT_ANY_EPOCH ? w != 0 : TileWordReady(w, want);
-                                    e.kind = TILEXR_TRACE_FLAG_POLL;
-                                    e.tile = tile;
-                                    e.row = row;
-                                    e.word = w;
-                                    e.epoch = want;
-                                    e.accepted = ok ? 1 : 0;
-                                    notReady = !ok;
-                                    giveUp = !ok && status != 0;
-                                });
-                                if (!notReady) {
-                                    break;
-                                }
-                                if (giveUp || ++failed > c->pollBudget) {
-                                    sched.Step(a, nullptr, [&](TileXREpTraceEvent &e) {
-                                        status = 1;
-                                        e.kind = TILEXR_TRACE_WAIT_EXPIRED;
-                                        e.tile = tile;
-                                        e.row = row;
-                                        e.epoch = want;
-                                    });
-                                    expired = true;
-                                    break;
-                                }
-                            }
-                        }
-                        if (expired) {
-                            continue;          // the token gets a row of zeros: nothing is read
-                        }
-                        bool bad = false;
-                        for (int k = 0; k < c->topK; ++k) {
-                            const int row = rowOf[static_cast<size_t>(token) * c->topK + k];
-                            if (row < 0) {
-                                continue;
-                            }
-                            sched.Step(a, nullptr, [&](TileXREpTraceEvent &e) {
-                                for (int p = 0; p < sh.parts; ++p) {
-                                    bad |= contents[static_cast<size_t>(row) * sh.parts + p] != epoch;
-                                }
-                                e.kind = TILEXR_TRACE_ROW_READ;
-                                e.row = row;
-                                e.tile = row / sh.tileRows;
-                                e.epoch = want;
-                            });
-                        }
-                        wrongPerConsumer[static_cast<size_t>(me)] += bad ? 1 : 0;
-                    }
+                    TraceClaimEnv env {&sched, c, a, me, epoch, c->inject == TILEXR_INJECT_OLD_EPOCH_CONSUMER ? epoch - 1 : epoch,
+                        &rowOf, &flags, &contents, &claimCounter, &status, &wrongPerConsumer[static_cast<size_t>(me)]};
+                    ClaimAndReduce(env, tokens);
                     sched.Finish(a);
                 });
             }
@@ -430,7 +576,7 @@ int TileXREpTraceCheck(const TileXREpTraceShape *shape, const TileXREpTraceEvent
     TileXREpTraceFinding *findings, int32_t maxFindings)
 {
     if (shape == nullptr || numEvents < 0 || (events == nullptr && numEvents > 0) || (findings == nullptr && maxFindings > 0) ||
-        shape->tileRows <= 0 || shape->parts <= 0 || shape->parts > 64 || shape->totalRows < 0) {
+        shape->tileRows <= 0 || shape->parts <= 0 || shape->parts > 64 || shape->totalRows < 0 || shape->tokens < 0) {
         return -1;
     }
     std::vector<TileXREpTraceFinding> out;
@@ -466,6 +612,17 @@ int TileXREpTraceCheck(const TileXREpTraceShape *shape, const TileXREpTraceEvent
     std::set<std::tuple<int, int, uint64_t>> staleReported;
     std::map<int, int64_t> counterValue;
     std::set<int> counterReported;
+    // the consumer side's bookkeeping, per round: who claimed which token, which tokens were finished (summed or given a
+    // row of zeros), and the rows an agent has read since its last token event
+    std::map<std::pair<int, int>, int> claimsOf;                        // (round, token) -> claims
+    std::map<std::pair<int, int>, int> finishedOf;                      // (round, token) -> times finished
+    std::map<int, std::vector<int>> readsSince;                         // agent -> ids of ROW_READ events
+    auto finish = [&](const TileXREpTraceEvent &e) {
+        if (++finishedOf[{e.round, e.row}] == 2) {
+            report(TILEXR_FINDING_TOKEN_CLAIMED_TWICE, e);
+        }
+        readsSince[e.agent].clear();
+    };
     for (int i = 0; i < numEvents; ++i) {
         const TileXREpTraceEvent &e = events[i];
         switch (e.kind) {
@@ -545,9 +702,48 @@ int TileXREpTraceCheck(const TileXREpTraceShape *shape, const TileXREpTraceEvent
                 if (sawReady.count(std::make_tuple(e.agent, e.row / shape->tileRows, e.epoch)) == 0) {
                     report(TILEXR_FINDING_READ_WITHOUT_WAIT, e);
                 }
+                readsSince[e.agent].push_back(i);
                 break;
             }
+            case TILEXR_TRACE_TOKEN_CLAIM: {
+                bool overlap = false;
+                for (int64_t t = static_cast<int64_t>(e.word); t < static_cast<int64_t>(e.word) + e.part; ++t) {
+                    if (t < shape->tokens) {
+                        overlap |= ++claimsOf[{e.round, static_cast<int>(t)}] > 1;
+                    }
+                }
+                if (overlap) {
+                    report(TILEXR_FINDING_TOKEN_CLAIMED_TWICE, e);
+                }
+                break;
+            }
+            case TILEXR_TRACE_TOKEN_REDUCED: {
+                // every row that went into the sum: had its tile been published for the epoch when it was read?
+                for (int readId : readsSince[e.agent]) {
+                    const TileXREpTraceEvent &r = events[readId];
+                    const auto it = storesOf.find({r.tile, r.epoch});
+                    if (it == storesOf.end() || it->second.front() > readId) {
+                        report(TILEXR_FINDING_TOKEN_REDUCED_WHILE_PENDING, e);
+                        out.back().tile = r.tile;
+                        break;
+                    }
+                }
+                finish(e);
+                break;
+            }
+            case TILEXR_TRACE_TOKEN_ZEROED:
+                finish(e);
+                break;
+            case TILEXR_TRACE_SLEEP:
+                break;
             case TILEXR_TRACE_ROUND_END:
+                for (int t = 0; t < shape->tokens; ++t) {
+                    if (claimsOf.count({e.round, t}) == 0 || finishedOf.count({e.round, t}) == 0) {
+                        TileXREpTraceEvent at = e;
+                        at.row = t;
+                        report(TILEXR_FINDING_TOKEN_NEVER_CLAIMED, at);
+                    }
+                }
                 for (const auto &cv : counterValue) {
                     if (cv.second != 0 && counterReported.insert(cv.first).second) {
                         TileXREpTraceEvent at = e;

@@ -1,9 +1,11 @@
 /* CPU model of the tile readiness-flag protocol: an abstract event trace and ordering diagnostics over it.
  *
- * Test infrastructure (it is linked into the hooks library, not into libtilexr-ep.so).  The producer side of the
- * model runs the very code the scatter kernels compile (ep_tile_publish.h: PublishLanded, CountLanded), the consumer
- * side the kernels' acceptance test (TileWordReady), each memory operation being one step of a seeded scheduler and one
- * event of the trace.  The diagnostics are a pure function of a trace, so hand-written traces can be checked too.
+ * Test infrastructure (it is linked into the hooks library, not into libtilexr-ep.so).  Both sides of the model run
+ * the very code the kernels compile: the producers ep_tile_publish.h (PublishLanded, CountLanded), the consumers
+ * ep_token_claim.h (ClaimAndReduce: tokens claimed from a shared counter, at most four held, scan, trusted pass,
+ * give-up and status word; JudgeSlot: what a slot does about a tile that is not there) with the kernels' acceptance
+ * test (TileWordReady).  Each memory operation is one step of a seeded scheduler and one event of the trace.  The
+ * diagnostics are a pure function of a trace, so hand-written traces can be checked too.
  *
  * The idea follows the reference's no-NPU checker (tools/checker/src/diagnostics.cpp:323-440: an event log of
  * READ / WRITE / FLAG_STORE / FLAG_WAIT and rules such as READ_BEFORE_WRITE, FLAG_STALE_MAGIC, FLAG_NO_PRODUCER,
@@ -28,7 +30,11 @@ enum {
     TILEXR_TRACE_FLAG_POLL = 5,       /* consumer read `word` from `tile`, wants `epoch`; `accepted` = took it as ready */
     TILEXR_TRACE_WAIT_EXPIRED = 6,    /* consumer gave up waiting for `tile` / `epoch` */
     TILEXR_TRACE_ROW_READ = 7,        /* consumer read row `row` expecting the contents of `epoch` */
-    TILEXR_TRACE_ROUND_END = 8        /* all agents of one dispatch + combine are done */
+    TILEXR_TRACE_ROUND_END = 8,       /* all agents of one dispatch + combine are done */
+    TILEXR_TRACE_TOKEN_CLAIM = 9,     /* consumer took tokens [word, word + part) from the shared claim counter */
+    TILEXR_TRACE_TOKEN_REDUCED = 10,  /* consumer summed token `row` from the rows it has read since its last token event */
+    TILEXR_TRACE_TOKEN_ZEROED = 11,   /* consumer gave token `row` a row of zeros (a wait of its tiles expired) */
+    TILEXR_TRACE_SLEEP = 12           /* consumer found nothing ready and backs off (`part` = level) */
 };
 
 typedef struct {
@@ -58,7 +64,11 @@ enum {
     TILEXR_FINDING_COUNTER_NOT_ZERO = 7,       /* a landing counter did not return to zero by the end of the round */
     TILEXR_FINDING_WRONG_WORD = 8,             /* a stored word's lower half is not the tile's row count */
     TILEXR_FINDING_READ_WITHOUT_WAIT = 9,      /* a row was read by an agent that never saw its tile ready for the epoch */
-    TILEXR_FINDING_WAIT_EXPIRED_EARLY = 10     /* a wait expired although the tile is published later (bound too short) */
+    TILEXR_FINDING_WAIT_EXPIRED_EARLY = 10,    /* a wait expired although the tile is published later (bound too short) */
+    TILEXR_FINDING_TOKEN_REDUCED_WHILE_PENDING = 11, /* a token was summed although a tile of one of its rows had not
+                                                  been published for the epoch yet */
+    TILEXR_FINDING_TOKEN_CLAIMED_TWICE = 12,   /* two claims of a round overlap, or a token was finished twice */
+    TILEXR_FINDING_TOKEN_NEVER_CLAIMED = 13    /* a token of the round was never claimed or never finished */
 };
 
 typedef struct {
@@ -76,6 +86,7 @@ typedef struct {
     int32_t maxRows;      /* rows the counters are sized for (>= totalRows) */
     int32_t tileRows;
     int32_t parts;        /* publishers per row (column slices) */
+    int32_t tokens;       /* tokens a combine reduces per round; 0: unknown, the claim rules are not applied */
 } TileXREpTraceShape;
 
 enum {
@@ -93,18 +104,24 @@ enum {
     TILEXR_INJECT_DOUBLE_REPORT = 4,       /* one part is reported twice */
     TILEXR_INJECT_REPORT_BEFORE_WRITE = 5, /* parts are reported before they are written */
     TILEXR_INJECT_CONSUMER_ENQUEUED_FIRST = 6, /* one shared queue, the waiting kernel ahead of its producer */
-    TILEXR_INJECT_OLD_EPOCH_CONSUMER = 7   /* consumers wait for the previous round's epoch */
+    TILEXR_INJECT_OLD_EPOCH_CONSUMER = 7,  /* consumers wait for the previous round's epoch */
+    TILEXR_INJECT_TRUST_WITHOUT_SCAN = 8,  /* one consumer's scan reports every held token ready without looking */
+    TILEXR_INJECT_CLAIM_NOT_ATOMIC = 9,    /* the claim counter is read and written back in two steps */
+    TILEXR_INJECT_CLAIM_SKIPS = 10,        /* one consumer's claims start one token late */
+    TILEXR_INJECT_IMPATIENT_CONSUMER = 11  /* one consumer gives up after its first scan without a ready token */
 };
 
 typedef struct {
     TileXREpTraceShape shape;
-    int32_t topK;          /* rows a consumer gathers per token: rows are dealt to tokens by a seeded permutation */
+    int32_t topK;          /* rows a consumer gathers per token: rows are dealt to tokens by a seeded permutation
+                              (shape.tokens must be 0 or ceil(totalRows / topK)) */
     int32_t producers;
     int32_t consumers;
     int32_t rounds;        /* dispatch + combine pairs in a row on the same flags and counters */
     int32_t scheduler;
     int32_t inject;
-    int32_t pollBudget;    /* failed polls after which a wait expires (stands for the wall-clock bound) */
+    int32_t pollBudget;    /* scans without a ready token after which what a consumer holds is given up (stands for the
+                              wall-clock bound) */
     uint32_t seed;
 } TileXREpTraceCase;
 
