@@ -16,14 +16,14 @@ import pytest
 import hostlib as H
 
 (LAUNCH, ROW_WRITE, COUNTER_ADD, COUNTER_RESET, FLAG_STORE, FLAG_POLL, WAIT_EXPIRED, ROW_READ, ROUND_END, TOKEN_CLAIM,
- TOKEN_REDUCED, TOKEN_ZEROED, SLEEP) = range(13)
+ TOKEN_REDUCED, TOKEN_ZEROED, SLEEP, CONSUMER_LEAVE, CLAIM_RESET) = range(15)
 (READ_BEFORE_WRITE, FLAG_STALE_EPOCH, FLAG_NO_PRODUCER, DEADLOCK, DOUBLE_PUBLISH, PUBLISH_BEFORE_LANDED,
  COUNTER_NOT_ZERO, WRONG_WORD, READ_WITHOUT_WAIT, WAIT_EXPIRED_EARLY, TOKEN_REDUCED_WHILE_PENDING, TOKEN_CLAIMED_TWICE,
- TOKEN_NEVER_CLAIMED) = range(1, 14)
+ TOKEN_NEVER_CLAIMED, CLAIM_WORD_NOT_RESET) = range(1, 15)
 SERIAL, ROUND_ROBIN, RANDOM, CONSUMER_EAGER = range(4)
 (INJECT_NONE, INJECT_READ_WITHOUT_WAIT, INJECT_ACCEPT_ANY_EPOCH, INJECT_MISSING_PRODUCER, INJECT_DOUBLE_REPORT,
  INJECT_REPORT_BEFORE_WRITE, INJECT_CONSUMER_ENQUEUED_FIRST, INJECT_OLD_EPOCH_CONSUMER, INJECT_TRUST_WITHOUT_SCAN,
- INJECT_CLAIM_NOT_ATOMIC, INJECT_CLAIM_SKIPS, INJECT_IMPATIENT_CONSUMER) = range(12)
+ INJECT_CLAIM_NOT_ATOMIC, INJECT_CLAIM_SKIPS, INJECT_IMPATIENT_CONSUMER, INJECT_NO_CLAIM_RESET) = range(13)
 
 
 class Event(C.Structure):
@@ -195,6 +195,10 @@ def test_consumer_side_rules():
     t = consumer_trace() + [ev(ROUND_END, agent=-1, epoch=E + 1, round_=2)]
     f = check(shape, t)
     assert kinds(f) == [TOKEN_NEVER_CLAIMED] and f[0].round == 2
+    # a launch whose first claim does not find the counter at zero (the launch before did not leave it so)
+    t = consumer_trace()
+    t[4] = ev(TOKEN_CLAIM, 1, 1, part=4, word=1, epoch=E)
+    assert CLAIM_WORD_NOT_RESET in kinds(check(shape, t))
     # without a token count the claim rules are off
     assert check(SHAPE, [e for e in consumer_trace() if e.kind != TOKEN_CLAIM]) == []
     assert lib().TileXREpTraceFindingName(TOKEN_REDUCED_WHILE_PENDING) == b"TOKEN_REDUCED_WHILE_PENDING"
@@ -263,6 +267,12 @@ def test_consumers_claim_hold_scan_and_reduce_as_the_kernels_do(scheduler):
                 elif e.kind == SLEEP:
                     assert polls_since_progress > 0 and held > 0      # it looked, found nothing, and still owes tokens
             assert held == 0
+        leaves = [e for e in ev_r if e.kind == CONSUMER_LEAVE]
+        assert sorted(e.word for e in leaves) == list(range(consumers))           # everybody leaves once
+        resets = [e for e in ev_r if e.kind == CLAIM_RESET]
+        assert sorted(e.counter for e in resets) == [0, 1] and all(e.word == 0 for e in resets)
+        assert all(e.agent == max(leaves, key=lambda x: x.id).agent and e.id > max(x.id for x in leaves) for e in resets)
+        assert not any(e.kind == TOKEN_CLAIM and e.id > min(x.id for x in resets) for e in ev_r)
     if scheduler == CONSUMER_EAGER:
         assert any(e.kind == SLEEP for e in events)       # consumers that run ahead of their producers do back off
 
@@ -312,6 +322,7 @@ def test_trace_covers_the_two_level_counters():
     (INJECT_CLAIM_NOT_ATOMIC, ROUND_ROBIN, {TOKEN_CLAIMED_TWICE}, None),
     (INJECT_CLAIM_SKIPS, RANDOM, {TOKEN_NEVER_CLAIMED}, False),
     (INJECT_IMPATIENT_CONSUMER, CONSUMER_EAGER, {WAIT_EXPIRED_EARLY}, False),
+    (INJECT_NO_CLAIM_RESET, RANDOM, {CLAIM_WORD_NOT_RESET, TOKEN_NEVER_CLAIMED}, False),   # the second launch claims from where the first stopped
 ])
 def test_each_planted_mistake_is_reported(inject, scheduler, expect, wrong_tokens):
     events, findings, wrong = run(100, 128, 8, 2, scheduler=scheduler, inject=inject, budget=60, rounds=2, seed=5)

@@ -331,12 +331,10 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     red.producerOrdered = p.tileFlags != nullptr && p.tileFlags == comm->lastFlagWords &&
         red.flagEpoch == comm->lastFlagEpoch && stream == comm->lastFlagStream;
     if (red.tileFlags != nullptr && !red.producerOrdered) {
-        // a launch that may wait: its workgroups claim their tokens from a shared counter (see ForEachGroup)
+        // a launch that may wait: its workgroups claim their tokens from a shared counter (ep_token_claim.h).  The words
+        // are zeroed when they are allocated and left at zero by every launch: nothing to clear here
         if (!comm->claimWord.Reserve(256, true)) {
             return TileXR::TILEXR_ERROR_INTERNAL;
-        }
-        if (ClearScratchWord(comm->claimWord.ptr, stream) != hipSuccess) {
-            return TileXR::TILEXR_ERROR_MKIRT;
         }
         red.claimWord = static_cast<uint32_t *>(comm->claimWord.ptr);
     }

@@ -189,7 +189,8 @@ struct ReduceLaunch {
     const uint64_t *tileFlags;       // optional: a tile is ready once the upper half of its word equals flagEpoch
     int64_t tileRows;
     uint64_t flagEpoch;
-    uint32_t *claimWord;             // launches that may wait: a zeroed device word the workgroups claim their tokens from
+    uint32_t *claimWord;             // launches that may wait: two device words the workgroups claim their tokens from,
+                                     // zero between launches (the last workgroup to leave puts them back)
     bool producerOrdered;            // the producer of the flags was enqueued earlier on this very stream: every wait
                                      // succeeds at its first poll, so the launch need not leave room for a producer
     int64_t waitTimeoutTicks;        // in wall_clock64 ticks

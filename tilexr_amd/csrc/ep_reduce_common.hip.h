@@ -42,7 +42,8 @@ struct ReduceArgs {
     int64_t waitTimeoutTicks;
     int32_t *deviceStatus;
     int flagsSettled;                // the producer of the flags finished before this launch began (same stream)
-    uint32_t *claim;                 // launches that may wait: zero at launch, the next group nobody has claimed yet
+    uint32_t *claim;                 // launches that may wait: two words, zero at launch and again when the launch is
+                                     // over (the next group nobody has claimed yet; workgroups that have left)
 };
 
 // Launchers of the register-resident kernels, one translation unit per (element type, with / without readiness flags).
@@ -379,6 +380,13 @@ __device__ __forceinline__ void ForEachGroup(const ReduceArgs &a, int groups, in
             {
                 for (int r = 0; r < (1 << level); ++r) {
                     __builtin_amdgcn_s_sleep(127);      // 127 x 64 clocks, about 3.5 us
+                }
+            }
+            __device__ __forceinline__ void Leave()
+            {
+                if (a.claim != nullptr && threadIdx.x == 0) {
+                    DeviceTileOps ops;
+                    LeaveClaimWords(ops, a.claim, gridDim.x);
                 }
             }
         };

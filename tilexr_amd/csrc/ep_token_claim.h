@@ -30,6 +30,10 @@
 //   bool GiveUpNow()                    the wait bound has passed since Touch(), or a wait of the launch has expired
 //   void Touch()                        progress was made: the wait bound starts again
 //   void Sleep(int level)               level 0, 1, 2: longer each time
+//   void Leave()                        this workgroup has claimed for the last time.  The claim counter is left at
+//                                       zero for the next launch by whoever leaves last (a second word counts the
+//                                       leavers), the way the publishers' landing counters are: no launch has to
+//                                       clear anything first
 #ifndef TILEXR_AMD_EP_TOKEN_CLAIM_H
 #define TILEXR_AMD_EP_TOKEN_CLAIM_H
 
@@ -124,6 +128,22 @@ TILEXR_EP_HD void ClaimAndReduce(Env &env, int groups)
             break;
         }
     }
+    env.Leave();
+}
+
+// The leaver's part, for an Env whose two words live in memory the operations `ops` reach (FetchAdd(p) -> value
+// before, Store(p, v)): the last of `workgroups` leavers puts both words back to zero.  Every claim of a workgroup has
+// returned before it leaves, so nothing can claim behind the reset.  Returns whether this call did the reset.
+template <typename Ops>
+TILEXR_EP_HD bool LeaveClaimWords(Ops &ops, uint32_t *claimWords, uint32_t workgroups)
+{
+    const uint32_t before = ops.FetchAdd(&claimWords[1]);
+    if (before + 1u != workgroups) {
+        return false;
+    }
+    ops.Store(&claimWords[1], 0u);
+    ops.Store(&claimWords[0], 0u);
+    return true;
 }
 
 } // namespace TileXREp

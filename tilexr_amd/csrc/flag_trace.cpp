@@ -213,7 +213,7 @@ struct TraceClaimEnv {
     const std::vector<int> *rowOf;          // [tokens, topK] rows of a token, -1 = none
     const std::vector<uint64_t> *flags;
     const std::vector<uint64_t> *contents;  // epoch that last wrote each (row, part)
-    uint32_t *claimCounter;
+    uint32_t *claimCounter;                 // two words, as on the device: next token to claim, consumers that have left
     std::atomic<int> *status;               // the launch's status word
     int *wrongTokens;
     int held[kClaimHeld] = {-1, -1, -1, -1};
@@ -375,6 +375,39 @@ struct TraceClaimEnv {
         return ++idleScans > c->pollBudget || *status != 0;
     }
     void Touch() { idleScans = 0; }
+    void Leave()
+    {
+        // LeaveClaimWords of ep_token_claim.h, its memory operations as steps of the scheduler
+        struct LeaveOps {
+            TraceClaimEnv *env;
+            uint32_t FetchAdd(uint32_t *p)
+            {
+                uint32_t before = 0;
+                env->sched->Step(env->agent, nullptr, [&](TileXREpTraceEvent &e) {
+                    before = (*p)++;
+                    e.kind = TILEXR_TRACE_CONSUMER_LEAVE;
+                    e.word = before;
+                    e.epoch = env->want;
+                });
+                return before;
+            }
+            void Store(uint32_t *p, uint32_t v)
+            {
+                env->sched->Step(env->agent, nullptr, [&](TileXREpTraceEvent &e) {
+                    *p = v;
+                    e.kind = TILEXR_TRACE_CLAIM_RESET;
+                    e.counter = static_cast<int32_t>(p - env->claimCounter);
+                    e.word = v;
+                    e.epoch = env->want;
+                });
+            }
+        } ops {this};
+        if (c->inject == TILEXR_INJECT_NO_CLAIM_RESET) {
+            ops.FetchAdd(&claimCounter[1]);      // counts itself out, and nobody puts the words back
+            return;
+        }
+        TileXREp::LeaveClaimWords(ops, claimCounter, static_cast<uint32_t>(c->consumers));
+    }
     void Sleep(int level)
     {
         bool yield = true;                  // nothing was ready: somebody else gets the turn
@@ -397,6 +430,7 @@ int Priority(int kind)
         case TILEXR_FINDING_TOKEN_REDUCED_WHILE_PENDING: return 4;
         case TILEXR_FINDING_TOKEN_CLAIMED_TWICE: return 4;
         case TILEXR_FINDING_TOKEN_NEVER_CLAIMED: return 4;
+        case TILEXR_FINDING_CLAIM_WORD_NOT_RESET: return 4;
         case TILEXR_FINDING_PUBLISH_BEFORE_LANDED: return 5;
         case TILEXR_FINDING_DOUBLE_PUBLISH: return 6;
         case TILEXR_FINDING_WRONG_WORD: return 7;
@@ -425,6 +459,7 @@ const char *TileXREpTraceFindingName(int32_t kind)
         case TILEXR_FINDING_TOKEN_REDUCED_WHILE_PENDING: return "TOKEN_REDUCED_WHILE_PENDING";
         case TILEXR_FINDING_TOKEN_CLAIMED_TWICE: return "TOKEN_CLAIMED_TWICE";
         case TILEXR_FINDING_TOKEN_NEVER_CLAIMED: return "TOKEN_NEVER_CLAIMED";
+        case TILEXR_FINDING_CLAIM_WORD_NOT_RESET: return "CLAIM_WORD_NOT_RESET";
         default: return "UNKNOWN";
     }
 }
@@ -447,6 +482,8 @@ int TileXREpTraceRun(const TileXREpTraceCase *c, TileXREpTraceEvent *events, int
     std::vector<uint64_t> flags(static_cast<size_t>(maxTiles), 0ull);
     // what memory holds: the epoch that last wrote each (row, part)
     std::vector<uint64_t> contents(static_cast<size_t>(sh.maxRows) * sh.parts, 0ull);
+    uint32_t claimWords[2] = {0u, 0u};      // what the waiting launches claim their tokens from: zero once, then left at
+                                            // zero by every launch's last leaver
     std::vector<TileXREpTraceEvent> log;
     std::mt19937 rng(c->seed);
     int wrong = 0;
@@ -495,7 +532,6 @@ int TileXREpTraceRun(const TileXREpTraceCase *c, TileXREpTraceEvent *events, int
         Scheduler sched(agents, c->scheduler, rng(), &log, round);
         std::vector<int> wrongPerConsumer(static_cast<size_t>(c->consumers), 0);
         std::atomic<int> status {0};    // the launch's status word: set by the first expired wait
-        uint32_t claimCounter = 0;      // the device word a waiting launch's workgroups claim their tokens from: cleared per launch
         std::vector<std::thread> pool;
         for (int a = 0; a < agentsN; ++a) {
             if (a < c->producers) {
@@ -541,7 +577,7 @@ int TileXREpTraceRun(const TileXREpTraceCase *c, TileXREpTraceEvent *events, int
                 pool.emplace_back([&, a] {
                     const int me = a - c->producers;
                     TraceClaimEnv env {&sched, c, a, me, epoch, c->inject == TILEXR_INJECT_OLD_EPOCH_CONSUMER ? epoch - 1 : epoch,
-                        &rowOf, &flags, &contents, &claimCounter, &status, &wrongPerConsumer[static_cast<size_t>(me)]};
+                        &rowOf, &flags, &contents, claimWords, &status, &wrongPerConsumer[static_cast<size_t>(me)]};
                     ClaimAndReduce(env, tokens);
                     sched.Finish(a);
                 });
@@ -617,6 +653,7 @@ int TileXREpTraceCheck(const TileXREpTraceShape *shape, const TileXREpTraceEvent
     std::map<std::pair<int, int>, int> claimsOf;                        // (round, token) -> claims
     std::map<std::pair<int, int>, int> finishedOf;                      // (round, token) -> times finished
     std::map<int, std::vector<int>> readsSince;                         // agent -> ids of ROW_READ events
+    std::set<int> roundsWithClaims;
     auto finish = [&](const TileXREpTraceEvent &e) {
         if (++finishedOf[{e.round, e.row}] == 2) {
             report(TILEXR_FINDING_TOKEN_CLAIMED_TWICE, e);
@@ -705,7 +742,14 @@ int TileXREpTraceCheck(const TileXREpTraceShape *shape, const TileXREpTraceEvent
                 readsSince[e.agent].push_back(i);
                 break;
             }
+            case TILEXR_TRACE_CONSUMER_LEAVE:
+            case TILEXR_TRACE_CLAIM_RESET:
+                break;
             case TILEXR_TRACE_TOKEN_CLAIM: {
+                // the first claim of a launch finds the counter at zero: the launch before has left it so
+                if (shape->tokens > 0 && roundsWithClaims.insert(e.round).second && e.word != 0) {
+                    report(TILEXR_FINDING_CLAIM_WORD_NOT_RESET, e);
+                }
                 bool overlap = false;
                 for (int64_t t = static_cast<int64_t>(e.word); t < static_cast<int64_t>(e.word) + e.part; ++t) {
                     if (t < shape->tokens) {

@@ -34,7 +34,9 @@ enum {
     TILEXR_TRACE_TOKEN_CLAIM = 9,     /* consumer took tokens [word, word + part) from the shared claim counter */
     TILEXR_TRACE_TOKEN_REDUCED = 10,  /* consumer summed token `row` from the rows it has read since its last token event */
     TILEXR_TRACE_TOKEN_ZEROED = 11,   /* consumer gave token `row` a row of zeros (a wait of its tiles expired) */
-    TILEXR_TRACE_SLEEP = 12           /* consumer found nothing ready and backs off (`part` = level) */
+    TILEXR_TRACE_SLEEP = 12,          /* consumer found nothing ready and backs off (`part` = level) */
+    TILEXR_TRACE_CONSUMER_LEAVE = 13, /* consumer has claimed for the last time: +1 on the leavers' word, `word` = value before */
+    TILEXR_TRACE_CLAIM_RESET = 14     /* the last leaver stored `word` (0) to claim word `counter` (1: leavers, 0: next token) */
 };
 
 typedef struct {
@@ -68,7 +70,8 @@ enum {
     TILEXR_FINDING_TOKEN_REDUCED_WHILE_PENDING = 11, /* a token was summed although a tile of one of its rows had not
                                                   been published for the epoch yet */
     TILEXR_FINDING_TOKEN_CLAIMED_TWICE = 12,   /* two claims of a round overlap, or a token was finished twice */
-    TILEXR_FINDING_TOKEN_NEVER_CLAIMED = 13    /* a token of the round was never claimed or never finished */
+    TILEXR_FINDING_TOKEN_NEVER_CLAIMED = 13,   /* a token of the round was never claimed or never finished */
+    TILEXR_FINDING_CLAIM_WORD_NOT_RESET = 14   /* a round's first claim did not find the claim counter at zero */
 };
 
 typedef struct {
@@ -108,7 +111,8 @@ enum {
     TILEXR_INJECT_TRUST_WITHOUT_SCAN = 8,  /* one consumer's scan reports every held token ready without looking */
     TILEXR_INJECT_CLAIM_NOT_ATOMIC = 9,    /* the claim counter is read and written back in two steps */
     TILEXR_INJECT_CLAIM_SKIPS = 10,        /* one consumer's claims start one token late */
-    TILEXR_INJECT_IMPATIENT_CONSUMER = 11  /* one consumer gives up after its first scan without a ready token */
+    TILEXR_INJECT_IMPATIENT_CONSUMER = 11, /* one consumer gives up after its first scan without a ready token */
+    TILEXR_INJECT_NO_CLAIM_RESET = 12      /* nobody puts the claim words back to zero when the launch is over */
 };
 
 typedef struct {
