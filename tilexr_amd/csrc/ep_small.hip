@@ -8,6 +8,8 @@
 // 1159-1168, 1240-1258); only the number of launches differs.  With readiness flags the rows are written through to memory
 // and reported landed as in the scatter kernels (ep_tile_publish.h); the rows the whole dispatch keeps, which the size of
 // the last tile depends on, every workgroup has counted anyway or counts with four more ballots.
+#include <type_traits>
+
 #include <hip/hip_runtime.h>
 
 #include "ep_block_scan.hip.h"
@@ -171,31 +173,25 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_kernel(SmallArgs a
     }
 }
 
-// Block-wide count of the lanes' set predicates over the kIdsPerLane id slots: ballots per wave, one LDS add per wave.
-__device__ __forceinline__ void AddBallots(const bool (&pred)[kIdsPerLane], int *sum, int lane)
-{
-    int n = 0;
-#pragma unroll
-    for (int j = 0; j < kIdsPerLane; ++j) {
-        n += __popcll(__ballot(pred[j]));
-    }
-    if (lane == 0 && n != 0) {
-        atomicAdd(sum, n);
-    }
-}
-
 // Without a capacity limit a route's row needs no histogram at all:
 //   row = (valid routes with a smaller expert id) + (earlier routes with the same expert id)
 // so one workgroup per route counts those two sets over the id table and writes its one row.  Workgroup b < E also
 // counts expert b's routes for the count outputs.  Eight times as many workgroups as tokens spread a decode batch
 // over the whole chip.
-template <int V, bool WT>
+//
+// The launch is two round trips to memory (id table and token row out, the row's stores back) with the counting in
+// between, and at this size the counting is paid in instructions: a wave that runs alone on its SIMD issues a dependent
+// instruction every 4 ns or so.  So every lane counts its own ids with compares and adds (no ballot and scalar count
+// per id), the four sets share two registers (16 bits each: at most 2048 ids), one pair of reductions per wave and one
+// LDS exchange between the four waves finish it.  IDS = ids per lane (4: up to 1024 routes, 8: up to 2048).
+template <int V, bool WT, int IDS>
 __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(SmallArgs a)
 {
-    __shared__ int s_sum[5];     // smaller ids, earlier equal ids, ids equal to blockIdx, ids not above blockIdx, valid ids
+    __shared__ int s_sum[kWavesPerBlock][3];     // per wave: smaller | earlier equal << 16, equal to blockIdx | not above << 16, valid
 
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
+    const int wave = tid / kWave;
     const int route = blockIdx.x;
     const int token = route / a.topK;
     const int n = a.bs * a.topK;
@@ -208,46 +204,44 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
         const int idx = j * kThreads + tid;
         v[j] = idx < vecs ? src[idx] : u32x4{0u, 0u, 0u, 0u};
     }
-    int e[kIdsPerLane];
+    int e[IDS];
 #pragma unroll
-    for (int j = 0; j < kIdsPerLane; ++j) {
+    for (int j = 0; j < IDS; ++j) {
         const int i = j * kThreads + tid;
-        const int id = i < n ? a.ids[i] : -1;
-        e[j] = (id >= 0 && id < a.numExperts) ? id : -1;
+        e[j] = i < n ? a.ids[i] : -1;
     }
     const int mine = a.ids[route];
-    const int key = (mine >= 0 && mine < a.numExperts) ? mine : -1;
-    if (tid < 5) {
-        s_sum[tid] = 0;
-    }
-    __syncthreads();
+    const unsigned experts = static_cast<unsigned>(a.numExperts);
+    const int key = static_cast<unsigned>(mine) < experts ? mine : -1;       // ids outside [0, E) are skipped, not errors
     const int expert = blockIdx.x;       // the expert this workgroup counts for the outputs (if there is one)
-    bool less[kIdsPerLane], before[kIdsPerLane], same[kIdsPerLane], upTo[kIdsPerLane];
+    int rowCounts = 0;      // valid ids below the key | earlier ids equal to it << 16
+    int outCounts = 0;      // ids equal to `expert` | valid ids not above it << 16
+    int valid = 0;
 #pragma unroll
-    for (int j = 0; j < kIdsPerLane; ++j) {
+    for (int j = 0; j < IDS; ++j) {
         const int i = j * kThreads + tid;
-        less[j] = e[j] >= 0 && e[j] < key;
-        before[j] = e[j] >= 0 && e[j] == key && i < route;
-        same[j] = e[j] == expert;
-        upTo[j] = e[j] >= 0 && e[j] <= expert;
+        const unsigned id = static_cast<unsigned>(e[j]);
+        const bool ok = id < experts;
+        rowCounts += (ok && e[j] < key ? 1 : 0) + (e[j] == key && i < route ? 0x10000 : 0);
+        outCounts += (e[j] == expert ? 1 : 0) + (ok && e[j] <= expert ? 0x10000 : 0);
+        valid += ok ? 1 : 0;
     }
-    AddBallots(less, &s_sum[0], lane);
-    AddBallots(before, &s_sum[1], lane);
-    if (WT) {
-        // rows the whole dispatch keeps: the size of the last tile
-        bool valid[kIdsPerLane];
 #pragma unroll
-        for (int j = 0; j < kIdsPerLane; ++j) {
-            valid[j] = e[j] >= 0;
+    for (int off = kWave / 2; off >= 1; off >>= 1) {
+        rowCounts += __shfl_xor(rowCounts, off);
+        outCounts += __shfl_xor(outCounts, off);
+        if (WT) {
+            valid += __shfl_xor(valid, off);
         }
-        AddBallots(valid, &s_sum[4], lane);
     }
-    if (expert < a.numExperts) {
-        AddBallots(same, &s_sum[2], lane);
-        AddBallots(upTo, &s_sum[3], lane);
+    if (lane == 0) {
+        s_sum[wave][0] = rowCounts;
+        s_sum[wave][1] = outCounts;
+        s_sum[wave][2] = valid;
     }
     __syncthreads();
-    const int row = key >= 0 ? s_sum[0] + s_sum[1] : -1;
+    const int rowSum = s_sum[0][0] + s_sum[1][0] + s_sum[2][0] + s_sum[3][0];
+    const int row = key >= 0 ? (rowSum & 0xffff) + (rowSum >> 16) : -1;
     if (tid == 0) {
         if (row >= 0) {
             int32_t *tuple = a.assist + static_cast<int64_t>(row) * 4;
@@ -260,9 +254,10 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
             a.rowOf[route] = row;
         }
         if (expert < a.numExperts) {
-            a.sendCountsOut[expert] = s_sum[3];
+            const int outSum = s_sum[0][1] + s_sum[1][1] + s_sum[2][1] + s_sum[3][1];
+            a.sendCountsOut[expert] = outSum >> 16;
             if (a.expertTokenNumsOut != nullptr) {
-                a.expertTokenNumsOut[expert] = a.tokenNumsType == 0 ? s_sum[3] : s_sum[2];
+                a.expertTokenNumsOut[expert] = a.tokenNumsType == 0 ? outSum >> 16 : outSum & 0xffff;
             }
         }
     }
@@ -283,7 +278,7 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
         __syncthreads();        // uniform: a workgroup without a row has left as a whole
         if (tid == 0) {
             TilePublishArgs t = a.tiles;
-            t.totalRows = s_sum[4];
+            t.totalRows = s_sum[0][2] + s_sum[1][2] + s_sum[2][2] + s_sum[3][2];      // rows the whole dispatch keeps: the size of the last tile
             DeviceTileOps ops;
             PublishLanded(ops, t, row, 1);
         }
@@ -330,12 +325,21 @@ hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l)
     if (l.capacity <= 0 && l.bs * l.topK >= l.numExperts) {
         // one workgroup per route (there are enough of them to cover the experts' count outputs)
         const dim3 routes(static_cast<unsigned>(l.bs * l.topK));
+        const bool few = l.bs * l.topK <= 4 * kThreads;
+        auto pick = [&](auto vecsPerLane) {
+            constexpr int kV = decltype(vecsPerLane)::value;
+            if (few) {
+                flags ? launch(ep_dispatch_small_route_kernel<kV, true, 4>, routes) : launch(ep_dispatch_small_route_kernel<kV, false, 4>, routes);
+            } else {
+                flags ? launch(ep_dispatch_small_route_kernel<kV, true, kIdsPerLane>, routes) : launch(ep_dispatch_small_route_kernel<kV, false, kIdsPerLane>, routes);
+            }
+        };
         if (v == 2) {
-            flags ? launch(ep_dispatch_small_route_kernel<2, true>, routes) : launch(ep_dispatch_small_route_kernel<2, false>, routes);
+            pick(std::integral_constant<int, 2>{});
         } else if (v == 4) {
-            flags ? launch(ep_dispatch_small_route_kernel<4, true>, routes) : launch(ep_dispatch_small_route_kernel<4, false>, routes);
+            pick(std::integral_constant<int, 4>{});
         } else {
-            flags ? launch(ep_dispatch_small_route_kernel<8, true>, routes) : launch(ep_dispatch_small_route_kernel<8, false>, routes);
+            pick(std::integral_constant<int, 8>{});
         }
         return hipGetLastError();
     }
