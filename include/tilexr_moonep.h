@@ -98,7 +98,21 @@ typedef enum TileXRMoonEpStage {
 
 /* Values the stages leave in plan->status[0] (device memory) once the stream has run.
  * reference: src/moonep/common/moonep_peer_window.h:36-43; the combine kernel stores its first failure, which is 0
- * on success (src/moonep/combine/kernels/tilexr_moonep_combine_kernel.cpp:727-733). */
+ * on success (src/moonep/combine/kernels/tilexr_moonep_combine_kernel.cpp:727-733).
+ *
+ * Which value a rank gets when plans are invalid is a closed-form function of F, the set of ranks whose OWN plan is
+ * invalid in this exchange (R = ranks of the world):
+ *   dispatch  rank r in F:      TILEXR_MOONEP_DISPATCH_STATUS_INVALID_ROUTE
+ *             rank r not in F:  TILEXR_MOONEP_DISPATCH_STATUS_REMOTE_FAILURE_BASE + p, p the first member of F in the
+ *                               order r+1, r+2, ..., R-1, 0, ..., r-1; SUCCESS when F is empty
+ *   combine   rank r in F:      TILEXR_MOONEP_COMBINE_STATUS_INVALID_ROUTE
+ *             rank r not in F:  TILEXR_MOONEP_COMBINE_STATUS_REMOTE_FAILURE_BASE + min(F); SUCCESS when F is empty
+ * What the output tensors of such an exchange hold is unspecified.  The orders are those in which the reference's kernels wait
+ * for their peers (dispatch: WaitAllPeers, tilexr_moonep_dispatch_kernel.cpp:506-521, peer = (rank + offset) % R;
+ * combine: CrossRankBarrier, tilexr_moonep_combine_kernel.cpp:391-411, rank order).  There a rank that failed because
+ * of a peer raises the same failed flag as the peer itself, so a third rank that meets that flag first names the
+ * messenger instead of the origin, depending on timing; here only members of F are ever named, which is the outcome
+ * of the reference's walk when no messenger's flag is seen before the origin's. */
 #define TILEXR_MOONEP_DISPATCH_STATUS_SUCCESS 2000
 #define TILEXR_MOONEP_DISPATCH_STATUS_INVALID_ROUTE 2001
 #define TILEXR_MOONEP_DISPATCH_STATUS_REMOTE_FAILURE_BASE 2100   /* + rank of the peer whose plan was invalid */

@@ -42,6 +42,25 @@ def random_dst(sh: M.Shape, rng, duplicates=True):
     return dst.astype(np.int32)
 
 
+def status_with_invalid_plans(world, invalid, stage):
+    """Device status of every rank when the ranks in `invalid` hold an invalid plan, written out from the rule in
+    include/tilexr_moonep.h without the oracle: an invalid rank reports its own code; a valid one names the first invalid
+    rank after itself going upwards with wrap-around (dispatch), or the lowest invalid rank (combine)."""
+    own, base, ok = {"dispatch": (2001, 2100, 2000), "combine": (3001, 3100, 0)}[stage]
+    invalid = sorted(set(invalid))
+    out = []
+    for r in range(world):
+        if not invalid:
+            out.append(ok)
+        elif r in invalid:
+            out.append(own)
+        elif stage == "dispatch":
+            out.append(base + min(invalid, key=lambda p: (p - r) % world))
+        else:
+            out.append(base + invalid[0])
+    return out
+
+
 def groups_as_sets(plan: M.DupPlan, rank):
     out = {}
     for g in range(int(plan.counts[rank, 0])):

@@ -293,6 +293,55 @@ def test_saved_plan_is_followed_as_given(row_cache):
         check_dispatch(sh, res, plans, M.dispatch_world(sh, dst, hidden, flags=0, dup=shuffled), fresh=False)
 
 
+def test_combine_with_groups_longer_than_a_wave():
+    """A saved plan may list any number of duplicates under one primary: groups of 66 and 70 rows (the reduce kernel deals
+    a token's rows to the 64 lanes of a wave, so these span two rounds) next to a short one.  Checked against the
+    oracle on random rows and, on rows of small integers whose sums are exact in bf16 whatever the order, against the
+    sum written out: the primary's slot returns the whole group, the duplicates' slots nothing."""
+    world, s, k, h = 2, 50, 2, 136
+    rng = np.random.default_rng(66)
+    sh = M.Shape(world, s, k, h, s * k)
+    dst = MC.random_dst(sh, rng, duplicates=False)
+    dl = M.build_dst_local(sh, dst)
+    dup = M.DupPlan.empty(sh)
+    members = {}
+    for q, sizes in ((0, (66,)), (1, (70, 3))):
+        used = rng.permutation(np.flatnonzero(dl[q] >= 0))
+        at = fill = 0
+        for g, size in enumerate(sizes):
+            rows = used[at:at + size + 1]
+            at += size + 1
+            dup.groups[q, g] = [rows[0], fill, size]
+            dup.loffs[q, fill:fill + size] = rows[1:]
+            fill += size
+            members[(q, int(rows[0]))] = [int(r) for r in rows]
+        dup.counts[q] = [len(sizes), fill]
+    ints = rng.integers(-3, 4, (world, sh.nvs, h)).astype(np.float32)
+    int_rows = (ints.view(np.uint32) >> 16).astype(np.uint16)
+    with World(world) as w:
+        for rows in (random_rows(rng, (world, sh.nvs, h)), int_rows):
+            plans = w.plan_tensors(sh, dst, dup=dup)
+            res = w.combine(sh, plans, dl, [dev_bits16(rows[r]) for r in range(world)])
+            w.sync()
+            want, _, status = M.combine_world(sh, dl, dup, rows)
+            assert status.tolist() == [0, 0] == [int(p["status"][0].item()) for p in plans]
+            for r in range(world):
+                np.testing.assert_array_equal(host_bits16(res[r]["y"]), want[r], err_msg=f"rank {r}")
+        # the integer rows once more, summed by hand
+        total = np.zeros((world, s * k, h), np.float32)
+        in_group = {(q, r) for (q, _), rows in members.items() for r in rows[1:]}
+        for q in range(world):
+            for row in np.flatnonzero(dl[q] >= 0):
+                if (q, int(row)) in in_group:
+                    continue
+                origin, slot = divmod(int(dl[q, row]), sh.nvs)
+                total[origin, slot] = sum(ints[q, r] for r in members.get((q, int(row)), [int(row)]))
+        by_hand = total.reshape(world, s, k, h).sum(axis=2)
+        for r in range(world):
+            got = (host_bits16(res[r]["y"]).astype(np.uint32) << 16).view(np.float32)
+            np.testing.assert_array_equal(got, by_hand[r])
+
+
 def test_device_status_of_bad_plans(row_cache):
     world, s, k, h = 3, 8, 2, 64
     rng = np.random.default_rng(9)
@@ -332,6 +381,40 @@ def test_device_status_of_bad_plans(row_cache):
         w.sync()
         assert [int(p["status"][0].item()) for p in plans] == [3101, 3001, 3101]
         # the world is still usable afterwards
+        plans = w.plan_tensors(sh, dst)
+        res = w.dispatch(sh, plans, hidden, flags=mp.FLAG_BUILD_DEDUP)
+        w.sync()
+        check_dispatch(sh, res, plans, M.dispatch_world(sh, dst, hidden, flags=M.FLAG_BUILD_DEDUP), fresh=True)
+
+
+@pytest.mark.parametrize("world,invalid", [(5, (1, 3)), (6, (0, 2, 5)), (4, (3,))])
+def test_device_status_with_several_invalid_plans(world, invalid):
+    """Several invalid plans in one exchange: every rank's status is the closed form stated in include/tilexr_moonep.h
+    (dispatch names the first invalid rank upwards from one's own, combine the lowest), and the world works afterwards."""
+    s, k, h = 8, 2, 64
+    rng = np.random.default_rng(31 + world)
+    sh = M.Shape(world, s, k, h, s * k)
+    dst = MC.random_dst(sh, rng, duplicates=False)
+    hidden = random_rows(rng, (world, s, h))
+    with World(world) as w:
+        bad = dst.copy()
+        for r in invalid:
+            bad[r, int(rng.integers(sh.n))] = world * sh.nvs
+        plans = w.plan_tensors(sh, bad)
+        w.dispatch(sh, plans, hidden, flags=mp.FLAG_BUILD_DEDUP)
+        w.sync()
+        got = [int(p["status"][0].item()) for p in plans]
+        assert got == MC.status_with_invalid_plans(world, invalid, "dispatch")
+        assert got == M.dispatch_world(sh, bad, hidden, flags=M.FLAG_BUILD_DEDUP)[2].tolist()
+        rows = [dev_bits16(random_rows(rng, (sh.nvs, h))) for r in range(world)]
+        dl = M.build_dst_local(sh, dst)
+        bad_dl = dl.copy()
+        for r in invalid:
+            bad_dl[r, int(rng.choice(np.flatnonzero(dl[r] >= 0)))] = world * sh.nvs
+        plans = w.plan_tensors(sh, dst, dup=M.DupPlan.empty(sh))
+        w.combine(sh, plans, bad_dl, rows)
+        w.sync()
+        assert [int(p["status"][0].item()) for p in plans] == MC.status_with_invalid_plans(world, invalid, "combine")
         plans = w.plan_tensors(sh, dst)
         res = w.dispatch(sh, plans, hidden, flags=mp.FLAG_BUILD_DEDUP)
         w.sync()

@@ -215,6 +215,37 @@ def test_invalid_routes_are_reported_per_rank():
     assert status[1] == M.COMBINE_INVALID_ROUTE and status[0] == M.COMBINE_REMOTE_FAILURE_BASE + 1
 
 
+@pytest.mark.parametrize("world,invalid", [(5, (1, 3)), (5, (0, 4)), (4, (2,)), (6, (1, 2, 5)), (3, (0, 1, 2)), (4, ())])
+def test_status_with_several_invalid_plans_follows_the_stated_rule(world, invalid):
+    """Several ranks with an invalid plan at once: who is named follows the closed form of include/tilexr_moonep.h
+    (dispatch: the first invalid rank upwards from one's own with wrap-around; combine: the lowest invalid rank), worked
+    out in moonep_cases.status_with_invalid_plans without the oracle."""
+    sh = M.Shape(world, 4, 2, 2, 8)
+    rng = np.random.default_rng(world * 10 + len(invalid))
+    dst = MC.random_dst(sh, rng, duplicates=False)
+    hidden = np.ones((world, 4, 2), np.uint16)
+    bad = dst.copy()
+    for r in invalid:
+        bad[r, int(rng.integers(sh.n))] = world * sh.nvs     # a rank that does not exist
+    status = M.dispatch_world(sh, bad, hidden, flags=M.FLAG_BUILD_DEDUP)[2]
+    assert status.tolist() == MC.status_with_invalid_plans(world, invalid, "dispatch")
+    dl = M.build_dst_local(sh, dst)
+    bad_dl = dl.copy()
+    for r in invalid:
+        used = np.flatnonzero(dl[r] >= 0)
+        bad_dl[r, int(rng.choice(used))] = world * sh.nvs
+    status = M.combine_world(sh, bad_dl, M.DupPlan.empty(sh), np.ones((world, sh.nvs, 2), np.uint16))[2]
+    assert status.tolist() == MC.status_with_invalid_plans(world, invalid, "combine")
+
+
+def test_the_stated_rule_on_hand_worked_cases():
+    """The helper itself against cases worked by hand."""
+    assert MC.status_with_invalid_plans(5, (1, 3), "dispatch") == [2101, 2001, 2103, 2001, 2101]
+    assert MC.status_with_invalid_plans(5, (1, 3), "combine") == [3101, 3001, 3101, 3001, 3101]
+    assert MC.status_with_invalid_plans(4, (0,), "dispatch") == [2001, 2100, 2100, 2100]
+    assert MC.status_with_invalid_plans(3, (), "dispatch") == [2000] * 3 and MC.status_with_invalid_plans(3, (), "combine") == [0] * 3
+
+
 # ---- the plan generator used by the GPU tests and the benchmark -----------------------------------------------------
 @pytest.mark.parametrize("world,s,k,experts,padding", [(1, 8, 4, 8, 1), (2, 16, 2, 8, 4), (4, 12, 4, 16, 1), (8, 6, 8, 32, 8)])
 def test_home_plan_is_a_consistent_plan(world, s, k, experts, padding):

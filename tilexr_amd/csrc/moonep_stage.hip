@@ -166,9 +166,9 @@ __device__ __forceinline__ bool SourceWrites(const Route &r, uint8_t direct, uin
 // one reading workgroup in K has to fetch a row from HBM between the writes of the others it runs at little more than
 // half its speed.  After this read it finds the rows in that cache whatever their history.
 constexpr int kWarmLoads = 2;
-__device__ __forceinline__ void WarmRows(const DispatchWorld &a, int64_t block, int64_t vecs)
+__device__ __forceinline__ void WarmRows(const DispatchWorld &a, int rank, int64_t block, int64_t vecs)
 {
-    const u32x4 *rows = static_cast<const u32x4 *>(a.hiddenSh[blockIdx.y]);
+    const u32x4 *rows = static_cast<const u32x4 *>(a.hiddenSh[rank]);
     const int64_t base = block * (kThreads * kWarmLoads) + threadIdx.x;
     u32x4 v[kWarmLoads];
 #pragma unroll
@@ -190,7 +190,7 @@ __device__ __forceinline__ void WarmRows(const DispatchWorld &a, int64_t block, 
 __global__ __launch_bounds__(kThreads) void moon_agree_kernel(DispatchWorld a, unsigned routeBlocks, int64_t warmVecs)
 {
     if (blockIdx.x >= routeBlocks) {
-        WarmRows(a, static_cast<int64_t>(blockIdx.x - routeBlocks), warmVecs);
+        WarmRows(a, blockIdx.y, static_cast<int64_t>(blockIdx.x - routeBlocks), warmVecs);
         return;
     }
     const int src = blockIdx.y;
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(kThreads) void moon_agree_kernel(DispatchWorld a, u
 // The same read as a launch of its own, for a Dispatch that builds its plan: nothing runs ahead of its scatter.
 __global__ __launch_bounds__(kThreads) void moon_warm_rows_kernel(DispatchWorld a, int64_t vecs)
 {
-    WarmRows(a, static_cast<int64_t>(blockIdx.x), vecs);
+    WarmRows(a, blockIdx.y, static_cast<int64_t>(blockIdx.x), vecs);
 }
 
 // One workgroup per (token, route, slice of 512 vectors) of source rank blockIdx.y.
@@ -817,27 +817,16 @@ __device__ __forceinline__ void WriteCombineStatus(const CombineWorld &a, int ra
     a.status[rank][0] = value;
 }
 
-__device__ __forceinline__ void AddRow(float (&acc)[kRowVecs][8], const u32x4 (&v)[kRowVecs])
-{
-#pragma unroll
-    for (int j = 0; j < kRowVecs; ++j) {
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            acc[j][2 * q] = __fadd_rn(acc[j][2 * q], __uint_as_float(v[j][q] << 16));
-            acc[j][2 * q + 1] = __fadd_rn(acc[j][2 * q + 1], __uint_as_float(v[j][q] & 0xffff0000u));
-        }
-    }
-}
-
-__device__ __forceinline__ void LoadRowSlice(const void *tensor, int64_t row, int h, int colBase, int lane, int lanes,
+// The lane's kRowVecs vectors of a row slice.  Lanes beyond the row's end read its last vector (and store nothing
+// later): every lane issues every load, unconditionally.
+__device__ __forceinline__ void LoadRowSlice(const void *tensor, int64_t row, int h, int vecs, int colBase, int lane, int lanes,
     u32x4 (&v)[kRowVecs])
 {
     const u32x4 *p = reinterpret_cast<const u32x4 *>(static_cast<const char *>(tensor) + row * h * 2);
-    const int vecs = h / 8;
 #pragma unroll
     for (int j = 0; j < kRowVecs; ++j) {
         const int idx = colBase + j * lanes + lane;
-        v[j] = idx < vecs ? __builtin_nontemporal_load(p + idx) : u32x4{0u, 0u, 0u, 0u};
+        v[j] = __builtin_nontemporal_load(p + (idx < vecs ? idx : vecs - 1));
     }
 }
 
@@ -877,13 +866,52 @@ __device__ __forceinline__ void LoadSlots(const CombineWorld &a, int rank, int t
     s->count[lane] = grouped ? groupCount : 0;
 }
 
+// What a lane of the reduce kernel knows about one of the rows its token slice sums: bits.  A row without duplicates is
+// a group of one (rounding a bf16 value to bf16 changes nothing).
+constexpr int kItemOpens = 1;       // the group's sum starts as this row (otherwise the row is added to it)
+constexpr int kItemCloses = 2;      // after this row the group's sum is rounded to bf16 and joins the token's sum
+constexpr int kItemValid = 4;       // clear: no item (the tail of a batch of loads)
+
+// sub = row (opens: a uniform condition) or sub + row.  -0.0 + x is x for every x, zeros of either sign included.
+__device__ __forceinline__ void StartOrAddRow(float (&sub)[kRowVecs][8], const u32x4 (&v)[kRowVecs], bool opens)
+{
+#pragma unroll
+    for (int j = 0; j < kRowVecs; ++j) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            sub[j][2 * e] = __fadd_rn(opens ? -0.0f : sub[j][2 * e], __uint_as_float(v[j][e] << 16));
+            sub[j][2 * e + 1] = __fadd_rn(opens ? -0.0f : sub[j][2 * e + 1], __uint_as_float(v[j][e] & 0xffff0000u));
+        }
+    }
+}
+
+__device__ __forceinline__ void AddRounded(float (&acc)[kRowVecs][8], const float (&sub)[kRowVecs][8])
+{
+#pragma unroll
+    for (int j = 0; j < kRowVecs; ++j) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint32_t packed = TileXREp::FloatPairToBf16Rne(sub[j][2 * e], sub[j][2 * e + 1]);
+            acc[j][2 * e] = __fadd_rn(acc[j][2 * e], __uint_as_float(packed << 16));
+            acc[j][2 * e + 1] = __fadd_rn(acc[j][2 * e + 1], __uint_as_float(packed & 0xffff0000u));
+        }
+    }
+}
+
 // Slot sum of one token slice of origin rank blockIdx.y.  Slots are taken in slot order from zero (combine kernel
 // :664-699); a slot that holds a primary with duplicates contributes bf16(fp32(primary) + fp32(dup) + ...) in the plan's
 // list order (combine kernel :489-530); slots that contribute nothing leave the sum as it is (their receive row stays
 // zero in the reference).
+//
+// One wave per slice.  Every row the slice reads -- primaries and the duplicates of their groups, in the order in which
+// they are summed -- becomes an item of one lane (which tensor, which row, what to do with it), so that all look-ups
+// (slot tables, then the duplicates' row numbers) are two round trips for the whole token whatever its groups look like,
+// and the rows themselves are read four at a time.  Items are dealt to the lanes 64 at a time.
 template <int G>
 __global__ __launch_bounds__(G) void moon_reduce_kernel(CombineWorld a, int colSlices)
 {
+    static_assert(G == kWave, "the items of a token are spread over the lanes of one wave");
+    constexpr int kRowsInFlight = 4;
     __shared__ TokenSlots s_slots;
     const int rank = blockIdx.y;
     const int unit = blockIdx.x;
@@ -907,54 +935,90 @@ __global__ __launch_bounds__(G) void moon_reduce_kernel(CombineWorld a, int colS
     }
     const int K = static_cast<int>(a.k);
     const uint32_t nvS = static_cast<uint32_t>(a.nvS);
-    for (int k = 0; k < K; ++k) {
-        // the lanes of the workgroup share one token: everything read from s_slots is uniform
-        const uint32_t where = __builtin_amdgcn_readfirstlane(s_slots.where[k]);
-        if (where == kNoRow) {
-            continue;
-        }
-        const int q = static_cast<int>(where / nvS);
-        const int64_t row = where % nvS;
-        const int count = __builtin_amdgcn_readfirstlane(s_slots.count[k]);
-        u32x4 v[kRowVecs];
-        LoadRowSlice(a.hiddenNvsh[q], row, h, colBase, lane, G, v);
-        if (count == 0) {
-            AddRow(acc, v);
-            continue;
-        }
-        const int start = __builtin_amdgcn_readfirstlane(s_slots.start[k]);
-        float sub[kRowVecs][8];
+    // lane k < K: slot k, the tensor and row of its primary, and how many items it makes
+    uint32_t where = kNoRow;
+    int slotStart = 0;
+    int slotCount = 0;
+    if (lane < K) {
+        where = s_slots.where[lane];
+        slotStart = s_slots.start[lane];
+        slotCount = s_slots.count[lane];
+    }
+    const bool travels = where != kNoRow;
+    const int slotQ = travels ? static_cast<int>(where / nvS) : 0;
+    const int slotRow = travels ? static_cast<int>(where % nvS) : 0;
+    const int slotItems = travels ? 1 + slotCount : 0;
+    int slotFirst = slotItems;                       // inclusive prefix over the K <= 32 slot lanes, then exclusive
 #pragma unroll
-        for (int j = 0; j < kRowVecs; ++j) {
+    for (int off = 1; off < kMaxTopK; off <<= 1) {
+        const int below = __shfl_up(slotFirst, off);
+        slotFirst += lane >= off ? below : 0;
+    }
+    const int total = __builtin_amdgcn_readlane(slotFirst, kMaxTopK - 1);      // lanes from K on add nothing
+    slotFirst -= slotItems;
+    float sub[kRowVecs][8];                          // sum of the group that is open (groups may span windows)
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                sub[j][2 * e] = __uint_as_float(v[j][e] << 16);
-                sub[j][2 * e + 1] = __uint_as_float(v[j][e] & 0xffff0000u);
+    for (int j = 0; j < kRowVecs; ++j) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            sub[j][e] = 0.0f;
+        }
+    }
+    // windows of 64 items (a token of a built plan has at most K; a saved plan may list any number of duplicates)
+#pragma unroll 1
+    for (int base = 0; base < total; base += kWave) {
+        const int here = total - base < kWave ? total - base : kWave;
+        // lane i < here: item base + i
+        int itemQ = 0;
+        int itemRow = 0;
+        int itemKind = 0;
+        const int32_t *listed = nullptr;             // where a duplicate's row number stands in its rank's dupLoffs
+#pragma unroll 1
+        for (int k = 0; k < K; ++k) {
+            const int items = __builtin_amdgcn_readlane(slotItems, k);
+            if (items == 0) {
+                continue;
             }
-        }
-        constexpr int kBatch = 4;
-        for (int i0 = 0; i0 < count; i0 += kBatch) {
-            u32x4 d[kBatch][kRowVecs];
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                if (i0 + u < count) {
-                    LoadRowSlice(a.hiddenNvsh[q], a.dupLoffs[q][start + i0 + u], h, colBase, lane, G, d[u]);
+            const int q = __builtin_amdgcn_readlane(slotQ, k);
+            const int row = __builtin_amdgcn_readlane(slotRow, k);
+            const int at = base + lane - __builtin_amdgcn_readlane(slotFirst, k);
+            if (at >= 0 && at < items) {
+                itemQ = q;
+                itemRow = row;
+                itemKind = kItemValid | (at == 0 ? kItemOpens : 0) | (at == items - 1 ? kItemCloses : 0);
+            }
+            if (items > 1) {
+                const int32_t *list = a.dupLoffs[q] + __builtin_amdgcn_readlane(slotStart, k);
+                if (at >= 1 && at < items) {
+                    listed = list + (at - 1);
                 }
             }
-#pragma unroll
-            for (int u = 0; u < kBatch; ++u) {
-                if (i0 + u < count) {
-                    AddRow(sub, d[u]);
-                }
-            }
         }
+        if (listed != nullptr) {
+            itemRow = *listed;
+        }
+#pragma unroll 1
+        for (int i0 = 0; i0 < here; i0 += kRowsInFlight) {
+            u32x4 v[kRowsInFlight][kRowVecs];
+            int kind[kRowsInFlight];
 #pragma unroll
-        for (int j = 0; j < kRowVecs; ++j) {
+            for (int u = 0; u < kRowsInFlight; ++u) {
+                // a batch that runs past the window reads its last row again and drops it: four loads are issued
+                // whatever the count, so the sums below wait for exactly the load they need
+                const int i = i0 + u < here ? i0 + u : here - 1;
+                kind[u] = i0 + u < here ? __builtin_amdgcn_readlane(itemKind, i) : 0;
+                const int q = __builtin_amdgcn_readlane(itemQ, i);
+                const int row = __builtin_amdgcn_readlane(itemRow, i);
+                LoadRowSlice(a.hiddenNvsh[q], row, h, vecs, colBase, lane, G, v[u]);
+            }
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const uint32_t packed = TileXREp::FloatPairToBf16Rne(sub[j][2 * e], sub[j][2 * e + 1]);
-                acc[j][2 * e] = __fadd_rn(acc[j][2 * e], __uint_as_float(packed << 16));
-                acc[j][2 * e + 1] = __fadd_rn(acc[j][2 * e + 1], __uint_as_float(packed & 0xffff0000u));
+            for (int u = 0; u < kRowsInFlight; ++u) {
+                if ((kind[u] & kItemValid) != 0) {
+                    StartOrAddRow(sub, v[u], (kind[u] & kItemOpens) != 0);
+                    if ((kind[u] & kItemCloses) != 0) {
+                        AddRounded(acc, sub);
+                    }
+                }
             }
         }
     }
@@ -1074,12 +1138,13 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
     // when they come from HBM
     const int64_t worldRowBytes = static_cast<int64_t>(w.world) * w.s * w.h * 2;
     const bool uncachedRows = worldRowBytes > gCachedRowBytes.load();
-    const bool perRoute = vec && !(uncachedRows && w.s * tokenSlices <= 0x7fffffff) && blocks <= 0x7fffffff;
+    const int64_t rowVecs = w.s * vecs;
+    const bool perToken = vec && uncachedRows && w.s * tokenSlices <= 0x7fffffff;
+    const bool perRoute = vec && !perToken && blocks <= 0x7fffffff;
     // up to half the memory-side cache of token rows: read them once so that the per-route kernel finds them there
     // (one rank's share of 4096 x 7168: 257 -> about 210 us per layer on rows that were not cached, a few us more
     // on rows that were)
     const bool warm = perRoute && worldRowBytes <= kWarmRowBytes;
-    const int64_t rowVecs = w.s * vecs;
     const unsigned warmBlocks = warm ? static_cast<unsigned>((rowVecs + kThreads * kWarmLoads - 1) / (kThreads * kWarmLoads)) : 0u;
     if (!w.fresh) {
         hipLaunchKernelGGL(moon_group_walk_kernel, dim3(rowBlocks, R), dim3(kThreads), 0, stream, w);
@@ -1096,7 +1161,7 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
     if (err != hipSuccess) {
         return err;
     }
-    if (vec && uncachedRows && w.s * tokenSlices <= 0x7fffffff) {
+    if (perToken) {
         gScatterName = "moon_scatter_token_kernel";
         const dim3 grid(static_cast<unsigned>(w.s * tokenSlices), R);
         if (w.fresh) {
@@ -1104,12 +1169,13 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
         } else {
             hipLaunchKernelGGL(moon_scatter_token_kernel<false>, grid, dim3(kTokenThreads), 0, stream, w, tokenSlices);
         }
-    } else if (vec && blocks <= 0x7fffffff) {
+    } else if (perRoute) {
         gScatterName = "moon_scatter_kernel";
+        const dim3 grid(static_cast<unsigned>(blocks), R);
         if (w.fresh) {
-            hipLaunchKernelGGL(moon_scatter_kernel<true>, dim3(static_cast<unsigned>(blocks), R), dim3(kThreads), 0, stream, w, colSlices);
+            hipLaunchKernelGGL(moon_scatter_kernel<true>, grid, dim3(kThreads), 0, stream, w, colSlices);
         } else {
-            hipLaunchKernelGGL(moon_scatter_kernel<false>, dim3(static_cast<unsigned>(blocks), R), dim3(kThreads), 0, stream, w, colSlices);
+            hipLaunchKernelGGL(moon_scatter_kernel<false>, grid, dim3(kThreads), 0, stream, w, colSlices);
         }
     } else {
         gScatterName = "moon_scatter_generic_kernel";
