@@ -179,7 +179,7 @@ def parse():
     return p.parse_args()
 
 
-def measured_ceilings(ep, torch, stream, dev, reps=10, narrow=None):
+def measured_ceilings(ep, torch, stream, dev, reps=10, narrow=None, far=False):
     """What this device's memory system delivers for plain access patterns, measured in this run with the library's
     own probe kernels (HIP events around `reps` launches each): pure read, pure write, copy, and the read : write
     mixes of the scatter (1 : 8) and the reduce (8 : 1).  GB/s of all bytes moved, reads plus writes.  The mixed
@@ -233,6 +233,24 @@ def measured_ceilings(ep, torch, stream, dev, reps=10, narrow=None):
             b.record(stream)
             stream.synchronize()
             out["hipMemcpyDtoD_GBps"] = round(2 * nbytes / (a.elapsed_ms(b) * 1e-3 / reps) / 1e9, 1)
+        del src, dst
+    if far:
+        # the two mixes once more over 2400 MiB: a source of 300 MiB that cannot stay in the 256 MiB memory-side cache
+        # between launches and eight regions 300 MiB apart -- what a world of several ranks on one device looks like
+        nbytes = 2400 << 20
+        src = torch.zeros((nbytes,), dtype=torch.uint8, device=dev)
+        dst = torch.zeros((nbytes,), dtype=torch.uint8, device=dev)
+        torch.cuda.synchronize()
+        for name, pattern in (("fan_out_1r8w_far", ep.PROBE_FAN_OUT), ("fan_in_8r1w_far", ep.PROBE_FAN_IN)):
+            for _ in range(3):
+                ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+            a, b = ep.HipEvent(timing=True), ep.HipEvent(timing=True)
+            a.record(stream)
+            for _ in range(reps):
+                ep.check(ep.memory_probe(pattern, src, dst, nbytes, stream), "memory probe")
+            b.record(stream)
+            stream.synchronize()
+            out[name + "_GBps"] = round((nbytes + nbytes // 8) / (a.elapsed_ms(b) * 1e-3 / reps) / 1e9, 1)
         del src, dst
     if narrow is not None:
         # the quantised reduce's mix with its addresses: rows of 2048 (4096) one-byte payloads, eight (six) per output
@@ -488,9 +506,10 @@ def main_moonep(args):
         roofline["event_pass_us_per_layer"] = round(event_pass_s / args.steps * 1e6, 2)
     ceilings = None
     if not args.no_ceilings:
-        ceilings = measured_ceilings(ep, torch, streams[0], dev)
+        ceilings = measured_ceilings(ep, torch, streams[0], dev, far=world > 1)
         if roofline is not None:
-            mix = ceilings["fan_out_1r8w_GBps"] if dom == "scatter" else ceilings["fan_in_8r1w_GBps"]
+            suffix = "_far_GBps" if world > 1 else "_GBps"
+            mix = ceilings["fan_out_1r8w" + suffix] if dom == "scatter" else ceilings["fan_in_8r1w" + suffix]
             roofline["frac_of_measured_mix"] = round(roofline["achieved"] / mix, 4)
             if dom == "reduce":
                 roofline["frac_of_measured_row_gather"] = round(roofline["achieved"] / ceilings["gather_rows_8r1w_GBps"], 4)
@@ -563,7 +582,7 @@ def main():
     status = torch.zeros((1,), dtype=torch.int32, device=dev)
     meta_ready, combined = ep.HipEvent(), ep.HipEvent()
 
-    def step_plain(d_x=d_x):
+    def step_plain(d_x=d_x, expand_x=expand_x, y=y):
         st, _ = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
                                       ep.DT_BF16, stream, quant_mode=quant, expert_capacity=w.capacity,
                                       dynamic_scales=scales, row_index_map=row_map)
@@ -572,7 +591,7 @@ def main():
                                       expert_out_quant_mode=quant, expert_out_scales=scales, expert_scales=d_w,
                                       row_index_map=row_map), "combine")
 
-    def step_flags_serial(d_x=d_x):
+    def step_flags_serial(d_x=d_x, expand_x=expand_x, y=y):
         # dispatch publishes a readiness word per tile of rows, combine waits for the tiles of every row it reads;
         # one stream, so the waits find every tile published
         st, epoch = ep.dispatch_memory_ex(d_x, d_ids, comm, bs, h, K, E, expand_x, assist, token_nums, send_counts,
@@ -843,7 +862,23 @@ def main():
         rot_us = (time.perf_counter() - t1) / rot_steps * 1e6
         rotating = {"schedule": SCHEDULES["plain" if schedule == "plain" else "flags-serial"], "input_tensors": copies, "steps": rot_steps, "us_per_layer": round(rot_us, 2),
                     "GBps": round((dispatch_bytes + combine_bytes) / (rot_us * 1e-6) / 1e9, 1)}
-        del xs
+        # and with the expanded rows and the output rotating too (sets of x, expandX, y of more than 1 GiB together): a
+        # step that overwrites the rows the previous step has just read finds part of them in the memory-side cache,
+        # a model whose layers have their own buffers, or whose expert stage runs between the two calls, does not
+        set_bytes = bs * h * 2 * 2 + expand_x.numel() * expand_x.element_size()
+        sets = max(2, -(-(1200 << 20) // set_bytes))
+        bufs = [(xs[i % copies], torch.empty_like(expand_x), torch.empty_like(y)) for i in range(sets)]
+        for b in bufs:
+            rot_step(*b)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for i in range(rot_steps):
+            rot_step(*bufs[i % sets])
+        torch.cuda.synchronize()
+        all_us = (time.perf_counter() - t1) / rot_steps * 1e6
+        rotating["all_buffers"] = {"sets": sets, "MiB_per_set": set_bytes >> 20, "us_per_layer": round(all_us, 2),
+                                   "GBps": round((dispatch_bytes + combine_bytes) / (all_us * 1e-6) / 1e9, 1)}
+        del xs, bufs
 
     # the same layer through the reference's own entry points (TileXRMoeEpDispatchMemory / TileXRMoeEpCombineMemoryV2),
     # which carry no row map from dispatch to combine: combine rebuilds it from the assist tuples first.  Plain
@@ -903,13 +938,26 @@ def main():
                 gather = ceilings[narrow[0] + "_GBps"] if narrow is not None else ceilings["gather_rows_8r1w_GBps"]
                 roofline["frac_of_measured_row_gather"] = round(roofline["achieved"] / gather, 4)
 
+    # decode-sized calls move so little that a kernel's time is its chain of dependent trips to memory, not its bytes:
+    # how many loads must return, one after the other, before the kernel's stores can go out
+    round_trips = None
+    if small:
+        round_trips = {
+            "dispatch": {"kernel": kernel_names["scatter"],
+                         "dependent_loads_before_store": {"ep_dispatch_small_route_kernel": 1, "ep_dispatch_small_kernel": 2}.get(kernel_names["scatter"]),
+                         "chain": "expert ids and the token row are requested together; the row is stored when both are back"
+                                  if kernel_names["scatter"] == "ep_dispatch_small_route_kernel" else
+                                  "expert ids, then (per-expert counts known) the token rows, then the stores"},
+            "combine": {"kernel": kernel_names["reduce"], "dependent_loads_before_store": 2,
+                        "chain": "the token's row map entries, then all of its rows at once (eight in flight per lane), then the store"},
+        }
     result = {
         "metric": "dispatch+combine effective HBM bandwidth per MoE layer (algorithmic bytes / time) on 1 MI355X",
         "value": round(gbps, 1), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 5), "us_per_layer": round(ms_per_step * 1e3, 2),
         "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
-        "config": dict(workloads.describe(w, ids), schedule=SCHEDULES[schedule], overlap=schedule == "flags-overlapped",
+        "config": dict(workloads.describe(w, ids), dependent_round_trips=round_trips, schedule=SCHEDULES[schedule], overlap=schedule == "flags-overlapped",
                        tile_rows=args.tile_rows if uses_flags else None, schedule_calibration_us=calibration,
                        other_schedules=other, expert_stage=expert_stage, graph_replay=graph_replay, rotating_inputs=rotating, reference_abi=reference_abi, kept_rows=kept_rows, dispatch_bytes=dispatch_bytes,
                        combine_bytes=combine_bytes, dispatch_us=round(dispatch_us, 2), combine_us=round(combine_us, 2)),

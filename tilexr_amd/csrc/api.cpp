@@ -91,7 +91,7 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
                 small.tileCounters = static_cast<uint32_t *>(comm->tileCounters.ptr);
                 small.epoch = flagEpoch;
             }
-            comm->lastKernel[kKernelScatter] = "ep_dispatch_small_kernel";
+            small.kernelNameOut = &comm->lastKernel[kKernelScatter];
             const int ret = Timed(comm, kKernelScatter, stream, "small dispatch", [&] { return LaunchSmallDispatch(small); });
             if (ret == kOk && p.tileFlagsOut != nullptr) {
                 comm->lastFlagWords = p.tileFlagsOut;

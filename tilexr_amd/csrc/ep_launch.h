@@ -224,6 +224,7 @@ struct SmallDispatchLaunch {
     int64_t tileRows;
     uint64_t epoch;
     hipStream_t stream;
+    const char **kernelNameOut = nullptr;   // optional: receives the name of the kernel template that was launched
 };
 bool SmallDispatchFits(const SmallDispatchLaunch &l);
 hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l);

@@ -27,7 +27,10 @@
 namespace TileXREp {
 namespace {
 
-template <int G, int V, int KIND, bool BF16, int COMMQ, bool FL>
+// WIDE: eight rows in flight per lane instead of four.  For launches with fewer waves than the device has SIMDs
+// (decode): a wave that has a SIMD to itself gains nothing from small registers, and a token's rows arrive in one
+// round trip instead of two.
+template <int G, int V, int KIND, bool BF16, int COMMQ, bool FL, bool WIDE = false>
 __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 {
     constexpr int kTokens = kThreads / G;
@@ -41,7 +44,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
     // Rows in flight per lane.  A whole workgroup per token is the geometry of launches that may wait on flags: at most two
     // such workgroups run per compute unit, so a wave may use half a SIMD's registers and keeps four rows in flight
     // whatever the row width; the other geometries run many more waves and trade rows in flight for occupancy.
-    constexpr int KB = G == kThreads ? 4 : (V <= 2 ? 4 : (V <= 4 ? 2 : 1));
+    constexpr int KB = WIDE ? 8 : (G == kThreads ? 4 : (V <= 2 ? 4 : (V <= 4 ? 2 : 1)));
     const int vecs = a.h / 8;
     // a unit is one token, or -- for wide rows -- one slice of G * V vectors of a token
     const int units = a.bs * a.colSlices;
@@ -196,6 +199,8 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 }
 
 
+constexpr int64_t kWideReduceUnits = 2048;      // token slices (waves) up to which a launch takes the WIDE kernel
+
 template <int G, int V, int KIND, bool BF16, int COMMQ, bool FL>
 void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
 {
@@ -215,6 +220,12 @@ void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
         int grid = static_cast<int>((units + perGroup - 1) / perGroup);
         if (gridLimit > 0 && grid > gridLimit * (kThreads / threads)) {
             grid = gridLimit * (kThreads / threads);
+        }
+        if constexpr (G == kWave && V == 2 && KIND == kReduceFp32 && COMMQ == 0 && !FL) {
+            if (units <= kWideReduceUnits) {
+                hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, FL, true>), dim3(grid), dim3(threads), 0, stream, a);
+                return;
+            }
         }
         hipLaunchKernelGGL((ep_reduce_vec_kernel<G, V, KIND, BF16, COMMQ, FL>), dim3(grid), dim3(threads), 0, stream, a);
     }

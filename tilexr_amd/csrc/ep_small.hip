@@ -324,6 +324,9 @@ hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l)
     auto launch = [&](auto kernel, dim3 grid) { hipLaunchKernelGGL(kernel, grid, dim3(kThreads), 0, l.stream, a); };
     if (l.capacity <= 0 && l.bs * l.topK >= l.numExperts) {
         // one workgroup per route (there are enough of them to cover the experts' count outputs)
+        if (l.kernelNameOut != nullptr) {
+            *l.kernelNameOut = "ep_dispatch_small_route_kernel";
+        }
         const dim3 routes(static_cast<unsigned>(l.bs * l.topK));
         const bool few = l.bs * l.topK <= 4 * kThreads;
         auto pick = [&](auto vecsPerLane) {
@@ -344,6 +347,9 @@ hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l)
         return hipGetLastError();
     }
     const dim3 grid(static_cast<unsigned>(l.bs));
+    if (l.kernelNameOut != nullptr) {
+        *l.kernelNameOut = "ep_dispatch_small_kernel";
+    }
     if (v == 2) {
         flags ? launch(ep_dispatch_small_kernel<2, true>, grid) : launch(ep_dispatch_small_kernel<2, false>, grid);
     } else if (v == 4) {
