@@ -39,15 +39,16 @@ def bits16(t):
 class Session:
     """One communicator (single rank) + a non-default stream."""
 
-    def __init__(self, rank_size=1, rank=0, legacy_routing=False):
-        """legacy_routing: the communicator's dispatches route with the count + place launches even where the
-        one-launch routing applies (the library reads TILEXR_EP_ROUTING when a communicator is created)."""
+    def __init__(self, rank_size=1, rank=0, legacy_routing=None):
+        """legacy_routing: True = the communicator's dispatches route with the count + place launches everywhere,
+        False = with the one-launch routing wherever it can take the call, None = the library picks by the size of the
+        call (it reads TILEXR_EP_ROUTING when a communicator is created)."""
         torch.cuda.set_device(0)
         previous = os.environ.get("TILEXR_EP_ROUTING")
-        if legacy_routing:
-            os.environ["TILEXR_EP_ROUTING"] = "legacy"
-        else:
+        if legacy_routing is None:
             os.environ.pop("TILEXR_EP_ROUTING", None)
+        else:
+            os.environ["TILEXR_EP_ROUTING"] = "legacy" if legacy_routing else "one-launch"
         try:
             self.comm = ep.Comm(rank_size, rank)
         finally:

@@ -128,6 +128,37 @@ def test_one_launch_routing_matches_oracle(case):
         assert np.array_equal(results[0][name], results[2][name]), name
 
 
+def test_routing_kernels_are_picked_by_the_size_of_the_call():
+    """Left to itself the library takes the one-launch routing where it was measured to be the faster one: small
+    tables always, tables up to 65 536 routes only against count + place (readiness flags ask for the rows ahead of
+    the scatter) and while routes x experts stays within 32 768 x 256."""
+    h = 16
+    cases = [  # bs, K, E, flags, kernel
+        (1024, 8, 256, False, "ep_route_rows_kernel"), (2048, 8, 2048, False, "ep_route_count_kernel"),
+        (2048, 8, 2048, True, "ep_route_rows_kernel"), (4096, 8, 256, False, "ep_route_count_kernel"),
+        (4096, 8, 256, True, "ep_route_rows_kernel"), (4096, 8, 512, True, "ep_route_count_kernel"),
+        (4096, 8, 16, True, "ep_route_count_kernel"), (8192, 6, 64, True, "ep_route_rows_kernel"),
+        (8192, 8, 256, True, "ep_route_count_kernel"),
+    ]
+    with Session() as s:
+        for bs, K, E, with_flags, kernel in cases:
+            rng = np.random.default_rng(bs + E)
+            ids = ids_for(rng, bs, K, E)
+            xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+            out = alloc_dispatch_outputs(bs, h, K, E)
+            counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
+            flags = torch.zeros(((bs * K + 63) // 64,), dtype=torch.int64, device=DEV) if with_flags else None
+            torch.cuda.synchronize()
+            st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                          out["token_nums"], counts, ep.DT_BF16, s.stream, row_index_map=out["row_map"],
+                                          tile_flags=flags, tile_rows=64 if with_flags else 0)
+            assert st == 0
+            s.sync()
+            assert ep.last_kernel_name(s.comm, ep.K_COUNT) == kernel, (bs, K, E, with_flags)
+            want = O.mem_dispatch(O.Case(1, bs, h, K, E), 0, xb[None], ids[None])
+            check_dispatch(fetch(out, "send_counts", counts), want)
+
+
 def test_one_launch_routing_with_unaligned_tables():
     """An id table that is not 16-byte aligned takes the count + place routing; an unaligned tuple array takes the
     one-launch routing with four-byte stores."""
@@ -137,7 +168,7 @@ def test_one_launch_routing_with_unaligned_tables():
     xt, xb = x_for(rng, bs, h, ep.DT_BF16)
     want = O.mem_dispatch(O.Case(1, bs, h, K, E, token_nums_type=1), 0, xb[None], ids[None])
     n = want["rows"]
-    with Session() as s:
+    with Session(legacy_routing=False) as s:
         for shift_ids, shift_assist in ((1, 0), (0, 1)):
             out = alloc_dispatch_outputs(bs, h, K, E)
             counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)

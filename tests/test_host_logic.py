@@ -412,7 +412,7 @@ def test_cxx_caller_links_against_the_headers_and_the_library(tmp_path):
     # C++14 like the reference's host code; no HIP or torch header is on the include path
     subprocess.run([gxx, "-std=c++14", "-Wall", "-Wextra", "-Werror", "-I", os.path.join(root, "include"),
                     os.path.join(root, "tests", "cxx", "caller.cpp"), "-o", exe, "-L", lib_dir, "-ltilexr-ep",
-                    f"-Wl,-rpath,{lib_dir}", "-Wl,-rpath-link,/opt/rocm/lib"], check=True)
+                    f"-Wl,-rpath,{lib_dir}", f"-Wl,-rpath-link,{os.environ.get('ROCM_PATH', '/opt/rocm')}/lib"], check=True)
     run = subprocess.run([exe], capture_output=True, text=True)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "caller ok" in run.stdout

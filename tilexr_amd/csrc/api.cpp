@@ -108,10 +108,13 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     } else if (p.xActiveMask != nullptr) {
         maskMode = p.activeMaskType == TILEXR_EP_ACTIVE_MASK_EXPERT ? kMaskPerRoute : kMaskTokenPrefix;
     }
-    // One launch resolves every route's row where the id table is small enough for every workgroup to read all of it
+    // One launch resolves every route's row where every expert's workgroup can afford to read the whole id table
     // (ep_rows.hip); otherwise count (ticket, last workgroup scans) and place, the latter folded into the scatter
     // unless something needs the rows ahead of it.
-    const bool oneLaunch = memoryRoute && !comm->legacyRouting && RouteRowsFits(p.expertIds, n, numKeys, maskMode, p.expertCapacity);
+    const bool rowsAhead = p.tileFlagsOut != nullptr || p.metaReadyEvent != nullptr;
+    const bool oneLaunch = memoryRoute && comm->routing != EpComm::Routing::kLegacy &&
+        RouteRowsFits(p.expertIds, n, numKeys, maskMode, p.expertCapacity) &&
+        (comm->routing == EpComm::Routing::kOneLaunch || RouteRowsPays(n, numKeys, rowsAhead));
     void *scratchBase = nullptr;
     if (p.noAlloc) {
         // this call may not allocate: the per-GPU static array or nothing
@@ -217,7 +220,7 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
         // flags are published: a workgroup that publishes stays until its stores have landed, and resolving the row
         // first (three dependent loads) makes that stay longer (measured on 4096 x 7168 x top-8: scatter 105 us fused,
         // 87 + 4 us apart).
-        separatePlace = p.tileFlagsOut != nullptr || p.metaReadyEvent != nullptr;
+        separatePlace = rowsAhead;
         if (separatePlace) {
             ret = Timed(comm, kKernelPlace, stream, "route place", [&] { return LaunchRoutePlace(place); });
             if (ret != kOk) {

@@ -162,7 +162,11 @@ int TileXRCommInitRankLocal(int rankSize, int rank, TileXRCommPtr *comm)
     c->world = world;
     c->rank = rank;
     const char *routing = std::getenv("TILEXR_EP_ROUTING");
-    c->legacyRouting = routing != nullptr && std::strcmp(routing, "legacy") == 0;
+    if (routing != nullptr && std::strcmp(routing, "legacy") == 0) {
+        c->routing = EpComm::Routing::kLegacy;
+    } else if (routing != nullptr && std::strcmp(routing, "one-launch") == 0) {
+        c->routing = EpComm::Routing::kOneLaunch;
+    }
     c->host.rank = rank;
     c->host.localRank = rank;
     c->host.rankSize = rankSize;

@@ -123,8 +123,11 @@ struct EpComm {
     const void *lastFlagWords = nullptr;
     uint64_t lastFlagEpoch = 0;
     hipStream_t lastFlagStream = nullptr;
-    bool legacyRouting = false;       // TILEXR_EP_ROUTING=legacy when the communicator was created: dispatches route with
-                                      // the count + place launches even where the one-launch routing applies (tests)
+    // TILEXR_EP_ROUTING when the communicator was created (a switch for tests): unset = the library picks the routing
+    // kernels by the size of the call; "legacy" = count (+ place) launches everywhere; "one-launch" = the one-launch
+    // routing wherever it can take the call, also where the other is measured to be faster
+    enum class Routing { kAuto, kLegacy, kOneLaunch };
+    Routing routing = Routing::kAuto;
     DebugState debug;                 // TileXREpSetDebugOptions
     hipEvent_t timing[5][2] = {};     // optional (start, stop) pairs around each kernel, see tilexr_ep.h
     const char *lastKernel[5] = {};   // name of the kernel template last launched for each kernel id

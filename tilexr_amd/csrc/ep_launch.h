@@ -90,6 +90,7 @@ struct RouteRowsLaunch {
     int64_t warmBytes;
     hipStream_t stream;
 };
+bool RouteRowsPays(int64_t routes, int64_t numKeys, bool rowsAhead);
 bool RouteRowsFits(const int32_t *ids, int64_t routes, int64_t numKeys, int maskMode, int64_t capacity);
 hipError_t LaunchRouteRows(const RouteRowsLaunch &l);
 

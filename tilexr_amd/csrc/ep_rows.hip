@@ -242,6 +242,22 @@ bool RouteRowsFits(const int32_t *ids, int64_t routes, int64_t numKeys, int mask
         capacity <= 0 && Aligned16(ids);
 }
 
+// Measured on dispatch + combine layers of 14 KiB rows over 8192 .. 65 536 routes x 8 .. 2048 experts, against count (+ place):
+// every expert's workgroup reads the whole table, so the launch grows with routes x experts where the count launch
+// does not (beyond 512 workgroups of 1024 lanes they run in turns, and the workgroups that read the token rows ahead
+// wait behind them); with few experts the routes of one expert are many and its workgroup numbers them alone.
+//   up to 16 384 routes    4-6 us faster (2-4 us when the other side needs no place launch, up to 512 experts)
+//   up to 65 536 routes    0-3 us faster while routes x experts <= 32 768 x 256 and an expert has 1024 routes or fewer
+//                          on average, and only against count + place (rowsAhead: readiness flags or the metadata
+//                          event want the rows resolved before the scatter); 2-45 us slower beyond that
+bool RouteRowsPays(int64_t routes, int64_t numKeys, bool rowsAhead)
+{
+    if (routes <= 16384) {
+        return rowsAhead || numKeys <= 512;
+    }
+    return rowsAhead && routes * numKeys <= int64_t{32768} * 256 && routes <= numKeys * 1024;
+}
+
 hipError_t LaunchRouteRows(const RouteRowsLaunch &l)
 {
     const int64_t n = l.bs * l.topK;
