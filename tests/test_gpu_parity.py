@@ -79,19 +79,23 @@ ROUTING_SHAPES = [
     (1024, 16, 3, 5, 0.1),          # 3072 routes: not a multiple of 256 per wave, slots 1
     (2049, 16, 1, 1, 0.0),          # one expert, topK 1
     (683, 16, 3, 2048, 0.05),       # as many experts as the tables hold, most of them without a route
-    (4096, 16, 8, 256, 0.0),        # 32 768 routes: the largest table of the eight-slot kernel
-    (4097, 16, 8, 256, 0.02),       # just beyond it: sixteen slots, the last waves hold nothing but padding
-    (8192, 16, 8, 64, 0.0),         # 65 536 routes: the largest table the one-launch routing takes
-    (8193, 16, 8, 64, 0.0),         # one token more: count + place
+    (4096, 16, 8, 256, 0.0),        # 32 768 routes: eight slots per wave, one batch of loads
+    (4097, 16, 8, 256, 0.02),       # just beyond it: nine slots, the last waves hold nothing but padding
+    (8192, 16, 8, 64, 0.0),         # 65 536 routes, 64 experts: four workgroups per expert
+    (8193, 16, 8, 64, 0.0),         # seventeen slots: two parts at least, the second nearly empty
+    (16384, 16, 8, 128, 0.01),      # 131 072 routes: 32 slots per wave in two parts of sixteen
+    (32768, 8, 8, 512, 0.0),        # 262 144 routes: the largest table the one-launch routing takes
+    (32769, 8, 8, 512, 0.0),        # one token more: count + place
     (3000, 16, 7, 37, 1.0),         # no route names an expert
     (3000, 16, 6, 9, 0.0),          # few experts: thousands of routes per key, several per lane and slot
+    (4096, 16, 8, 8, 0.0),          # eight experts, eight workgroups each: one slot of every wave's eight per workgroup
 ]
 
 
 @pytest.mark.parametrize("case", ROUTING_SHAPES)
 def test_one_launch_routing_matches_oracle(case):
     """The routing kernel that resolves every route's row in one launch (memory route, no mask, no capacity limit, up
-    to 65 536 routes), at the edges of what it takes; ids drawn with repeats within a token too.  Compared with the
+    to 262 144 routes), at the edges of what it takes; ids drawn with repeats within a token too.  Compared with the
     oracle and, bit for bit, with the count + place routing on the same inputs."""
     bs, h, K, E, invalid = case
     rng = np.random.default_rng(bs * 31 + K * 7 + E)
@@ -112,7 +116,7 @@ def test_one_launch_routing_matches_oracle(case):
                                               token_nums_type=nums_type, row_index_map=out["row_map"])
                 assert st == 0
                 s.sync()
-                expect = "ep_route_count_kernel" if legacy or bs * K > 65536 else "ep_route_rows_kernel"
+                expect = "ep_route_count_kernel" if legacy or bs * K > 262144 else "ep_route_rows_kernel"
                 assert ep.last_kernel_name(s.comm, ep.K_COUNT) == expect
                 got = fetch(out, "send_counts", counts)
                 want = O.mem_dispatch(O.Case(1, bs, h, K, E, token_nums_type=nums_type), 0, xb[None], ids[None])
@@ -130,20 +134,21 @@ def test_one_launch_routing_matches_oracle(case):
 
 def test_routing_kernels_are_picked_by_the_size_of_the_call():
     """Left to itself the library takes the one-launch routing where it was measured to be the faster one: small
-    tables always, tables up to 65 536 routes only against count + place (readiness flags ask for the rows ahead of
-    the scatter) and while routes x experts stays within 32 768 x 256."""
-    h = 16
-    cases = [  # bs, K, E, flags, kernel
-        (1024, 8, 256, False, "ep_route_rows_kernel"), (2048, 8, 2048, False, "ep_route_count_kernel"),
-        (2048, 8, 2048, True, "ep_route_rows_kernel"), (4096, 8, 256, False, "ep_route_count_kernel"),
-        (4096, 8, 256, True, "ep_route_rows_kernel"), (4096, 8, 512, True, "ep_route_count_kernel"),
-        (4096, 8, 16, True, "ep_route_count_kernel"), (8192, 6, 64, True, "ep_route_rows_kernel"),
-        (8192, 8, 256, True, "ep_route_count_kernel"),
+    tables always; larger ones while routes x experts stays small, less far when the same launch also reads token rows
+    ahead of a scatter that copies per route (rows wider than 4 KiB, plain payload) and then only against count + place
+    (readiness flags ask for the rows ahead of the scatter)."""
+    cases = [  # bs, K, E, h, flags, kernel
+        (1024, 8, 256, 16, False, "ep_route_rows_kernel"), (2048, 8, 2048, 16, False, "ep_route_count_kernel"),
+        (2048, 8, 2048, 16, True, "ep_route_rows_kernel"), (4096, 8, 256, 16, False, "ep_route_rows_kernel"),
+        (4096, 8, 1024, 16, True, "ep_route_count_kernel"), (8192, 6, 64, 16, True, "ep_route_rows_kernel"),
+        (8192, 8, 256, 16, True, "ep_route_count_kernel"), (16384, 8, 64, 16, False, "ep_route_count_kernel"),
+        (4096, 8, 256, 2056, False, "ep_route_count_kernel"), (4096, 8, 256, 2056, True, "ep_route_rows_kernel"),
+        (4096, 8, 512, 2056, True, "ep_route_count_kernel"), (6144, 8, 64, 2056, True, "ep_route_count_kernel"),
     ]
     with Session() as s:
-        for bs, K, E, with_flags, kernel in cases:
+        for bs, K, E, h, with_flags, kernel in cases:
             rng = np.random.default_rng(bs + E)
-            ids = ids_for(rng, bs, K, E)
+            ids = rng.integers(0, E, (bs, K)).astype(np.int32)
             xt, xb = x_for(rng, bs, h, ep.DT_BF16)
             out = alloc_dispatch_outputs(bs, h, K, E)
             counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
@@ -154,9 +159,11 @@ def test_routing_kernels_are_picked_by_the_size_of_the_call():
                                           tile_flags=flags, tile_rows=64 if with_flags else 0)
             assert st == 0
             s.sync()
-            assert ep.last_kernel_name(s.comm, ep.K_COUNT) == kernel, (bs, K, E, with_flags)
-            want = O.mem_dispatch(O.Case(1, bs, h, K, E), 0, xb[None], ids[None])
-            check_dispatch(fetch(out, "send_counts", counts), want)
+            assert ep.last_kernel_name(s.comm, ep.K_COUNT) == kernel, (bs, K, E, h, with_flags)
+            if h == 16:
+                want = O.mem_dispatch(O.Case(1, bs, h, K, E), 0, xb[None], ids[None])
+                check_dispatch(fetch(out, "send_counts", counts), want)
+            del out
 
 
 def test_one_launch_routing_with_unaligned_tables():

@@ -112,9 +112,11 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     // (ep_rows.hip); otherwise count (ticket, last workgroup scans) and place, the latter folded into the scatter
     // unless something needs the rows ahead of it.
     const bool rowsAhead = p.tileFlagsOut != nullptr || p.metaReadyEvent != nullptr;
+    // the scatter kernel that copies per route wants the token rows close by: the routing launch reads them ahead
+    const bool warm = ScatterCopiesPerRoute(p.x, p.expandXOut, p.bs, p.h, p.topK, static_cast<int>(p.quantMode));
     const bool oneLaunch = memoryRoute && comm->routing != EpComm::Routing::kLegacy &&
         RouteRowsFits(p.expertIds, n, numKeys, maskMode, p.expertCapacity) &&
-        (comm->routing == EpComm::Routing::kOneLaunch || RouteRowsPays(n, numKeys, rowsAhead));
+        (comm->routing == EpComm::Routing::kOneLaunch || RouteRowsPays(n, numKeys, rowsAhead, warm));
     void *scratchBase = nullptr;
     if (p.noAlloc) {
         // this call may not allocate: the per-GPU static array or nothing
@@ -140,8 +142,6 @@ int RunDispatchSingle(EpComm *comm, const EpDispatchParams &p, bool memoryRoute,
     const CountScratch scratch = CarveCountScratch(scratchBase, plan, expertHist);
     int32_t *rowOf = p.rowIndexMapOut != nullptr ? p.rowIndexMapOut :
         reinterpret_cast<int32_t *>(static_cast<char *>(scratchBase) + plan.rowOfOff);
-    // the scatter kernel that copies per route wants the token rows close by
-    const bool warm = ScatterCopiesPerRoute(p.x, p.expandXOut, p.bs, p.h, p.topK, static_cast<int>(p.quantMode));
     int ret = kOk;
     RoutePlaceLaunch place {};
     bool separatePlace = false;

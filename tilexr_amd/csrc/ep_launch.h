@@ -72,7 +72,7 @@ struct RouteCountLaunch {
 
 // Memory route, one rank, keys = experts, no mask, no capacity limit: rows and assist tuples of all routes in one launch
 // (ep_rows.hip), for id tables small enough that every workgroup reads the whole table itself.
-constexpr int kRowsTableRoutes = 65536;
+constexpr int kRowsTableRoutes = 262144;
 struct RouteRowsLaunch {
     const int32_t *ids;
     int64_t bs;
@@ -90,7 +90,7 @@ struct RouteRowsLaunch {
     int64_t warmBytes;
     hipStream_t stream;
 };
-bool RouteRowsPays(int64_t routes, int64_t numKeys, bool rowsAhead);
+bool RouteRowsPays(int64_t routes, int64_t numKeys, bool rowsAhead, bool readsRowsAhead);
 bool RouteRowsFits(const int32_t *ids, int64_t routes, int64_t numKeys, int maskMode, int64_t capacity);
 hipError_t LaunchRouteRows(const RouteRowsLaunch &l);
 
