@@ -132,6 +132,41 @@ def test_one_launch_routing_matches_oracle(case):
         assert np.array_equal(results[0][name], results[2][name]), name
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_one_launch_routing_on_random_tables(seed):
+    """Tables of random size (up to 120 000 routes: one to thirty slots per wave, one to sixteen workgroups per key),
+    random topK and expert count, ids with repeats and a random share of ids that name no expert: rows, tuples, counts
+    and row map against the oracle."""
+    rng = np.random.default_rng(9000 + seed)
+    K = int(rng.integers(1, 10))
+    bs = int(rng.integers(1, 120000 // K + 1)) if seed % 4 else int(rng.integers(1, 3000))
+    E = int(rng.choice([1, 2, 3, 7, 8, 16, 33, 64, 100, 256, 257, 700, 2048]))
+    h = 8
+    ids = rng.integers(0, E, (bs, K)).astype(np.int32)
+    bad = rng.random(ids.shape) < float(rng.choice([0.0, 0.01, 0.3]))
+    ids[bad] = rng.choice([-1, -9, E, E + 3, 2 ** 31 - 1, -2 ** 31], size=int(bad.sum()))
+    xt, xb = x_for(rng, bs, h, ep.DT_BF16)
+    nums_type = seed % 2
+    with Session(legacy_routing=False) as s:
+        out = alloc_dispatch_outputs(bs, h, K, E)
+        counts = torch.full((E,), -1, dtype=torch.int32, device=DEV)
+        st, _ = ep.dispatch_memory_ex(xt, to_dev(ids), s.comm, bs, h, K, E, out["expand_x"], out["assist"],
+                                      out["token_nums"], counts, ep.DT_BF16, s.stream, token_nums_type=nums_type,
+                                      row_index_map=out["row_map"])
+        assert st == 0
+        s.sync()
+        small = bs * K <= 2048       # decode-sized calls take the single-launch dispatch whatever the switch says
+        assert small or ep.last_kernel_name(s.comm, ep.K_COUNT) == "ep_route_rows_kernel"
+        got = fetch(out, "send_counts", counts)
+        want = O.mem_dispatch(O.Case(1, bs, h, K, E, token_nums_type=nums_type), 0, xb[None], ids[None])
+        check_dispatch(got, want)
+        assert np.array_equal(got["send_counts"], want["send_counts"])
+        rm = np.full(bs * K, -1, np.int32)
+        n = want["rows"]
+        rm[want["assist"][:n, 1] * K + want["assist"][:n, 2]] = np.arange(n, dtype=np.int32)
+        assert np.array_equal(got["row_map"].reshape(-1), rm)
+
+
 def test_routing_kernels_are_picked_by_the_size_of_the_call():
     """Left to itself the library takes the one-launch routing where it was measured to be the faster one: small
     tables always; larger ones while routes x experts stays small, less far when the same launch also reads token rows
