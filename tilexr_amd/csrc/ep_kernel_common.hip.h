@@ -54,6 +54,15 @@ constexpr int kAuxAgentScopeKept = 16;      // sc1 alone: for small tables a lat
                                             // the same table afterwards ran 10 us slower: 92 instead of 82 us)
 constexpr unsigned kRawBufferWord3 = 0x00020000u;
 
+// Workgroup b of a launch runs on XCD b % kXcdCount.  Units (token x part) placed by XCD: unit u belongs to token
+// (u / 8 / parts) * 8 + u % 8, part (u / 8) % parts, so that all parts of a token run on XCD token % 8; the tokens are
+// padded to a multiple of eight.
+constexpr int kXcdCount = 8;
+__host__ __device__ inline int XcdPlacedUnits(int tokens, int parts)
+{
+    return (tokens + kXcdCount - 1) / kXcdCount * kXcdCount * parts;
+}
+
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t RowResource(const void *row, int bytes)
 {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(row), 0, bytes, kRawBufferWord3);

@@ -192,12 +192,18 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
     const int tid = threadIdx.x;
     const int lane = tid & (kWave - 1);
     const int wave = tid / kWave;
-    const int route = blockIdx.x;
-    const int token = route / a.topK;
+    // Workgroup b runs on XCD b % 8: the K routes of token t go to workgroups of XCD t % 8, where the decode-sized
+    // combine places the token's slices as well, so that the rows it reads are still in the L2 that they were written
+    // through (the tokens are padded to a multiple of eight: a workgroup of the padding has no route, only an expert to
+    // count for).
+    const int placed = static_cast<int>(blockIdx.x) / kXcdCount;
+    const int token = (placed / a.topK) * kXcdCount + static_cast<int>(blockIdx.x) % kXcdCount;
+    const bool hasRoute = token < a.bs;
+    const int route = hasRoute ? token * a.topK + placed % a.topK : 0;
     const int n = a.bs * a.topK;
     const int vecs = a.h / 8;
 
-    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.x) + static_cast<int64_t>(token) * a.h * 2);
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(static_cast<const char *>(a.x) + static_cast<int64_t>(hasRoute ? token : 0) * a.h * 2);
     u32x4 v[V];
 #pragma unroll
     for (int j = 0; j < V; ++j) {
@@ -212,7 +218,7 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
     }
     const int mine = a.ids[route];
     const unsigned experts = static_cast<unsigned>(a.numExperts);
-    const int key = static_cast<unsigned>(mine) < experts ? mine : -1;       // ids outside [0, E) are skipped, not errors
+    const int key = hasRoute && static_cast<unsigned>(mine) < experts ? mine : -1;       // ids outside [0, E) are skipped, not errors
     const int expert = blockIdx.x;       // the expert this workgroup counts for the outputs (if there is one)
     int rowCounts = 0;      // valid ids below the key | earlier ids equal to it << 16
     int outCounts = 0;      // ids equal to `expert` | valid ids not above it << 16
@@ -250,7 +256,7 @@ __global__ __launch_bounds__(kThreads) void ep_dispatch_small_route_kernel(Small
             tuple[2] = route % a.topK;
             tuple[3] = key + a.expertIdBias;
         }
-        if (a.rowOf != nullptr) {
+        if (a.rowOf != nullptr && hasRoute) {
             a.rowOf[route] = row;
         }
         if (expert < a.numExperts) {
@@ -327,7 +333,7 @@ hipError_t LaunchSmallDispatch(const SmallDispatchLaunch &l)
         if (l.kernelNameOut != nullptr) {
             *l.kernelNameOut = "ep_dispatch_small_route_kernel";
         }
-        const dim3 routes(static_cast<unsigned>(l.bs * l.topK));
+        const dim3 routes(static_cast<unsigned>(XcdPlacedUnits(static_cast<int>(l.bs), static_cast<int>(l.topK))));
         const bool few = l.bs * l.topK <= 4 * kThreads;
         auto pick = [&](auto vecsPerLane) {
             constexpr int kV = decltype(vecsPerLane)::value;
