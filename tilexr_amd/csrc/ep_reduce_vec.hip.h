@@ -114,7 +114,10 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                 acc[j][e] = 0.0f;
             }
         }
-        uint64_t todo = __ballot(myRow >= 0);
+        // WIDE takes the slots as they stand, eight per trip (lane numbers known when the code is built: no chain of
+        // scalar instructions from one slot to the next); the others compact the slots that have a row
+        uint64_t todo = WIDE ? (a.slots > 0 ? 1ull : 0ull) : __ballot(myRow >= 0);
+        int firstSlot = 0;
         // control flow below is uniform across the lanes that share a token (the MXFP8 round trip shuffles)
         while (todo != 0) {
             u32x4 v16[KB][V];
@@ -122,18 +125,27 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
             float weightOfK[KB];
 #pragma unroll
             for (int u = 0; u < KB; ++u) {
-                const bool any = todo != 0;
-                const int k = any ? __builtin_ctzll(todo) : 0;
-                todo &= todo - 1;
+                const bool any = WIDE ? firstSlot + u < a.slots : todo != 0;
+                const int k = WIDE ? firstSlot + u : (any ? __builtin_ctzll(todo) : 0);
+                if (!WIDE) {
+                    todo &= todo - 1;
+                }
                 const int row = any ? __builtin_amdgcn_readlane(myRow, k) : -1;
                 rowOfK[u] = row;
                 weightOfK[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(myWeight), k));
                 const char *base = static_cast<const char *>(a.expertOut) + static_cast<int64_t>(row < 0 ? 0 : row) * a.rowBytes;
-                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, vecs * 16);
+                // WIDE: a slot without a row gets a resource of no bytes, and a lane beyond the row's end is beyond the
+                // resource's: both read as zeros without a test per load (at this size the kernel is paid in
+                // instructions)
+                const __amdgpu_buffer_rsrc_t rsrc = RowResource(base, WIDE && row < 0 ? 0 : vecs * 16);
 #pragma unroll
                 for (int j = 0; j < V; ++j) {
                     const int idx = colBase + j * G + lane;
-                    v16[u][j] = (row >= 0 && idx < vecs) ? RowLoad<FL>(base, rsrc, idx * 16) : u32x4{0u, 0u, 0u, 0u};
+                    if (WIDE) {
+                        v16[u][j] = __builtin_amdgcn_raw_buffer_load_b128(rsrc, idx * 16, 0, kAuxNonTemporal);
+                    } else {
+                        v16[u][j] = (row >= 0 && idx < vecs) ? RowLoad<FL>(base, rsrc, idx * 16) : u32x4{0u, 0u, 0u, 0u};
+                    }
                 }
             }
 #pragma unroll
@@ -178,6 +190,10 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
                         }
                     }
                 }
+            }
+            if (WIDE) {
+                firstSlot += KB;
+                todo = firstSlot < a.slots ? 1ull : 0ull;
             }
         }
         if (a.sharedExpertX != nullptr && active) {
