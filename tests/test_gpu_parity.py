@@ -39,7 +39,7 @@ def check_dispatch(got, want, rows_key="rows"):
 
 
 SHAPES = [(7, 8, 2, 5), (64, 64, 4, 16), (33, 40, 3, 7), (16, 33, 2, 4), (300, 1024, 8, 64), (2100, 256, 8, 256),
-          (128, 7168, 8, 256), (5, 16400, 2, 4)]
+          (128, 7168, 8, 256), (5, 16400, 2, 4), (19, 2048, 12, 32)]
 
 
 @pytest.mark.parametrize("shape", SHAPES)
