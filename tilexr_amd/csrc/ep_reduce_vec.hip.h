@@ -22,6 +22,8 @@
 #error "include from ep_reduce_vec_*.hip"
 #endif
 
+#include <algorithm>
+
 #include "ep_reduce_common.hip.h"
 
 namespace TileXREp {
@@ -29,11 +31,26 @@ namespace {
 
 // WIDE: eight rows in flight per lane instead of four.  For launches with fewer waves than the device has SIMDs
 // (decode): a wave that has a SIMD to itself gains nothing from small registers, and a token's rows arrive in one
-// round trip instead of two.  Such a launch with sliced rows (single-wave workgroups) also places its units by XCD:
-// workgroup b runs on XCD b % 8 and takes a slice of a token t with t % 8 == b % 8, as the decode-sized dispatch does
-// with a token's routes, so that rows which still sit in the L2 of the XCD that wrote them are read there (the eight L2s
-// are not one cache: rows written on one XCD and read on another travel through memory; 128 tokens x 7168 x top-8,
-// dispatch and combine in turn: 8.4 + 6.3 us without the placement, 5.7 + 3.2 us with it).
+// round trip instead of two.
+//
+// Launches with sliced rows (single-wave workgroups) that do not wait place their units by XCD: workgroup b runs on
+// XCD b % 8 and takes a slice of a token t with t % 8 == b % 8, as the dispatch kernels do with a token's routes, so that
+// rows which still sit in the L2 of the XCD that wrote them are read there (the eight L2s are not one cache: rows
+// written on one XCD and read on another travel through memory).  128 tokens x 7168 x top-8, dispatch and combine in
+// turn: 8.4 + 6.3 us without the placement, 5.7 + 3.2 us with it; a layer of 384 tokens 26.6 -> 21.5 us; from 1024 tokens
+// on (117 MB of rows against 32 MB of L2) it makes no difference, and the launch keeps the plain order.
+template <bool FL>
+__host__ __device__ inline bool PlacesByXcd(const ReduceArgs &a, int lanesPerUnit)
+{
+    // sliced rows are launched with one wave per workgroup and one unit per wave; a launch that may wait has whole
+    // workgroups per token and claims them as they become ready.  Up to three times the L2s' 32 MB of rows: beyond that
+    // nothing is left to find there, and consecutive workgroups that read consecutive slices of the same rows are the
+    // better order for memory (4096 tokens x 7168 x top-8: 88.7 us against 90.3 us placed by XCD)
+    constexpr int64_t kPlacedRowBytes = int64_t{96} << 20;
+    return lanesPerUnit == kWave && a.colSlices > 1 && (!FL || a.flagsSettled != 0) &&
+        static_cast<int64_t>(a.bs) * a.slots * a.rowBytes <= kPlacedRowBytes;
+}
+
 template <int G, int V, int KIND, bool BF16, int COMMQ, bool FL, bool WIDE = false>
 __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
 {
@@ -53,7 +70,7 @@ __global__ __launch_bounds__(kThreads) void ep_reduce_vec_kernel(ReduceArgs a)
     // a unit is one token, or -- for wide rows -- one slice of G * V vectors of a token
     // the launch may use fewer waves per workgroup than kThreads / kWave (single-wave workgroups for sliced rows)
     const int unitsPerGroup = static_cast<int>(blockDim.x) / G;
-    const bool byXcd = WIDE && unitsPerGroup == 1;
+    const bool byXcd = PlacesByXcd<FL>(a, G);
     const int units = byXcd ? XcdPlacedUnits(a.bs, a.colSlices) : a.bs * a.colSlices;
     const int groups = (units + unitsPerGroup - 1) / unitsPerGroup;
 
@@ -254,13 +271,14 @@ void LaunchVec(const ReduceArgs &a, int gridLimit, hipStream_t stream)
         bool wide = false;
         if constexpr (G == kWave && V == 2 && KIND == kReduceFp32 && COMMQ == 0 && !FL) {
             wide = units <= kWideReduceUnits;
-            if (wide && perGroup == 1) {
-                units = XcdPlacedUnits(a.bs, a.colSlices);
-            }
+        }
+        if (PlacesByXcd<FL>(a, G)) {
+            units = XcdPlacedUnits(a.bs, a.colSlices);
         }
         int grid = static_cast<int>((units + perGroup - 1) / perGroup);
         if (gridLimit > 0 && grid > gridLimit * (kThreads / threads)) {
-            grid = gridLimit * (kThreads / threads);
+            // a multiple of eight, so that a workgroup's later units (blockIdx.x + i * gridDim.x) stay on its XCD
+            grid = std::max(gridLimit * (kThreads / threads) / kXcdCount * kXcdCount, kXcdCount);
         }
         if constexpr (G == kWave && V == 2 && KIND == kReduceFp32 && COMMQ == 0 && !FL) {
             if (wide) {
