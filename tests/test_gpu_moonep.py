@@ -342,6 +342,37 @@ def test_combine_with_groups_longer_than_a_wave():
             np.testing.assert_array_equal(got, by_hand[r])
 
 
+def test_rows_that_are_not_finite():
+    """Infinities, the largest finite values, NaNs and zeros of both signs among the rows, with and without duplicate
+    groups: dispatch copies bits; combine's sums equal the oracle's element for element, NaNs up to sign and payload
+    (which of two NaN operands an addition returns differs between the host's adder and the device's)."""
+    world, s, k, h = 2, 24, 4, 72
+    rng = np.random.default_rng(405)
+    special = np.array([0x7f80, 0xff80, 0x7f7f, 0xff7f, 0x7fc0, 0xffc1, 0x7f81, 0x0000, 0x8000, 0x0001, 0x3f80, 0xbf80], np.uint16)
+    for dups in (False, True):
+        sh = M.Shape(world, s, k, h, s * k + 5)
+        dst = MC.random_dst(sh, rng, duplicates=dups)
+        hidden = special[rng.integers(0, len(special), size=(world, s, h))]
+        want_out, _, _, want_dup = M.dispatch_world(sh, dst, hidden, flags=M.FLAG_BUILD_DEDUP)
+        with World(world) as w:
+            plans = w.plan_tensors(sh, dst)
+            res = w.dispatch(sh, plans, hidden, flags=mp.FLAG_BUILD_DEDUP)
+            w.sync()
+            for r in range(world):
+                assert int(plans[r]["status"][0].item()) == mp.DISPATCH_STATUS_SUCCESS
+                np.testing.assert_array_equal(host_bits16(res[r]["out"]), want_out[r])
+            dl = M.build_dst_local(sh, dst)
+            got = w.combine(sh, plans, dl, [res[r]["out"] for r in range(world)])
+            w.sync()
+            want_y, _, _ = M.combine_world(sh, dl, want_dup, want_out)
+            for r in range(world):
+                a, b = host_bits16(got[r]["y"]), want_y[r]
+                nan_a, nan_b = (a & 0x7fff) > 0x7f80, (b & 0x7fff) > 0x7f80
+                np.testing.assert_array_equal(nan_a, nan_b)
+                np.testing.assert_array_equal(a[~nan_a], b[~nan_b])
+                assert nan_a.any() and ((a & 0x7fff) == 0x7f80).any()
+
+
 def test_device_status_of_bad_plans(row_cache):
     world, s, k, h = 3, 8, 2, 64
     rng = np.random.default_rng(9)

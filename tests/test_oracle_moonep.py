@@ -114,6 +114,35 @@ def test_without_duplicates_oracle_equals_reference_model(mref, world, s, k, h, 
     np.testing.assert_array_equal(wy, rwy)
 
 
+def same_up_to_nan_payload(a, b):
+    """Equal bit for bit, except that two NaNs may differ in sign and payload (which of two NaN operands an addition
+    returns is the adder's business: the CPU's and the GPU's differ)."""
+    a, b = np.asarray(a, np.uint16), np.asarray(b, np.uint16)
+    nan_a, nan_b = (a & 0x7fff) > 0x7f80, (b & 0x7fff) > 0x7f80
+    return np.array_equal(nan_a, nan_b) and np.array_equal(a[~nan_a], b[~nan_b])
+
+
+def test_rows_that_are_not_finite_against_reference_model(mref):
+    """Infinities, the largest finite values (sums that overflow), NaNs and zeros of both signs among the rows: dispatch
+    copies bits; combine's sums agree with the reference's CPU model element for element, NaNs up to their payload."""
+    world, s, k, h = 2, 12, 4, 16
+    rng = np.random.default_rng(404)
+    sh = M.Shape(world, s, k, h, s * k + 3)
+    dst = MC.random_dst(sh, rng, duplicates=False)
+    special = np.array([0x7f80, 0xff80, 0x7f7f, 0xff7f, 0x7fc0, 0xffc1, 0x7f81, 0x0000, 0x8000, 0x0001, 0x3f80, 0xbf80], np.uint16)
+    hidden = special[rng.integers(0, len(special), size=(world, s, h))]
+    out, _, status, dup = M.dispatch_world(sh, dst, hidden, flags=M.FLAG_BUILD_DEDUP)
+    rout, _ = mref.ref_dispatch(sh, dst, hidden)
+    assert status.tolist() == [M.DISPATCH_OK] * world
+    np.testing.assert_array_equal(out, rout)
+    y, _, cstatus = M.combine_world(sh, M.build_dst_local(sh, dst), dup, out)
+    ry, _ = mref.ref_combine(sh, dst, out)
+    assert cstatus.tolist() == [M.COMBINE_OK] * world
+    assert same_up_to_nan_payload(y, ry)
+    kinds = ((y & 0x7fff) > 0x7f80).sum(), ((y & 0x7fff) == 0x7f80).sum()
+    assert kinds[0] > 0 and kinds[1] > 0          # the draw does produce NaN sums (inf - inf) and infinite ones
+
+
 @pytest.mark.parametrize("world,s,k,h", [(1, 6, 4, 8), (2, 5, 4, 8), (4, 4, 8, 16), (8, 2, 32, 8)])
 def test_with_duplicates_against_reference_model(mref, world, s, k, h):
     rng = np.random.default_rng(world * 7 + k)
