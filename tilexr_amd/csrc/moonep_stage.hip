@@ -907,22 +907,36 @@ __device__ __forceinline__ void AddRounded(float (&acc)[kRowVecs][8], const floa
 // they are summed -- becomes an item of one lane (which tensor, which row, what to do with it), so that all look-ups
 // (slot tables, then the duplicates' row numbers) are two round trips for the whole token whatever its groups look like,
 // and the rows themselves are read four at a time.  Items are dealt to the lanes 64 at a time.
+//
+// `placed`: units are dealt by XCD (workgroup b runs on XCD b % 8 and takes a slice of a token t with t % 8 == b % 8, the
+// XCD on which the scatter kernels run the token's routes), for worlds whose rows can still be in the XCDs' L2s when
+// Combine follows Dispatch: rows written on one XCD and read on another travel through memory.  The tokens are padded
+// to a multiple of eight.
 template <int G>
-__global__ __launch_bounds__(G) void moon_reduce_kernel(CombineWorld a, int colSlices)
+__global__ __launch_bounds__(G) void moon_reduce_kernel(CombineWorld a, int colSlices, int placed)
 {
     static_assert(G == kWave, "the items of a token are spread over the lanes of one wave");
     constexpr int kRowsInFlight = 4;
     __shared__ TokenSlots s_slots;
     const int rank = blockIdx.y;
     const int unit = blockIdx.x;
-    const int token = unit / colSlices;
-    const int colBase = (unit % colSlices) * (G * kRowVecs);
+    int token = unit / colSlices;
+    int slice = unit % colSlices;
+    if (placed != 0) {
+        const int j = unit / kXcds;
+        token = (j / colSlices) * kXcds + unit % kXcds;
+        slice = j % colSlices;
+    }
     const int lane = threadIdx.x;
-    const int h = static_cast<int>(a.h);
-    const int vecs = h / 8;
     if (unit == 0 && lane == 0) {
         WriteCombineStatus(a, rank);
     }
+    if (token >= a.s) {
+        return;
+    }
+    const int colBase = slice * (G * kRowVecs);
+    const int h = static_cast<int>(a.h);
+    const int vecs = h / 8;
     LoadSlots(a, rank, token, colBase == 0, &s_slots);
     TileXREp::LdsBarrier();
     float acc[kRowVecs][8];
@@ -1224,14 +1238,17 @@ hipError_t LaunchMoonCombine(const CombineWorld &w, hipStream_t stream, const La
     const int64_t vecs = w.h / 8;
     constexpr int G = kWave;
     const int colSlices = static_cast<int>((vecs + G * kRowVecs - 1) / (G * kRowVecs));
-    const int64_t units = w.s * colSlices;
+    // up to three times the L2s' 32 MB of receive rows in the world: the slices of a token go to the XCD that wrote its rows
+    const bool placed = static_cast<int64_t>(w.world) * w.nvS * w.h * 2 <= (int64_t{96} << 20);
+    const int64_t units = (placed ? (w.s + kXcds - 1) / kXcds * kXcds : w.s) * colSlices;
     hipError_t err = RecordIf(timing.start, stream);
     if (err != hipSuccess) {
         return err;
     }
     if (vec && units <= 0x7fffffff) {
         gReduceName = "moon_reduce_kernel";
-        hipLaunchKernelGGL(moon_reduce_kernel<G>, dim3(static_cast<unsigned>(units), R), dim3(G), 0, stream, w, colSlices);
+        hipLaunchKernelGGL(moon_reduce_kernel<G>, dim3(static_cast<unsigned>(units), R), dim3(G), 0, stream, w, colSlices,
+            placed ? 1 : 0);
     } else {
         gReduceName = "moon_reduce_generic_kernel";
         hipLaunchKernelGGL(moon_reduce_generic_kernel, dim3(static_cast<unsigned>(w.s), R), dim3(kThreads), 0, stream, w);
