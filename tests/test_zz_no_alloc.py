@@ -59,6 +59,26 @@ def test_no_alloc_dispatch_matches_the_allocating_entry_point(legacy_routing):
             assert 0 < rows <= bs * K
 
 
+def test_no_alloc_dispatch_at_the_largest_size_it_documents():
+    """131 072 routes over 2048 experts: the count scratch of the largest call the header promises fits the array."""
+    bs, h, K, E = 16384, 8, 8, 2048
+    rng = np.random.default_rng(21)
+    ids = rng.integers(0, E, (bs, K)).astype(np.int32)
+    x = torch.from_numpy(rng.standard_normal((bs, h)).astype(np.float32)).to(torch.bfloat16).to(DEV)
+    d_ids = torch.from_numpy(ids).to(DEV)
+    with Session() as s:
+        want, got = _outputs(bs, h, K, E, 3.0), _outputs(bs, h, K, E, 3.0)
+        torch.cuda.synchronize()
+        assert _call(ep.dispatch_memory, s, x, d_ids, bs, h, K, E, want) == 0
+        assert _call(ep.dispatch_memory_no_alloc, s, x, d_ids, bs, h, K, E, got) == 0
+        s.sync()
+        assert ep.last_kernel_name(s.comm, ep.K_COUNT) == "ep_route_count_kernel"
+        for name in want:
+            assert torch.equal(want[name].view(torch.int16) if name == "expand_x" else want[name],
+                               got[name].view(torch.int16) if name == "expand_x" else got[name]), name
+        assert int(got["counts"][-1].item()) == bs * K
+
+
 def test_no_alloc_dispatch_rejects_what_does_not_fit():
     with Session() as s:
         fake = torch.zeros((16,), dtype=torch.int32, device=DEV)

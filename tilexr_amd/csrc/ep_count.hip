@@ -359,7 +359,8 @@ CountScratchLayout PlanCountScratch(int64_t routes, int64_t numKeys, int64_t num
     auto align = [](int64_t v) { return (v + 255) / 256 * 256; };
     CountScratchLayout p {};
     p.chunkShift = kMinChunkShift;
-    while (p.chunkShift < kMaxChunkShift && ((routes + (1ll << p.chunkShift) - 1) >> p.chunkShift) > kTargetChunks) {
+    const int64_t targetChunks = numKeys > 1024 ? kTargetChunks / 2 : kTargetChunks;
+    while (p.chunkShift < kMaxChunkShift && ((routes + (1ll << p.chunkShift) - 1) >> p.chunkShift) > targetChunks) {
         ++p.chunkShift;
     }
 
