@@ -7,6 +7,7 @@
 //
 // Routing: token t picks experts (t + k * (experts / topK)) % experts, k = 0 .. topK-1 (distinct).  x[t][c] is a small
 // integer, exact in bf16, so that the unweighted combine of the memory route has to return topK * x exactly.
+#include <chrono>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
@@ -47,10 +48,11 @@ int Fail(const char *what, long long at, long long got, long long want)
 
 int main(int argc, char **argv)
 {
-    if (argc != 5) {
-        std::fprintf(stderr, "usage: demo <bs> <h> <topK> <experts>\n");
+    if (argc != 5 && argc != 6) {
+        std::fprintf(stderr, "usage: demo <bs> <h> <topK> <experts> [layers timed back to back after the check]\n");
         return 2;
     }
+    const int64_t timedLayers = argc == 6 ? std::atoll(argv[5]) : 0;
     const int64_t bs = std::atoll(argv[1]);
     const int64_t h = std::atoll(argv[2]);
     const int64_t topK = std::atoll(argv[3]);
@@ -172,6 +174,32 @@ int main(int argc, char **argv)
         }
     }
 
+    // the same two calls per layer as a serving loop makes them: no synchronisation between layers, so a layer costs
+    // whichever is longer, the host's two calls or the device's kernels
+    double usPerLayer = 0.0;
+    if (timedLayers > 0) {
+        for (int pass = 0; pass < 2; ++pass) {     // the first pass warms up
+            HIP_OK(hipStreamSynchronize(stream));
+            const auto t0 = std::chrono::steady_clock::now();
+            for (int64_t l = 0; l < timedLayers; ++l) {
+                st = TileXRMoeEpDispatchMemory(dX, static_cast<int32_t *>(dIds), comm, bs, h, topK, experts, dExpand,
+                    static_cast<int64_t *>(dTokenNums), static_cast<int32_t *>(dCounts), static_cast<int32_t *>(dAssist),
+                    TileXR::TILEXR_DATA_TYPE_BFP16, stream);
+                if (st == 0) {
+                    st = TileXRMoeEpCombineMemory(dExpand, static_cast<int32_t *>(dAssist), static_cast<int32_t *>(dCounts),
+                        comm, bs, h, topK, experts, dY, TileXR::TILEXR_DATA_TYPE_BFP16, stream);
+                }
+                if (st != 0) {
+                    std::fprintf(stderr, "timed layer %lld returned %d\n", static_cast<long long>(l), st);
+                    return 1;
+                }
+            }
+            HIP_OK(hipStreamSynchronize(stream));
+            const auto t1 = std::chrono::steady_clock::now();
+            usPerLayer = std::chrono::duration<double, std::micro>(t1 - t0).count() / static_cast<double>(timedLayers);
+        }
+    }
+
     TileXRCommDestroy(comm);
     HIP_OK(hipFree(dX));
     HIP_OK(hipFree(dIds));
@@ -181,7 +209,11 @@ int main(int argc, char **argv)
     HIP_OK(hipFree(dAssist));
     HIP_OK(hipFree(dY));
     HIP_OK(hipStreamDestroy(stream));
-    std::printf("OK bs=%lld h=%lld topK=%lld experts=%lld rows=%lld\n", static_cast<long long>(bs), static_cast<long long>(h),
+    std::printf("OK bs=%lld h=%lld topK=%lld experts=%lld rows=%lld", static_cast<long long>(bs), static_cast<long long>(h),
         static_cast<long long>(topK), static_cast<long long>(experts), static_cast<long long>(n));
+    if (timedLayers > 0) {
+        std::printf(" layers=%lld us_per_layer=%.2f", static_cast<long long>(timedLayers), usPerLayer);
+    }
+    std::printf("\n");
     return 0;
 }

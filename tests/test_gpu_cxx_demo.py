@@ -27,3 +27,17 @@ def test_cxx_demo(bs, h, top_k, experts):
     run = subprocess.run([DEMO, str(bs), str(h), str(top_k), str(experts)], capture_output=True, text=True, timeout=100)
     assert run.returncode == 0, run.stdout + run.stderr
     assert run.stdout.startswith("OK "), run.stdout
+
+
+def test_cxx_demo_times_decode_layers_back_to_back():
+    """The two calls of a decode-sized layer from a C++ loop with no synchronisation in between: the program reports the
+    time per layer, which this test prints and bounds only loosely (a host that is busy elsewhere must not fail it)."""
+    if not os.path.exists(DEMO):
+        pytest.fail(f"{DEMO} is missing: build it with `make -C tilexr_amd/csrc` (or __graft_entry__.build())")
+    print("cxx demo bs=128 h=7168 top_k=8 experts=256 layers=2000", flush=True)
+    run = subprocess.run([DEMO, "128", "7168", "8", "256", "2000"], capture_output=True, text=True, timeout=100)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert run.stdout.startswith("OK "), run.stdout
+    fields = dict(f.split("=") for f in run.stdout.split()[1:])
+    print(run.stdout.strip(), flush=True)
+    assert 0.0 < float(fields["us_per_layer"]) < 100.0

@@ -404,6 +404,60 @@ def test_memory_combine_matches_oracle(shape, dtype):
             assert np.array_equal(bits16(y), want)
 
 
+@pytest.mark.parametrize("route", ["memory", "mvp"])
+def test_small_combine_reads_the_assist_table_itself(route):
+    """Through the reference's entry points combine gets no row map.  Up to 2048 routes the reduce finds a token's rows
+    in the assist table itself (one launch); beyond that, or with rows the kernel's waves cannot cover, a first launch
+    inverts the table.  Both give the oracle's result; the cases sit on either side of every limit."""
+    cases = [  # bs, h, K, E, kernel
+        (256, 64, 8, 32, "ep_reduce_small_kernel"),        # 2048 routes: the most one workgroup scans
+        (257, 64, 8, 32, "ep_reduce_vec_kernel"),
+        (2048, 8, 1, 4, "ep_reduce_small_kernel"),         # one slot per token, rows of one vector
+        (5, 16384, 3, 9, "ep_reduce_small_kernel"),        # sixteen waves per row
+        (5, 16392, 3, 9, "ep_reduce_generic_kernel"),
+        (128, 7168, 8, 256, "ep_reduce_small_kernel"),     # decode
+        (64, 36, 15, 40, "ep_reduce_generic_kernel"),      # rows that are no multiple of 16 bytes
+        (40, 1024, 15, 40, "ep_reduce_small_kernel"),
+    ]
+    dtype = ep.DT_BF16 if route == "memory" else ep.DT_FP16
+    tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+    with Session() as s:
+        for bs, h, K, E, kernel in cases:
+            rng = np.random.default_rng(bs + h + K)
+            ids = ids_for(rng, bs, K, E, invalid=0.1)
+            _, xb = x_for(rng, bs, h, dtype, scale=3.0)
+            case = O.Case(1, bs, h, K, E, dtype=dtype)
+            d = (O.mem_dispatch if route == "memory" else O.mvp_dispatch)(case, 0, xb[None], ids[None])
+            rows = d["rows"]
+            eo = d["expand_x"].view(np.uint16).copy()
+            for r in range(rows):
+                eo[r] = np.roll(eo[r], r % 5)
+            counts = d["send_counts" if route == "memory" else "recv_counts"]
+            w = (0.25 + rng.random((bs, K))).astype(np.float32)
+            y = torch.full((bs, h), 7.0, dtype=tdt, device=DEV)
+            d_eo = torch.zeros((bs * K, h), dtype=torch.int16, device=DEV)
+            d_eo[:eo.shape[0]] = torch.from_numpy(eo.view(np.int16)).to(DEV)
+            d_assist = torch.full((bs * K, 4), -1, dtype=torch.int32, device=DEV)
+            d_assist[:d["assist"].shape[0]] = torch.from_numpy(d["assist"]).to(DEV)
+            torch.cuda.synchronize()
+            print(f"small combine: {route} bs={bs} h={h} K={K} E={E}", flush=True)
+            if route == "memory":
+                st = ep.combine_memory_v2(d_eo, d_assist, to_dev(counts), s.comm, bs, h, K, E, y, dtype, s.stream,
+                                          expert_scales=to_dev(w))
+            else:
+                st = ep.combine_v2(d_eo, d_assist, to_dev(counts), s.comm, bs, h, K, E, y, dtype, s.stream)
+            assert st == 0
+            s.sync()
+            assert ep.last_kernel_name(s.comm, ep.K_REDUCE) == kernel, (bs, h, K, E)
+            host_eo = d_eo.cpu().numpy().view(np.uint16)[None]
+            host_assist = d_assist.cpu().numpy()[None]
+            if route == "memory":
+                want = O.mem_combine(case, 0, host_eo, host_assist, counts[None], expert_scales=w)
+            else:
+                want = O.mvp_combine(case, 0, host_eo, host_assist, counts[None])
+            assert np.array_equal(bits16(y), want), (bs, h, K, E)
+
+
 @pytest.mark.parametrize("shape", [(24, 64, 4, 16), (33, 96, 3, 7), (12, 1024, 8, 64), (6, 7168, 8, 256), (9, 40, 2, 4)])
 @pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
 @pytest.mark.parametrize("mode", [3, 4])

@@ -284,13 +284,8 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     comm->debug.magic = magic;
 
     const uint64_t epoch = static_cast<uint64_t>(magic) & 0xffffffffull;
-    uint64_t *inverse = nullptr;
+    InvertLaunch inv {};
     if (p.rowIndexMap == nullptr) {
-        if (!comm->combineScratch.Reserve(static_cast<size_t>(n) * sizeof(uint64_t), true)) {
-            return TileXR::TILEXR_ERROR_INTERNAL;
-        }
-        inverse = static_cast<uint64_t *>(comm->combineScratch.ptr);
-        InvertLaunch inv {};
         inv.assist = p.assistInfoForCombine;
         inv.counts = p.epRecvCounts;
         inv.numCounts = memoryRoute ? p.moeExpertNum : 1;
@@ -301,20 +296,15 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
         inv.bs = p.bs;
         inv.topK = p.topK;
         inv.epoch = epoch;
-        inv.inverse = inverse;
         inv.stream = stream;
-        const int ret = Timed(comm, kKernelInvert, stream, "invert", [&] { return LaunchInvert(inv); });
-        if (ret != kOk) {
-            return ret;
-        }
     }
 
     ReduceLaunch red {};
     red.expertOut = p.expertOut;
     red.rowBytes = p.expertOutQuantMode == 0 ? p.h * 2 : p.h;
-    red.inverseTagged = inverse;
     red.epoch = epoch;
     red.rowIndexMap = p.rowIndexMap;
+    red.assistTable = p.rowIndexMap == nullptr ? &inv : nullptr;
     red.expertScales = memoryRoute ? p.expertScales : nullptr;
     red.tokenMask = memoryRoute ? reinterpret_cast<const uint8_t *>(p.xActiveMask) : nullptr;
     red.sharedExpertX = memoryRoute ? p.sharedExpertX : nullptr;
@@ -346,6 +336,22 @@ int RunCombineSingle(EpComm *comm, const EpCombineParams &p, bool memoryRoute, i
     red.numComputeUnits = comm->world->numComputeUnits;
     red.kernelNameOut = &comm->lastKernel[kKernelReduce];
     red.stream = stream;
+    if (SmallReduceFits(red)) {
+        // decode-sized: the reduce reads the assist table itself
+        return Timed(comm, kKernelReduce, stream, "reduce", [&] { return LaunchSmallReduce(red); });
+    }
+    if (p.rowIndexMap == nullptr) {
+        if (!comm->combineScratch.Reserve(static_cast<size_t>(n) * sizeof(uint64_t), true)) {
+            return TileXR::TILEXR_ERROR_INTERNAL;
+        }
+        inv.inverse = static_cast<uint64_t *>(comm->combineScratch.ptr);
+        const int ret = Timed(comm, kKernelInvert, stream, "invert", [&] { return LaunchInvert(inv); });
+        if (ret != kOk) {
+            return ret;
+        }
+        red.inverseTagged = inv.inverse;
+        red.assistTable = nullptr;
+    }
     return Timed(comm, kKernelReduce, stream, "reduce", [&] { return LaunchReduce(red); });
 }
 

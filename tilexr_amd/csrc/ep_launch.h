@@ -171,7 +171,8 @@ struct ReduceLaunch {
     int64_t rowBytes;
     const uint64_t *inverseTagged;   // either this (with epoch) ...
     uint64_t epoch;
-    const int32_t *rowIndexMap;      // ... or a plain row map (-1 = none)
+    const int32_t *rowIndexMap;      // ... or a plain row map (-1 = none) ...
+    const InvertLaunch *assistTable; // ... or the assist table itself (LaunchSmallReduce only)
     const uint64_t *orderKeys;       // optional, per-add kind: rows are summed in ascending orderKeys[row]
     const float *expertScales;       // optional [bs, topK]
     const uint8_t *tokenMask;        // optional [bs]
@@ -202,6 +203,11 @@ struct ReduceLaunch {
     const char **kernelNameOut;      // optional: receives the name of the kernel template that was launched
     hipStream_t stream;
 };
+
+// Combine of a small batch (at most kSmallRoutes routes, 16-bit rows, no readiness flags) in a single launch: every
+// token's workgroup finds its rows in the assist table itself, so no launch has to invert the table first.
+bool SmallReduceFits(const ReduceLaunch &l);
+hipError_t LaunchSmallReduce(const ReduceLaunch &l);
 
 // Memory-route dispatch of a small batch (plain copies, one rank, no mask, no readiness flags) in a single launch:
 // every workgroup counts the whole id table itself instead of waiting for a counting kernel.
