@@ -418,6 +418,7 @@ def test_small_combine_reads_the_assist_table_itself(route):
         (128, 7168, 8, 256, "ep_reduce_small_kernel"),     # decode
         (64, 36, 15, 40, "ep_reduce_generic_kernel"),      # rows that are no multiple of 16 bytes
         (40, 1024, 15, 40, "ep_reduce_small_kernel"),
+        (32, 256, 64, 80, "ep_reduce_small_kernel"),       # as many slots as a wave has lanes
     ]
     dtype = ep.DT_BF16 if route == "memory" else ep.DT_FP16
     tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
