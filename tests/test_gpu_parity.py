@@ -459,6 +459,72 @@ def test_small_combine_reads_the_assist_table_itself(route):
             assert np.array_equal(bits16(y), want), (bs, h, K, E)
 
 
+@pytest.mark.parametrize("seed", range(32))
+def test_small_combine_on_random_calls(seed):
+    """Seeded draws around the single-launch combine: shape (on both sides of its 2048 routes), route, element type,
+    gate weights, token mask, shared-expert row, and now and then a table with corrupted tuples, a duplicate claim on
+    a slot and a count that points past the buffer.  Every result is the oracle's, bit for bit."""
+    from test_oracle_routes import corrupt_tuples
+    rng = np.random.default_rng(4200 + seed)
+    route = "memory" if seed % 3 else "mvp"
+    dtype = ep.DT_BF16 if rng.integers(0, 2) else ep.DT_FP16
+    tdt = torch.bfloat16 if dtype == ep.DT_BF16 else torch.float16
+    K = int(rng.integers(1, 17))
+    bs = int(rng.integers(1, 2500 // K + 1))
+    E = int(rng.integers(K, 300))
+    h = int(rng.choice([8, 64, 136, 1000, 1024, 2048, 4096, 7168, 16384]))
+    ids = ids_for(rng, bs, K, E, invalid=float(rng.choice([0.0, 0.1, 0.6])))
+    _, xb = x_for(rng, bs, h, dtype, scale=3.0)
+    case = O.Case(1, bs, h, K, E, dtype=dtype)
+    d = (O.mem_dispatch if route == "memory" else O.mvp_dispatch)(case, 0, xb[None], ids[None])
+    rows = d["rows"]
+    eo = d["expand_x"].view(np.uint16).copy()
+    for r in range(rows):
+        eo[r] = np.roll(eo[r], r % 5)
+    assist = d["assist"].copy()
+    counts = d["send_counts" if route == "memory" else "recv_counts"].copy()
+    spoiled = seed % 4 == 1 and rows > 8
+    if spoiled:
+        corrupt_tuples(rng, assist[None], [rows], bs, K, 1, max(3, rows // 10))
+        if route == "memory":
+            intact = [r for r in range(rows) if np.array_equal(assist[r], d["assist"][r])]
+            assist[intact[-1], :3] = assist[intact[0], :3]
+            counts[-1] = bs * K + 999
+    use_w, use_mask, use_shared = (bool(v) for v in rng.integers(0, 2, 3))
+    w = (0.25 + rng.random((bs, K))).astype(np.float32)
+    tmask = (rng.random(bs) < 0.7).astype(np.uint8)
+    _, sxb = x_for(rng, bs, h, dtype)
+    print(f"small combine seed={seed}: {route} bs={bs} h={h} K={K} E={E} dtype={dtype} spoiled={spoiled} "
+          f"weights={use_w} mask={use_mask} shared={use_shared}", flush=True)
+    with Session() as s:
+        y = torch.full((bs, h), 7.0, dtype=tdt, device=DEV)
+        d_eo = torch.full((bs * K, h), 0x7f7f, dtype=torch.int16, device=DEV)
+        d_eo[:eo.shape[0]] = torch.from_numpy(eo.view(np.int16)).to(DEV)
+        d_assist = torch.full((bs * K, 4), -77, dtype=torch.int32, device=DEV)
+        d_assist[:assist.shape[0]] = torch.from_numpy(assist).to(DEV)
+        torch.cuda.synchronize()
+        if route == "memory":
+            st = ep.combine_memory_v2(d_eo, d_assist, to_dev(counts), s.comm, bs, h, K, E, y, dtype, s.stream,
+                                      expert_scales=to_dev(w) if use_w else None,
+                                      active_mask=to_dev(tmask) if use_mask else None,
+                                      active_mask_type=ep.MASK_TOKEN if use_mask else ep.MASK_NONE,
+                                      shared_expert_x=to_dev(sxb) if use_shared else None)
+        else:
+            st = ep.combine_v2(d_eo, d_assist, to_dev(counts), s.comm, bs, h, K, E, y, dtype, s.stream)
+        assert st == 0
+        s.sync()
+        small = bs * K <= 2048 and h % 8 == 0
+        assert (ep.last_kernel_name(s.comm, ep.K_REDUCE) == "ep_reduce_small_kernel") == small
+        host_eo = d_eo.cpu().numpy().view(np.uint16)[None]
+        host_assist = d_assist.cpu().numpy()[None]
+        if route == "memory":
+            want = O.mem_combine(case, 0, host_eo, host_assist, counts[None], expert_scales=w if use_w else None,
+                                 token_mask=tmask if use_mask else None, shared_expert_x=sxb if use_shared else None)
+        else:
+            want = O.mvp_combine(case, 0, host_eo, host_assist, counts[None])
+        assert np.array_equal(bits16(y), want)
+
+
 @pytest.mark.parametrize("shape", [(24, 64, 4, 16), (33, 96, 3, 7), (12, 1024, 8, 64), (6, 7168, 8, 256), (9, 40, 2, 4)])
 @pytest.mark.parametrize("dtype", [ep.DT_BF16, ep.DT_FP16])
 @pytest.mark.parametrize("mode", [3, 4])
