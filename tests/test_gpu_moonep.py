@@ -150,6 +150,7 @@ CASES = [
     (3, 9, 32, 256, 11, True, True),
     (16, 4, 4, 64, 2, True, True),
     (2, 300, 8, 2048, 700, True, True),      # more than one 2048-row pass of the plan build, many unused rows
+    (1, 2100, 8, 64, 700, True, True),       # nine passes: the plan's workgroups in the scatter launch read chunk totals
     (2, 13, 3, 17, 4, True, True),           # odd hidden size: element-wise kernels
     (4, 6, 5, 24, 0, False, True),           # rows of three 16-byte vectors
 ]

@@ -10,6 +10,9 @@
 //
 //   dispatch  walk      saved plans: parent records from dupGroups / dupLoffs
 //             agree     saved plans: per duplicate route, whether the plan's primary is the token's own primary row
+//             records   fresh plans of smaller worlds: what the routes record (below), ahead of the scatter, in the
+//                       launch that reads the token rows ahead; the plan is then built by extra workgroups of the
+//                       scatter launch instead of by launches after it
 //             scatter   rows, weights, row tags; fresh plans: parent / sibling records of duplicates
 //             build     fresh plans: dupGroups / dupCounts from the parent records
 //             finish    per row: what is left to write (zeros, or a copy of the primary of a saved plan) and writing it;

@@ -28,6 +28,9 @@ constexpr int kXcds = 8;
 constexpr int kRowVecs = 2;     // 16-byte vectors per lane per row slice
 
 std::atomic<int64_t> gCachedRowBytes {int64_t{256} << 20};     // TileXRMoonEpSetCachedRowBytes
+constexpr int kFusedPlanChunks = 1024;  // chunks of 2048 rows per rank up to which the scatter launch builds a fresh plan
+constexpr int64_t kFusedPlanRowBytes = int64_t{256} << 20;     // ... and bytes of rows the world's routes write
+constexpr int kSelfPlanChunks = 8;      // ... and up to which its plan workgroups add up the earlier chunks themselves
 constexpr int64_t kWarmRowBytes = int64_t{128} << 20;          // token rows of a world that are read ahead of the per-route scatter
 
 const char *gScatterName = "";
@@ -216,14 +219,97 @@ __global__ __launch_bounds__(kThreads) void moon_warm_rows_kernel(DispatchWorld 
     WarmRows(a, blockIdx.y, static_cast<int64_t>(blockIdx.x), vecs);
 }
 
-// One workgroup per (token, route, slice of 512 vectors) of source rank blockIdx.y.
-template <bool FRESH>
-__global__ __launch_bounds__(kThreads) void moon_scatter_kernel(DispatchWorld a, int colSlices)
+// Fresh plans, one thread per route of source rank blockIdx.y: everything a route records (RouteRecords) and the
+// failure of a route that names no rank, ahead of the scatter.  Nothing the plan is built from is then written by the
+// scatter launch, so extra workgroups of that launch build it (moon_scatter_kernel, PLAN) instead of launches after it.
+// The workgroups from `routeBlocks` on read the token rows ahead, as in moon_agree_kernel.
+__global__ __launch_bounds__(kThreads) void moon_records_kernel(DispatchWorld a, unsigned routeBlocks, int64_t warmVecs)
 {
-    __shared__ int32_t s_dst[kMaxTopK];
+    if (blockIdx.x >= routeBlocks) {
+        WarmRows(a, blockIdx.y, static_cast<int64_t>(blockIdx.x - routeBlocks), warmVecs);
+        return;
+    }
     const int src = blockIdx.y;
-    const int xcd = blockIdx.x % kXcds;
-    const int j = blockIdx.x / kXcds;
+    const int64_t route = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+    if (route >= a.s * a.k) {
+        return;
+    }
+    const int K = static_cast<int>(a.k);
+    const int k = static_cast<int>(route % K);
+    const int32_t *words = a.dst[src] + route - k;
+    const float weight = a.weightsSk[src] != nullptr ? a.weightsSk[src][route] : 0.0f;
+    const Route r = Decode(words[k], a.nvS, a.world);
+    if (!r.ok) {
+        RecordFailure(a.tables, src, a.epoch, kDispatchInvalidRoute);
+        return;
+    }
+    const int64_t at = static_cast<int64_t>(r.peer) * a.tables.stride + r.row;
+    if (a.weightsSk[src] != nullptr) {
+        a.weightsNvs[r.peer][r.row] = weight;
+    }
+    a.tables.rowTag[at] = Tag(a.epoch, kRowNamed | kRowWritten);
+    if (!r.duplicate) {
+        return;
+    }
+    // the token's other routes to the same rank: the first non-duplicate before this one is the primary, the duplicates
+    // with a smaller row stand before this one in the primary's group (RouteRecords, one lane per route there)
+    int primaryRow = -1;
+    uint32_t siblings = 0;
+    uint32_t before = 0;
+    for (int j = 0; j < K; ++j) {
+        const Route o = Decode(words[j], a.nvS, a.world);
+        if (!o.ok || o.peer != r.peer) {
+            continue;
+        }
+        if (!o.duplicate) {
+            primaryRow = (primaryRow < 0 && j < k) ? o.row : primaryRow;
+        } else {
+            siblings += 1u;
+            before += o.row < r.row ? 1u : 0u;
+        }
+    }
+    if (primaryRow < 0) {
+        RecordFailure(a.tables, src, a.epoch, kDispatchInvalidRoute);
+        return;
+    }
+    a.tables.parentTag[at] = Tag(a.epoch, static_cast<uint32_t>(primaryRow) + 1u);
+    a.tables.sibling[at] = before | (siblings << 16);
+}
+
+// defined with the kernels that build the duplicate plan, below
+template <bool SELF>
+__device__ __forceinline__ void DedupGroupsOfChunk(const DispatchWorld &a, int rank, int chunk, bool lastChunk,
+    int (*s_part)[kThreads / kWave], int *s_base);
+
+// One workgroup per (token, route, slice of 512 vectors) of source rank blockIdx.y.
+//
+// PLAN: a fresh plan whose records were written ahead (moon_records_kernel) is built here as well: the first `planBlocks` workgroups
+// of the launch (a multiple of eight, so that the rest keep their XCDs) take one chunk of destination rank blockIdx.y
+// each.  They depend on nothing this launch writes and are done long before the rows are.  The totals of the chunks
+// before its own a workgroup adds up itself while the chunks are few (planSelf), a trip to memory per chunk, and those
+// trips are slow beside the scatter's traffic (measured: 5 us each; 32 chunks took longer than the rows); otherwise a
+// launch of moon_dedup_totals_kernel ahead of this one has left them.
+template <bool FRESH, bool PLAN>
+__global__ __launch_bounds__(kThreads) void moon_scatter_kernel(DispatchWorld a, int colSlices, unsigned planBlocks, int planChunks,
+    int planSelf)
+{
+    static_assert(FRESH || !PLAN, "only a Dispatch that builds its plan has plan workgroups");
+    __shared__ int32_t s_dst[kMaxTopK];
+    if (PLAN && blockIdx.x < planBlocks) {
+        __shared__ int s_part[2][kThreads / kWave];
+        __shared__ int s_base[2];
+        const int chunk = blockIdx.x;
+        if (chunk < planChunks && planSelf != 0) {
+            DedupGroupsOfChunk<true>(a, blockIdx.y, chunk, chunk == planChunks - 1, s_part, s_base);
+        } else if (chunk < planChunks) {
+            DedupGroupsOfChunk<false>(a, blockIdx.y, chunk, chunk == planChunks - 1, s_part, s_base);
+        }
+        return;
+    }
+    const unsigned block = blockIdx.x - (PLAN ? planBlocks : 0u);
+    const int src = blockIdx.y;
+    const int xcd = block % kXcds;
+    const int j = block / kXcds;
     const int K = static_cast<int>(a.k);
     const int perToken = K * colSlices;
     const int token = (j / perToken) * kXcds + xcd;
@@ -237,7 +323,7 @@ __global__ __launch_bounds__(kThreads) void moon_scatter_kernel(DispatchWorld a,
     const int vecs = h / 8;
     const int colBase = slice * (kRowVecs * kThreads);
     const int32_t *words = a.dst[src] + static_cast<int64_t>(token) * K;
-    const bool records = slice == 0;
+    const bool records = slice == 0 && !PLAN;       // PLAN: written ahead by moon_records_kernel
     if (FRESH && records && lane < K) {
         s_dst[lane] = words[lane];
     }
@@ -474,27 +560,56 @@ __global__ __launch_bounds__(kThreads) void moon_dedup_totals_kernel(DispatchWor
     }
 }
 
-// SELF: the workgroup adds up the chunks before its own from the row records themselves, which is cheaper than a launch
-// of the totals kernel while there are few chunks (the work grows with the square of their number).
-template <bool SELF>
-__global__ __launch_bounds__(kThreads) void moon_dedup_groups_kernel(DispatchWorld a)
+// What the thread's rows of the chunks before `chunks` add to their totals.  Both words of a row are asked for whatever
+// the first one says: one trip to memory per chunk, not two.  (One chunk at a time: the kernel that runs this beside a
+// scatter must stay small in registers, see LaunchMoonDispatch.)
+constexpr int kTotalsAhead = 1;
+__device__ __forceinline__ void AddEarlierChunks(const DispatchWorld &a, int rank, int chunks, int *open, int *size)
 {
-    __shared__ int s_part[2][kThreads / kWave];
-    __shared__ int s_base[2];
-    const int rank = blockIdx.y;
+    const uint64_t *parent = a.tables.parentTag + static_cast<int64_t>(rank) * a.tables.stride;
+    const uint32_t *sibling = a.tables.sibling + static_cast<int64_t>(rank) * a.tables.stride;
+    for (int c0 = 0; c0 < chunks; c0 += kTotalsAhead) {
+        uint64_t p[kTotalsAhead][kBuildPer];
+        uint32_t sib[kTotalsAhead][kBuildPer];
+#pragma unroll
+        for (int u = 0; u < kTotalsAhead; ++u) {
+#pragma unroll
+            for (int i = 0; i < kBuildPer; ++i) {
+                const int64_t row = static_cast<int64_t>(c0 + u) * kBuildRows + static_cast<int64_t>(threadIdx.x) * kBuildPer + i;
+                const bool in = c0 + u < chunks && row < a.nvS;
+                p[u][i] = in ? parent[row] : 0ull;          // the epoch is never zero: an untagged word
+                sib[u][i] = in ? sibling[row] : 0u;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < kTotalsAhead; ++u) {
+#pragma unroll
+            for (int i = 0; i < kBuildPer; ++i) {
+                const bool opens = Tagged(p[u][i], a.epoch) && (sib[u][i] & 0xffffu) == 0;
+                *open += opens ? 1 : 0;
+                *size += opens ? static_cast<int>(sib[u][i] >> 16) : 0;
+            }
+        }
+    }
+}
+
+// Groups and slice starts of one chunk of destination rank `rank` (see above).
+// SELF: the workgroup adds up the chunks before its own from the row records themselves -- when the chunks are few, and
+// when it runs as an extra workgroup of the scatter launch, where nothing waits for it; otherwise from the totals that a
+// launch of moon_dedup_totals_kernel left.
+template <bool SELF>
+__device__ __forceinline__ void DedupGroupsOfChunk(const DispatchWorld &a, int rank, int chunk, bool lastChunk,
+    int (*s_part)[kThreads / kWave], int *s_base)
+{
     const int tid = threadIdx.x;
     // totals of the chunks before this one
     int beforeOpen = 0;
     int beforeSize = 0;
     if (SELF) {
-        for (int c = 0; c < static_cast<int>(blockIdx.x); ++c) {
-            const ChunkRows earlier = LoadChunkRows(a, rank, static_cast<int64_t>(c) * kBuildRows);
-            beforeOpen += earlier.localOpen;
-            beforeSize += earlier.localSize;
-        }
+        AddEarlierChunks(a, rank, chunk, &beforeOpen, &beforeSize);
     } else {
         const int32_t *totals = a.tables.chunkTotals + static_cast<int64_t>(rank) * a.tables.groupStride * 2;
-        for (int c = tid; c < static_cast<int>(blockIdx.x); c += kThreads) {
+        for (int c = tid; c < chunk; c += kThreads) {
             beforeOpen += totals[2 * c];
             beforeSize += totals[2 * c + 1];
         }
@@ -506,7 +621,7 @@ __global__ __launch_bounds__(kThreads) void moon_dedup_groups_kernel(DispatchWor
         s_base[1] = baseSize;
     }
     __syncthreads();
-    const ChunkRows c = LoadChunkRows(a, rank, static_cast<int64_t>(blockIdx.x) * kBuildRows);
+    const ChunkRows c = LoadChunkRows(a, rank, static_cast<int64_t>(chunk) * kBuildRows);
     int totalOpen, totalSize;
     ScanPair(c.localOpen, c.localSize, s_part, &exclOpen, &exclSize, &totalOpen, &totalSize);
     int group = s_base[0] + exclOpen;
@@ -529,10 +644,18 @@ __global__ __launch_bounds__(kThreads) void moon_dedup_groups_kernel(DispatchWor
             start += c.sizes[i];
         }
     }
-    if (blockIdx.x == gridDim.x - 1 && tid == 0) {
+    if (lastChunk && tid == 0) {
         a.dupCounts[rank][0] = s_base[0] + totalOpen;
         a.dupCounts[rank][1] = s_base[1] + totalSize;
     }
+}
+
+template <bool SELF>
+__global__ __launch_bounds__(kThreads) void moon_dedup_groups_kernel(DispatchWorld a)
+{
+    __shared__ int s_part[2][kThreads / kWave];
+    __shared__ int s_base[2];
+    DedupGroupsOfChunk<SELF>(a, blockIdx.y, blockIdx.x, blockIdx.x == gridDim.x - 1, s_part, s_base);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -1136,6 +1259,30 @@ const char *MoonReduceKernelName()
     return gReduceName;
 }
 
+// What follows the routes' records: the duplicate plan of a fresh Dispatch, then the rows and weights no route wrote.
+hipError_t LaunchPlanAndFinish(const DispatchWorld &w, hipStream_t stream, bool vec, bool plan)
+{
+    const unsigned R = static_cast<unsigned>(w.world);
+    if (w.fresh && plan) {
+        const unsigned chunks = static_cast<unsigned>((w.nvS + kBuildRows - 1) / kBuildRows);
+        if (chunks <= kSelfTotalChunks) {
+            hipLaunchKernelGGL(moon_dedup_groups_kernel<true>, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+        } else {
+            hipLaunchKernelGGL(moon_dedup_totals_kernel, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+            MOON_LAUNCH_CHECK();
+            hipLaunchKernelGGL(moon_dedup_groups_kernel<false>, dim3(chunks, R), dim3(kThreads), 0, stream, w);
+        }
+        MOON_LAUNCH_CHECK();
+    }
+    const unsigned groups = static_cast<unsigned>((w.nvS + kFinishRows - 1) / kFinishRows);
+    if (vec) {
+        hipLaunchKernelGGL(moon_finish_kernel<true>, dim3(groups, R), dim3(kThreads), 0, stream, w);
+    } else {
+        hipLaunchKernelGGL(moon_finish_kernel<false>, dim3(groups, R), dim3(kThreads), 0, stream, w);
+    }
+    return hipGetLastError();
+}
+
 hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const LaunchTiming &timing)
 {
     const unsigned R = static_cast<unsigned>(w.world);
@@ -1160,10 +1307,31 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
     // on rows that were)
     const bool warm = perRoute && worldRowBytes <= kWarmRowBytes;
     const unsigned warmBlocks = warm ? static_cast<unsigned>((rowVecs + kThreads * kWarmLoads - 1) / (kThreads * kWarmLoads)) : 0u;
-    if (!w.fresh) {
+    const unsigned routeBlocks = static_cast<unsigned>((w.s * w.k + kThreads - 1) / kThreads);
+    // A fresh plan of a world whose rows are copied per route and come to at most kFusedPlanRowBytes: what the routes
+    // record is written ahead of the scatter, by the launch that reads the token rows ahead, and the plan is built by
+    // extra workgroups of the scatter launch; only the finish kernel follows the scatter.  Three launches instead of five
+    // while a rank has at most kSelfPlanChunks chunks, four (the chunk totals need one) beyond: 128 tokens x 7168 x top-8
+    // 36.6 -> 34.2 us per layer, 384 tokens 47.8 -> 41.6, 1024 tokens 77.5 -> 71.8, 4096 tokens x 2048 99.8 -> 93.6.  The
+    // scatter kernel that holds the plan's code has 50 registers per lane instead of 16, and its short-lived workgroups
+    // then start more slowly: from about 256 MB of rows on that costs more than the launches saved (4096 tokens x 7168
+    // 201 -> 204 us, 8192 tokens 365 -> 386 us), so larger worlds keep the plain kernel and the launches after it.
+    const int planChunks = static_cast<int>((w.nvS + kBuildRows - 1) / kBuildRows);
+    const bool planInScatter = w.fresh && perRoute && planChunks <= kFusedPlanChunks &&
+        static_cast<int64_t>(w.world) * w.s * w.k * w.h * 2 <= kFusedPlanRowBytes;
+    const bool planSelf = planChunks <= kSelfPlanChunks;
+    const unsigned planBlocks = planInScatter ? static_cast<unsigned>((planChunks + kXcds - 1) / kXcds * kXcds) : 0u;
+    if (planInScatter) {
+        hipLaunchKernelGGL(moon_records_kernel, dim3(routeBlocks + warmBlocks, R), dim3(kThreads), 0, stream, w, routeBlocks,
+            warm ? rowVecs : int64_t{0});
+        MOON_LAUNCH_CHECK();
+        if (!planSelf) {
+            hipLaunchKernelGGL(moon_dedup_totals_kernel, dim3(static_cast<unsigned>(planChunks), R), dim3(kThreads), 0, stream, w);
+            MOON_LAUNCH_CHECK();
+        }
+    } else if (!w.fresh) {
         hipLaunchKernelGGL(moon_group_walk_kernel, dim3(rowBlocks, R), dim3(kThreads), 0, stream, w);
         MOON_LAUNCH_CHECK();
-        const unsigned routeBlocks = static_cast<unsigned>((w.s * w.k + kThreads - 1) / kThreads);
         hipLaunchKernelGGL(moon_agree_kernel, dim3(routeBlocks + warmBlocks, R), dim3(kThreads), 0, stream, w, routeBlocks,
             warm ? rowVecs : int64_t{0});
         MOON_LAUNCH_CHECK();
@@ -1185,11 +1353,14 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
         }
     } else if (perRoute) {
         gScatterName = "moon_scatter_kernel";
-        const dim3 grid(static_cast<unsigned>(blocks), R);
-        if (w.fresh) {
-            hipLaunchKernelGGL(moon_scatter_kernel<true>, grid, dim3(kThreads), 0, stream, w, colSlices);
+        const dim3 grid(static_cast<unsigned>(blocks) + planBlocks, R);
+        if (planInScatter) {
+            hipLaunchKernelGGL((moon_scatter_kernel<true, true>), grid, dim3(kThreads), 0, stream, w, colSlices, planBlocks,
+                planChunks, planSelf ? 1 : 0);
+        } else if (w.fresh) {
+            hipLaunchKernelGGL((moon_scatter_kernel<true, false>), grid, dim3(kThreads), 0, stream, w, colSlices, 0u, 0, 0);
         } else {
-            hipLaunchKernelGGL(moon_scatter_kernel<false>, grid, dim3(kThreads), 0, stream, w, colSlices);
+            hipLaunchKernelGGL((moon_scatter_kernel<false, false>), grid, dim3(kThreads), 0, stream, w, colSlices, 0u, 0, 0);
         }
     } else {
         gScatterName = "moon_scatter_generic_kernel";
@@ -1205,24 +1376,7 @@ hipError_t LaunchMoonDispatch(const DispatchWorld &w, hipStream_t stream, const 
     if (err != hipSuccess) {
         return err;
     }
-    if (w.fresh) {
-        const unsigned chunks = static_cast<unsigned>((w.nvS + kBuildRows - 1) / kBuildRows);
-        if (chunks <= kSelfTotalChunks) {
-            hipLaunchKernelGGL(moon_dedup_groups_kernel<true>, dim3(chunks, R), dim3(kThreads), 0, stream, w);
-        } else {
-            hipLaunchKernelGGL(moon_dedup_totals_kernel, dim3(chunks, R), dim3(kThreads), 0, stream, w);
-            MOON_LAUNCH_CHECK();
-            hipLaunchKernelGGL(moon_dedup_groups_kernel<false>, dim3(chunks, R), dim3(kThreads), 0, stream, w);
-        }
-        MOON_LAUNCH_CHECK();
-    }
-    const unsigned groups = static_cast<unsigned>((w.nvS + kFinishRows - 1) / kFinishRows);
-    if (vec) {
-        hipLaunchKernelGGL(moon_finish_kernel<true>, dim3(groups, R), dim3(kThreads), 0, stream, w);
-    } else {
-        hipLaunchKernelGGL(moon_finish_kernel<false>, dim3(groups, R), dim3(kThreads), 0, stream, w);
-    }
-    return hipGetLastError();
+    return LaunchPlanAndFinish(w, stream, vec, !planInScatter);
 }
 
 hipError_t LaunchMoonCombine(const CombineWorld &w, hipStream_t stream, const LaunchTiming &timing)
