@@ -406,13 +406,15 @@ def test_memory_combine_matches_oracle(shape, dtype):
 
 @pytest.mark.parametrize("route", ["memory", "mvp"])
 def test_small_combine_reads_the_assist_table_itself(route):
-    """Through the reference's entry points combine gets no row map.  Up to 2048 routes the reduce finds a token's rows
-    in the assist table itself (one launch); beyond that, or with rows the kernel's waves cannot cover, a first launch
-    inverts the table.  Both give the oracle's result; the cases sit on either side of every limit."""
+    """Through the reference's entry points combine gets no row map.  Up to 2048 routes (and a million tokens x tuples)
+    the reduce finds a token's rows in the assist table itself (one launch); beyond that, or with rows the kernel's
+    waves cannot cover, a first launch inverts the table.  Both give the oracle's result; the cases sit on either side of every limit."""
     cases = [  # bs, h, K, E, kernel
         (256, 64, 8, 32, "ep_reduce_small_kernel"),        # 2048 routes: the most one workgroup scans
         (257, 64, 8, 32, "ep_reduce_vec_kernel"),
-        (2048, 8, 1, 4, "ep_reduce_small_kernel"),         # one slot per token, rows of one vector
+        (1024, 8, 1, 4, "ep_reduce_small_kernel"),         # one slot per token, rows of one vector
+        (2048, 8, 1, 4, "ep_reduce_vec_kernel"),           # more tokens than it pays to let every one read the table
+        (512, 64, 4, 32, "ep_reduce_small_kernel"),        # tokens x tuples at its limit
         (5, 16384, 3, 9, "ep_reduce_small_kernel"),        # sixteen waves per row
         (5, 16392, 3, 9, "ep_reduce_generic_kernel"),
         (128, 7168, 8, 256, "ep_reduce_small_kernel"),     # decode
@@ -513,7 +515,7 @@ def test_small_combine_on_random_calls(seed):
             st = ep.combine_v2(d_eo, d_assist, to_dev(counts), s.comm, bs, h, K, E, y, dtype, s.stream)
         assert st == 0
         s.sync()
-        small = bs * K <= 2048 and h % 8 == 0
+        small = bs * K <= 2048 and bs * bs * K <= 1 << 20 and h % 8 == 0
         assert (ep.last_kernel_name(s.comm, ep.K_REDUCE) == "ep_reduce_small_kernel") == small
         host_eo = d_eo.cpu().numpy().view(np.uint16)[None]
         host_assist = d_assist.cpu().numpy()[None]

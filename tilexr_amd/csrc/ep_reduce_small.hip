@@ -29,6 +29,10 @@ constexpr int kSmallReduceVecs = 2;         // 16-byte vectors per lane
 constexpr int kSmallReduceRows = 8;         // rows in flight per lane
 constexpr int kScanBatch = 4;               // tuples a lane has in flight
 constexpr int kScanWaves = 4;               // a workgroup has at least this many waves for the table
+// Every token's workgroup reads the whole table, so the launch reads tokens x tuples of it in all: up to a million the
+// reading costs less than the launch that would invert the table (512 tokens x 2048 tuples: 0.8 us over the reduce that is
+// handed a row map, against 2.6 us for that launch), beyond that more (1024 x 2048: 3.4 us, 2048 x 2048: 8.6 us).
+constexpr int64_t kSmallScanTuples = int64_t{1} << 20;
 
 struct SmallReduceArgs {
     const void *expertOut;
@@ -207,7 +211,7 @@ bool SmallReduceFits(const ReduceLaunch &l)
     const int64_t n = l.bs * l.topK;
     const int64_t vecs = l.h / 8;
     return l.assistTable != nullptr && l.rowIndexMap == nullptr && l.inverseTagged == nullptr && l.orderKeys == nullptr &&
-        l.bs > 0 && n <= kSmallRoutes && l.topK <= kMaxTopK && l.sharedSlots == 0 && l.tileFlags == nullptr &&
+        l.bs > 0 && n <= kSmallRoutes && l.bs * n <= kSmallScanTuples && l.topK <= kMaxTopK && l.sharedSlots == 0 && l.tileFlags == nullptr &&
         l.inQuant == 0 && l.commQuant == 0 && l.h % 8 == 0 && l.rowBytes == l.h * 2 &&
         vecs <= static_cast<int64_t>(kSmallReduceThreads / kWave) * kWave * kSmallReduceVecs &&
         l.assistTable->maxRows == n && l.assistTable->maxCountPerEntry == n && l.assistTable->bs == l.bs &&
